@@ -1,0 +1,238 @@
+/*
+ * libsmall_hip -- C ABI of the MI355X (gfx950) implementation of the SMaLL layer hot path.
+ *
+ * Every entry point is what a binding of the reference's layer functions would call: plain
+ * ints, device pointers and a HIP stream; no C++ or torch types.  The C++ header
+ * include/small.h re-creates the reference's `small::` templates on top of this ABI.
+ *
+ * Conventions
+ *   - All tensor pointers are DEVICE pointers, 16-byte aligned, in the reference's packed
+ *     layout with channel block SMALL_HIP_CB (= FloatBuffer::C_ob = C_ib = QUInt8Buffer::C_ob):
+ *       activations  [batch][C/16][H][W][16]
+ *       conv filter  [Co/16][Ci/cib][kh][kw][cib][16]   cib = 16, or Ci when Ci is 1, 2 or 3
+ *       dw filter    [C/16][kh][kw][16]
+ *       bias         [C] (channel order == packed order)
+ *     (reference: include/small/abstract_layer.hpp:1419-1432, include/small/buffers.hpp:33-120)
+ *   - `batch` independent images lie back to back; image n of a batched call equals the
+ *     reference's (batch-1) call on image n.  The reference has no batch argument.
+ *   - Pads are given in the reference's public order: top, bottom, left, right.
+ *   - Output height/width follow include/small/utils.hpp:159-165 applied to the padded input.
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Calls are asynchronous with
+ *     respect to the host; results are ordered on the stream.
+ *   - Return value: SMALL_HIP_OK, or an error code.  SMALL_HIP_ESTRIDE / ECHANNELS / ESCALE are
+ *     returned exactly where the reference throws std::invalid_argument
+ *     (include/small/interface_abstract.hpp); the C++ header turns them back into the same
+ *     exceptions with the same messages.
+ *   - In-place use (out == in) is allowed for the activation entry points, as in the reference.
+ */
+#ifndef SMALL_HIP_H
+#define SMALL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMALL_HIP_CB 16
+
+#define SMALL_HIP_OK 0
+#define SMALL_HIP_ESTRIDE 1   /* "<op> ERROR: stride unsupported."      */
+#define SMALL_HIP_ECHANNELS 2 /* "<op> ERROR: in_channels unsupported." */
+#define SMALL_HIP_ESCALE 3    /* "Upsample ERROR: scale factor unsupported (only 1 or 2)." */
+#define SMALL_HIP_EINVAL 4    /* null / misaligned pointer, non-positive size, Co % 16 != 0 */
+#define SMALL_HIP_EHIP 5      /* a HIP runtime call failed; see small_hip_last_error() */
+#define SMALL_HIP_ENOMEM 6
+
+#define SMALL_HIP_ACT_NONE 0
+#define SMALL_HIP_ACT_RELU 1
+#define SMALL_HIP_ACT_LEAKY 2
+
+typedef void *small_hip_stream_t;
+
+/* The quantisation fields the reference's QUInt8Buffer carries
+ * (include/small/platforms/reference/QUInt8Buffer.hpp:222-230).  Arithmetic reads `zero` of
+ * the input and filter buffers and `multiplier`, `lshift`, `rshift` of the output buffer
+ * (include/small/q_abstract_layer.hpp:921-938). */
+typedef struct small_hip_quant
+{
+    int32_t zero;
+    int32_t multiplier;
+    int32_t lshift;
+    int32_t rshift;
+} small_hip_quant;
+
+/* ---- runtime ------------------------------------------------------------------------- */
+const char *small_hip_version(void);
+const char *small_hip_strerror(int status);
+/* message of the last failure on the calling thread */
+const char *small_hip_last_error(void);
+int small_hip_device_count(void);
+int small_hip_set_device(int device);
+/* device memory for the Buffer classes (FloatBuffer.hpp:67-78 uses posix_memalign on the host) */
+int small_hip_malloc(void **ptr, size_t bytes);
+int small_hip_free(void *ptr);
+int small_hip_host_malloc(void **ptr, size_t bytes); /* pinned host memory */
+int small_hip_host_free(void *ptr);
+int small_hip_memcpy_h2d(void *dst, const void *src, size_t bytes, small_hip_stream_t stream);
+int small_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, small_hip_stream_t stream);
+int small_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, small_hip_stream_t stream);
+int small_hip_memset(void *dst, int value, size_t bytes, small_hip_stream_t stream);
+int small_hip_stream_synchronize(small_hip_stream_t stream);
+
+/* ---- float32 layers -------------------------------------------------------------------- */
+/* small::Conv2D<FloatBuffer>          include/small/interface.hpp:49-56,
+ *                                     include/small/interface_abstract.hpp:46-221 */
+int small_hip_conv2d_f32(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                         int b_pad, int l_pad, int r_pad, int output_channels, int input_channels,
+                         int input_height, int input_width, const float *input,
+                         const float *filter, float *output, small_hip_stream_t stream);
+/* small::PartialConv2D<FloatBuffer>   interface.hpp:94-101, interface_abstract.hpp:416-587:
+ * accumulates onto the existing contents of `output` */
+int small_hip_partial_conv2d_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                 int t_pad, int b_pad, int l_pad, int r_pad, int output_channels,
+                                 int input_channels, int input_height, int input_width,
+                                 const float *input, const float *filter, float *output,
+                                 small_hip_stream_t stream);
+/* Fused Bias + PartialConv2D + activation in one pass: the three-call sequence of
+ * Conv2DLayer::compute_output (include/small/Conv2DLayer.hpp:827-879), named after
+ * small::Conv2D_Bias_ReLU (include/small/fused_interface_abstract.hpp:217-290).
+ * bias may be NULL; act is SMALL_HIP_ACT_*; slope is used by ACT_LEAKY only. */
+int small_hip_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                  int t_pad, int b_pad, int l_pad, int r_pad, int output_channels,
+                                  int input_channels, int input_height, int input_width,
+                                  const float *input, const float *filter, const float *bias,
+                                  int act, float slope, float *output, small_hip_stream_t stream);
+/* small::DepthwiseConv2D<FloatBuffer>         interface.hpp:138-145, interface_abstract.hpp:994-1051 */
+int small_hip_depthwise_conv2d_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                   int t_pad, int b_pad, int l_pad, int r_pad, int input_channels,
+                                   int input_height, int input_width, const float *input,
+                                   const float *filter, float *output, small_hip_stream_t stream);
+/* small::PartialDepthwiseConv2D<FloatBuffer>  interface.hpp:182-190, interface_abstract.hpp:1127-1186 */
+int small_hip_partial_depthwise_conv2d_f32(int batch, int kernel_height, int kernel_width,
+                                           int stride, int t_pad, int b_pad, int l_pad, int r_pad,
+                                           int input_channels, int input_height, int input_width,
+                                           const float *input, const float *filter, float *output,
+                                           small_hip_stream_t stream);
+/* Fused Bias + PartialDepthwiseConv2D + activation (DepthwiseConv2DLayer::compute_output) */
+int small_hip_depthwise_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width,
+                                            int stride, int t_pad, int b_pad, int l_pad, int r_pad,
+                                            int input_channels, int input_height, int input_width,
+                                            const float *input, const float *filter,
+                                            const float *bias, int act, float slope, float *output,
+                                            small_hip_stream_t stream);
+/* small::MaxPool2D<FloatBuffer>       interface.hpp:276-282, interface_abstract.hpp:778-834.
+ * Padded positions count as 0 (abstract_layer.hpp:514-521, 718-728). */
+int small_hip_maxpool2d_f32(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                            int b_pad, int l_pad, int r_pad, int input_channels, int input_height,
+                            int input_width, const float *input, float *output,
+                            small_hip_stream_t stream);
+/* small::AveragePool2D<FloatBuffer>   interface.hpp:316-322, interface_abstract.hpp:910-978.
+ * Divides by kh*kw including padded positions (abstract_layer.hpp:565-569). */
+int small_hip_avgpool2d_f32(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                            int b_pad, int l_pad, int r_pad, int input_channels, int input_height,
+                            int input_width, const float *input, float *output,
+                            small_hip_stream_t stream);
+/* small::ReLUActivation<FloatBuffer>  interface.hpp:382-386, interface_abstract.hpp:1541-1566 */
+int small_hip_relu_f32(int batch, int input_channels, int input_height, int input_width,
+                       const float *input, float *output, small_hip_stream_t stream);
+/* small::LeakyReLUActivation<FloatBuffer>  interface_abstract.hpp:1616-1646 (the slope arrives
+ * there as a 1-element buffer; here it is passed by value) */
+int small_hip_leaky_relu_f32(int batch, int input_channels, int input_height, int input_width,
+                             const float *input, float negative_slope, float *output,
+                             small_hip_stream_t stream);
+/* small::Accum<FloatBuffer>           interface.hpp:451-455, interface_abstract.hpp:1950-1978 */
+int small_hip_accum_f32(int batch, int input_channels, int input_height, int input_width,
+                        const float *input, float *output, small_hip_stream_t stream);
+/* small::Bias / small::PartialBias<FloatBuffer>  interface_abstract.hpp:1992-2064 */
+int small_hip_bias_f32(int batch, int num_channels, int output_height, int output_width,
+                       const float *bias, float *output, small_hip_stream_t stream);
+int small_hip_partial_bias_f32(int batch, int num_channels, int output_height, int output_width,
+                               const float *bias, float *output, small_hip_stream_t stream);
+/* small::UpSample2D<FloatBuffer>      interface.hpp:352-357, interface_abstract.hpp:1845-1889 */
+int small_hip_upsample2d_f32(int batch, int scale_factor, int input_channels, int input_height,
+                             int input_width, const float *input, float *output,
+                             small_hip_stream_t stream);
+/* small::Concat<BufferT>              interface.hpp:475-481, interface_abstract.hpp:2072-2105
+ * (element_size = 4 for FloatBuffer, 1 for QUInt8Buffer) */
+int small_hip_concat(int batch, uint32_t input0_channels, uint32_t input1_channels,
+                     uint32_t input_height, uint32_t input_width, const void *input0,
+                     const void *input1, void *output, size_t element_size,
+                     small_hip_stream_t stream);
+/* Fully connected layer y = W x, i.e. Conv2D(1,1,1,0,0,0,0,No,Ni,1,1,...) on a 1x1 image, the way
+ * every reference model spells it (include/small/models/MobileNetTiny.hpp:531-538).  The
+ * reference's own small::Dense (interface_abstract.hpp:2113-2132) is a per-channel scale with no
+ * callers; see small_hip_dense_literal_f32. */
+int small_hip_dense_f32(int batch, int output_elements, int input_elements, const float *input,
+                        const float *filter, float *output, small_hip_stream_t stream);
+/* small::Dense<FloatBuffer> exactly as written: out[o*Ni + i] = in[o*Ni + i] * filter[o] */
+int small_hip_dense_literal_f32(int output_elements, int input_elements, const float *input,
+                                const float *filter, float *output, small_hip_stream_t stream);
+
+/* ---- quantised uint8 layers ------------------------------------------------------------- */
+/* small::Conv2D<QUInt8Buffer>         interface_abstract.hpp:229-404, q_abstract_layer.hpp:894-1567 */
+int small_hip_conv2d_u8(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                        int b_pad, int l_pad, int r_pad, int output_channels, int input_channels,
+                        int input_height, int input_width, const uint8_t *input,
+                        const small_hip_quant *input_q, const uint8_t *filter,
+                        const small_hip_quant *filter_q, uint8_t *output,
+                        const small_hip_quant *output_q, small_hip_stream_t stream);
+/* The same convolution split in two for callers whose filters are constant (the reference's
+ * Conv2DLayer packs its filter once at construction, include/small/Conv2DLayer.hpp:135-341):
+ * _prepare_filter re-orders a packed uint8 filter (input_channels % 16 == 0) into the kernel's
+ * operand order and tabulates the per-tap filter sums the zero-point correction needs; it does
+ * not depend on any zero point.  `prepared` is caller-owned device memory of
+ * small_hip_conv2d_u8_prepared_filter_bytes() bytes.  small_hip_conv2d_u8 does both steps in a
+ * library-owned scratch buffer on every call. */
+size_t small_hip_conv2d_u8_prepared_filter_bytes(int kernel_height, int kernel_width,
+                                                 int output_channels, int input_channels);
+int small_hip_conv2d_u8_prepare_filter(int kernel_height, int kernel_width, int output_channels,
+                                       int input_channels, const uint8_t *filter, void *prepared,
+                                       small_hip_stream_t stream);
+int small_hip_conv2d_u8_prepared(int batch, int kernel_height, int kernel_width, int stride,
+                                 int t_pad, int b_pad, int l_pad, int r_pad, int output_channels,
+                                 int input_channels, int input_height, int input_width,
+                                 const uint8_t *input, const small_hip_quant *input_q,
+                                 const void *prepared, const small_hip_quant *filter_q,
+                                 uint8_t *output, const small_hip_quant *output_q,
+                                 small_hip_stream_t stream);
+/* small::DepthwiseConv2D<QUInt8Buffer>  interface_abstract.hpp:1059-1116 */
+int small_hip_depthwise_conv2d_u8(int batch, int kernel_height, int kernel_width, int stride,
+                                  int t_pad, int b_pad, int l_pad, int r_pad, int input_channels,
+                                  int input_height, int input_width, const uint8_t *input,
+                                  const small_hip_quant *input_q, const uint8_t *filter,
+                                  const small_hip_quant *filter_q, uint8_t *output,
+                                  const small_hip_quant *output_q, small_hip_stream_t stream);
+/* small::MaxPool2D<QUInt8Buffer>      interface_abstract.hpp:843-899 */
+int small_hip_maxpool2d_u8(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                           int b_pad, int l_pad, int r_pad, int input_channels, int input_height,
+                           int input_width, const uint8_t *input, const small_hip_quant *input_q,
+                           uint8_t *output, const small_hip_quant *output_q,
+                           small_hip_stream_t stream);
+/* small::ReLUActivation<QUInt8Buffer> interface_abstract.hpp:1577-1602 */
+int small_hip_relu_u8(int batch, int input_channels, int input_height, int input_width,
+                      const uint8_t *input, const small_hip_quant *input_q, uint8_t *output,
+                      const small_hip_quant *output_q, small_hip_stream_t stream);
+/* Fully connected uint8 layer = small::Conv2D<QUInt8Buffer>(1,1,...) on a 1x1 image */
+int small_hip_dense_u8(int batch, int output_elements, int input_elements, const uint8_t *input,
+                       const small_hip_quant *input_q, const uint8_t *filter,
+                       const small_hip_quant *filter_q, uint8_t *output,
+                       const small_hip_quant *output_q, small_hip_stream_t stream);
+/* No counterpart in the reference (interface_abstract.hpp:1981 "todo", :983): defined here as
+ *   Accum:        out = requant_out((in + in_q.zero) + (out + out_q.zero))
+ *   AveragePool:  out = requant_out(sum over valid taps of (in + in_q.zero));
+ *                 the caller folds 1/(kh*kw) into out_q.multiplier / rshift */
+int small_hip_accum_u8(int batch, int input_channels, int input_height, int input_width,
+                       const uint8_t *input, const small_hip_quant *input_q, uint8_t *output,
+                       const small_hip_quant *output_q, small_hip_stream_t stream);
+int small_hip_avgpool2d_u8(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                           int b_pad, int l_pad, int r_pad, int input_channels, int input_height,
+                           int input_width, const uint8_t *input, const small_hip_quant *input_q,
+                           uint8_t *output, const small_hip_quant *output_q,
+                           small_hip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMALL_HIP_H */

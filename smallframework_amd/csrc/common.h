@@ -1,0 +1,76 @@
+// Shared host-side helpers for libsmall_hip (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/small_hip.h"
+
+namespace shp
+{
+
+constexpr int CB = SMALL_HIP_CB;          // channel block of every packed tensor
+constexpr int WAVE = 64;                  // gfx950 wavefront
+constexpr int NUM_XCD = 8;                // MI355X: 8 XCDs x 32 CUs, one L2 per XCD
+constexpr int NUM_CU = 256;
+
+void set_error(const char *fmt, ...);
+
+inline int fail_hip(hipError_t e, const char *what)
+{
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return SMALL_HIP_EHIP;
+}
+
+#define SHP_HIP(call)                                                                             \
+    do                                                                                            \
+    {                                                                                             \
+        hipError_t e__ = (call);                                                                  \
+        if (e__ != hipSuccess) return shp::fail_hip(e__, #call);                                  \
+    } while (0)
+
+#define SHP_LAUNCH_CHECK(name)                                                                    \
+    do                                                                                            \
+    {                                                                                             \
+        hipError_t e__ = hipGetLastError();                                                       \
+        if (e__ != hipSuccess) return shp::fail_hip(e__, name);                                   \
+    } while (0)
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int einval(const char *msg)
+{
+    set_error("%s", msg);
+    return SMALL_HIP_EINVAL;
+}
+
+// include/small/utils.hpp:159-165 applied to the padded extent; 0 when the kernel does not fit
+inline int out_dim(int in, int pad_front, int pad_back, int k, int stride)
+{
+    long padded = (long)in + pad_front + pad_back;
+    if (k > padded) return 0;
+    return (int)((padded - k) / stride + 1);
+}
+
+// window geometry shared by convolution, depthwise and pooling kernels
+struct Geom
+{
+    int H, W, Ho, Wo, kh, kw, stride, pt, pl;
+};
+
+// Library-owned device scratch for the calling thread's current device: grows on demand and is
+// re-used by later calls.  Work that uses it is ordered by the stream it is launched on, so
+// calls that share a device must not overlap on different streams.
+int get_workspace(size_t bytes, void **ptr);
+
+inline hipStream_t as_stream(small_hip_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool pads_ok(int t, int b, int l, int r)
+{
+    return t >= 0 && b >= 0 && l >= 0 && r >= 0 && t < 256 && b < 256 && l < 256 && r < 256;
+}
+
+} // namespace shp

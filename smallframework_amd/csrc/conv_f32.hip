@@ -1,0 +1,395 @@
+// Conv2D / PartialConv2D / Dense (float32) for gfx950.
+//
+// Two kernels:
+//
+//  conv_mfma_f32_kernel   input_channels % 16 == 0.  Implicit GEMM on v_mfma_f32_32x32x2_f32:
+//      D[co][px] += sum_k  F[co][k] * I[k][px],   k = (tap, ci)
+//    MFMA rows are output channels, MFMA columns are output pixels flattened over
+//    (image, oh, ow).  With the packed layouts a K-step of 16 (one input-channel block at one
+//    filter tap) needs no shuffling at all:
+//      - B operand: lane (px = lane%32, half = lane/32) reads 8 consecutive floats of its
+//        pixel's 64-byte channel block: two 16-byte loads straight from global memory into the
+//        register the MFMA consumes.  The two wave halves take channels 0-7 and 8-15, so MFMA
+//        number kk of the step contracts channels {kk, 8+kk}; the pairing of k inside an MFMA
+//        is free as long as A and B agree.
+//      - A operand: lane (co = lane%32, half) reads F[ci = 8*half+kk][co%16] of its channel
+//        block's [16 ci][16 co] tile: 8 dword loads, each coalesced over 16 lanes.
+//      - D: lane holds 4 consecutive output channels of one pixel per register quad, i.e.
+//        16-byte stores into the packed [px][16] output.
+//    Padded taps are contributed as zeros by predicating the B operand.  The loads of step
+//    s+1 are issued before the MFMAs of step s (register double buffer).
+//    A wave owns COT x PXT tiles of 32 x 32; the four waves of a workgroup share the output
+//    channel group (their filter reads hit in the vector cache) and take consecutive pixel
+//    tiles.  Workgroup ids are re-mapped so that all channel groups of a pixel range run on
+//    one XCD and share its L2.
+//
+//  conv_smallci_f32_kernel   input_channels in {1,2,3} (first layers).  K is only
+//    Ci*kh*kw (27 for a 3x3 RGB stem), so these layers are bound by HBM traffic of their
+//    large outputs; a lane computes the 16 output channels of one pixel with scalar-loaded
+//    weights on the vector ALU.
+//
+// Epilogue (both kernels, in registers): optional accumulate onto the existing output
+// (PartialConv2D), optional bias, optional ReLU / LeakyReLU.
+#include "common.h"
+
+using namespace shp;
+
+namespace
+{
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+struct ConvArgs
+{
+    const float *in;
+    const float *filt;
+    const float *bias;   // may be null
+    float *out;
+    int batch, Co, Ci, H, W, Ho, Wo, kh, kw, stride, pt, pl;
+    int act;
+    float slope;
+    int accumulate;
+    // derived
+    int P;               // batch * Ho * Wo
+    int n_co_groups;     // ceil(Co / (32*COT))
+    int n_px_blocks;     // ceil(P / (32*PXT*4))
+    int n_blocks;        // n_co_groups * n_px_blocks
+    int per_xcd;         // ceil(n_blocks / 8)
+};
+
+__device__ __forceinline__ float act1(float v, int act, float slope)
+{
+    if (act == SMALL_HIP_ACT_RELU) return v > 0.f ? v : 0.f;
+    if (act == SMALL_HIP_ACT_LEAKY) return v > 0.f ? v : v * slope;
+    return v;
+}
+
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
+{
+    // XCD-aware id: hardware deals consecutive workgroup ids round-robin over the 8 XCDs
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;
+    const int cg = lid % a.n_co_groups;
+    const int pxb = lid / a.n_co_groups;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int HoWo = a.Ho * a.Wo;
+    const int CiB = a.Ci / CB;
+    const int CoB = a.Co / CB;
+    const int taps = a.kh * a.kw;
+    const size_t in_blk = (size_t)a.H * a.W * CB;     // floats per input channel block
+
+    // ---- per-lane pixel columns --------------------------------------------------------
+    const float *in_img[PXT];   // image base + half offset
+    int ih0[PXT], iw0[PXT];
+    bool pvalid[PXT];
+    size_t out_pix[PXT];        // float index of (n, co block 0, pixel), co block stride = HoWo*16
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo;
+        const int rem = pc - n * HoWo;
+        const int oh = rem / a.Wo;
+        const int ow = rem - oh * a.Wo;
+        ih0[t] = oh * a.stride - a.pt;
+        iw0[t] = ow * a.stride - a.pl;
+        in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+    }
+    // ---- per-lane filter rows ------------------------------------------------------------
+    const float *w_row[COT];
+    int co_of[COT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+    {
+        const int co = (cg * COT + c) * 32 + col;
+        co_of[c] = co;
+        const int cc = co < a.Co ? co : a.Co - 1;   // rows past Co compute garbage, never stored
+        w_row[c] = a.filt + (size_t)(cc / CB) * CiB * taps * (CB * CB) + (cc % CB) + half * 8 * CB;
+    }
+
+    floatx16 acc[COT][PXT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
+
+    // ---- K loop state: tap (ta, tb) outer, input channel block inner ---------------------
+    int ta = 0, tb = 0, cib = 0;
+    const int nsteps = taps * CiB;
+
+    auto load_step = [&](float (&A)[COT][8], float4 (&B)[PXT][2]) {
+        const int tap = ta * a.kw + tb;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
+            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
+            float4 v0 = p[0], v1 = p[1];
+            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
+            B[t][0] = v0;
+            B[t][1] = v1;
+        }
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+        {
+            const float *w = w_row[c] + ((size_t)cib * taps + tap) * (CB * CB);
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) A[c][kk] = w[kk * CB];
+        }
+        // advance
+        if (++cib == CiB)
+        {
+            cib = 0;
+            if (++tb == a.kw) { tb = 0; ++ta; }
+        }
+    };
+
+    auto compute_step = [&](const float (&A)[COT][8], const float4 (&B)[PXT][2]) {
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+        {
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                const float4 bv = B[t][kk >> 2];
+                const float b = (kk & 3) == 0 ? bv.x : (kk & 3) == 1 ? bv.y : (kk & 3) == 2 ? bv.z : bv.w;
+#pragma unroll
+                for (int c = 0; c < COT; ++c)
+                    acc[c][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[c][kk], b, acc[c][t], 0, 0, 0);
+            }
+        }
+    };
+
+    float A0[COT][8], A1[COT][8];
+    float4 B0[PXT][2], B1[PXT][2];
+    load_step(A0, B0);
+    for (int s = 0; s < nsteps; s += 2)
+    {
+        if (s + 1 < nsteps) load_step(A1, B1);
+        compute_step(A0, B0);
+        if (s + 1 < nsteps)
+        {
+            if (s + 2 < nsteps) load_step(A0, B0);
+            compute_step(A1, B1);
+        }
+    }
+
+    // ---- epilogue --------------------------------------------------------------------------
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+    {
+        const int co_tile = (cg * COT + c) * 32;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            if (!pvalid[t]) continue;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int co4 = co_tile + 8 * q + 4 * half;     // rows 8q + 4*half + {0..3}
+                if (co4 >= a.Co) continue;
+                float4 v = make_float4(acc[c][t][4 * q + 0], acc[c][t][4 * q + 1],
+                                       acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
+                float4 *o = reinterpret_cast<float4 *>(a.out + out_pix[t] +
+                                                       (size_t)(co4 / CB) * HoWo * CB + (co4 % CB));
+                if (a.accumulate)
+                {
+                    const float4 old = *o;
+                    v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+                }
+                if (a.bias)
+                {
+                    const float4 bb = *reinterpret_cast<const float4 *>(a.bias + co4);
+                    v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+                }
+                v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
+                v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
+                *o = v;
+            }
+        }
+    }
+    (void)co_of;
+}
+
+// ---------------------------------------------------------------------------------------------
+// first layers: Ci in {1,2,3}; input block is [H][W][Ci], filter [Co/16][kh][kw][Ci][16]
+// grid.x over pixels, grid.y = output channel block (uniform per workgroup -> scalar weight loads)
+template <int CI>
+__global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
+{
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= a.P) return;
+    const int cob = blockIdx.y;
+    const int HoWo = a.Ho * a.Wo;
+    const int n = p / HoWo;
+    const int rem = p - n * HoWo;
+    const int oh = rem / a.Wo;
+    const int ow = rem - oh * a.Wo;
+    const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+    const float *img = a.in + (size_t)n * a.H * a.W * CI;
+    const float *w = a.filt + (size_t)cob * a.kh * a.kw * CI * CB;
+    float *o = a.out + (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB;
+
+    float acc[CB];
+    if (a.accumulate)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const float4 v = reinterpret_cast<const float4 *>(o)[q];
+            acc[4 * q] = v.x; acc[4 * q + 1] = v.y; acc[4 * q + 2] = v.z; acc[4 * q + 3] = v.w;
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < CB; ++j) acc[j] = a.bias ? a.bias[cob * CB + j] : 0.f;
+    }
+    for (int ta = 0; ta < a.kh; ++ta)
+    {
+        const int ih = ih0 + ta;
+        if (ih < 0 || ih >= a.H) continue;
+        for (int tb = 0; tb < a.kw; ++tb)
+        {
+            const int iw = iw0 + tb;
+            if (iw < 0 || iw >= a.W) continue;
+            const float *ip = img + ((size_t)ih * a.W + iw) * CI;
+            const float *wp = w + (size_t)(ta * a.kw + tb) * CI * CB;
+#pragma unroll
+            for (int ci = 0; ci < CI; ++ci)
+            {
+                const float x = ip[ci];
+#pragma unroll
+                for (int j = 0; j < CB; ++j) acc[j] = fmaf(x, wp[ci * CB + j], acc[j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        float4 v = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+        if (a.accumulate && a.bias)
+        {
+            v.x += a.bias[cob * CB + 4 * q]; v.y += a.bias[cob * CB + 4 * q + 1];
+            v.z += a.bias[cob * CB + 4 * q + 2]; v.w += a.bias[cob * CB + 4 * q + 3];
+        }
+        v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
+        v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
+        reinterpret_cast<float4 *>(o)[q] = v;
+    }
+}
+
+template <int COT, int PXT>
+void launch_mfma(ConvArgs &a, hipStream_t s)
+{
+    a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
+    a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
+    a.n_blocks = a.n_co_groups * a.n_px_blocks;
+    a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
+    hipLaunchKernelGGL((conv_mfma_f32_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+}
+
+int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+             int Ci, int H, int W, const float *in, const float *filt, const float *bias, int act, float slope,
+             int accumulate, float *out, small_hip_stream_t stream)
+{
+    // interface_abstract.hpp:70-220: pick the channel branch first, the stride inside it
+    const bool blocked = Ci > 0 && Ci % CB == 0;
+    const bool small_ci = Ci == 1 || Ci == 2 || Ci == 3;
+    if (!blocked && !small_ci) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (Co % CB != 0) { set_error("%s: output_channels must be a multiple of 16 (pad the filter)", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out || !aligned16(filt) || !aligned16(out) || (blocked && !aligned16(in)) ||
+        (bias && !aligned16(bias)))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    if (act < SMALL_HIP_ACT_NONE || act > SMALL_HIP_ACT_LEAKY) { set_error("%s: bad activation", op); return SMALL_HIP_EINVAL; }
+
+    ConvArgs a{};
+    a.in = in; a.filt = filt; a.bias = bias; a.out = out;
+    a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W;
+    a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
+    a.Ho = out_dim(H, pt, pb, kh, stride);
+    a.Wo = out_dim(W, pl, pr, kw, stride);
+    a.act = act; a.slope = slope; a.accumulate = accumulate;
+    const long P = (long)batch * a.Ho * a.Wo;
+    if (P == 0) return SMALL_HIP_OK;
+    if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
+    a.P = (int)P;
+    hipStream_t s = as_stream(stream);
+
+    if (small_ci)
+    {
+        const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
+        if (Ci == 1) hipLaunchKernelGGL(conv_smallci_f32_kernel<1>, grid, dim3(256), 0, s, a);
+        else if (Ci == 2) hipLaunchKernelGGL(conv_smallci_f32_kernel<2>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(conv_smallci_f32_kernel<3>, grid, dim3(256), 0, s, a);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
+
+    // tile choice: the largest wave tile that still gives the chip ~2 waves per SIMD
+    const long target_waves = 2L * NUM_CU * 4;
+    auto waves = [&](int cot, int pxt) {
+        return (long)((Co + 32 * cot - 1) / (32 * cot)) * ((P + 32 * pxt - 1) / (32 * pxt));
+    };
+    if (Co % 64 == 0 && waves(2, 2) >= target_waves) launch_mfma<2, 2>(a, s);
+    else if (waves(1, 2) >= target_waves) launch_mfma<1, 2>(a, s);
+    else launch_mfma<1, 1>(a, s);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int small_hip_conv2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
+                         int H, int W, const float *in, const float *filt, float *out,
+                         small_hip_stream_t stream)
+{
+    return conv_f32("small_hip_conv2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt,
+                    nullptr, SMALL_HIP_ACT_NONE, 0.f, 0, out, stream);
+}
+
+int small_hip_partial_conv2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+                                 int Ci, int H, int W, const float *in, const float *filt, float *out,
+                                 small_hip_stream_t stream)
+{
+    return conv_f32("small_hip_partial_conv2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in,
+                    filt, nullptr, SMALL_HIP_ACT_NONE, 0.f, 1, out, stream);
+}
+
+int small_hip_conv2d_bias_act_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                  int Co, int Ci, int H, int W, const float *in, const float *filt,
+                                  const float *bias, int act, float slope, float *out,
+                                  small_hip_stream_t stream)
+{
+    return conv_f32("small_hip_conv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in,
+                    filt, bias, act, slope, 0, out, stream);
+}
+
+int small_hip_dense_f32(int batch, int No, int Ni, const float *in, const float *filt, float *out,
+                        small_hip_stream_t stream)
+{
+    return conv_f32("small_hip_dense_f32", batch, 1, 1, 1, 0, 0, 0, 0, No, Ni, 1, 1, in, filt, nullptr,
+                    SMALL_HIP_ACT_NONE, 0.f, 0, out, stream);
+}
+
+} // extern "C"

@@ -1,0 +1,459 @@
+// Conv2D / Dense (uint8, int32 accumulation, fused requantisation) for gfx950.
+//
+// The reference accumulates  acc = sum over VALID taps of (I + zI) * (F + zF)  in int32
+// (include/small/platforms/reference/intrinsics_quint8.h:191-223; padded taps are skipped, not
+// multiplied by the zero point) and requantises in the same pass.  Here the uint8 operands are
+// re-biased to signed bytes (x' = x - 128 = x ^ 0x80) so that the contraction runs on
+// v_mfma_i32_16x16x64_i8, and the zero-point terms are added back exactly in the epilogue:
+//
+//   acc = S + ZF * SI[px] + ZI * (SF[co][px] + ZF * Ci * nv[px])         (mod 2^32)
+//     S   = sum_valid I' * F'            (MFMA)
+//     SI  = sum_valid I'                 (v_sad_u8 on the bytes the lane loads anyway)
+//     SF  = sum over the valid taps of Wsum[co][tap],  Wsum = sum_ci F'   (filter pre-pass)
+//     nv  = number of valid taps,  ZI = zI + 128,  ZF = zF + 128
+//
+// A filter pre-pass (one small kernel) turns the packed filter [Co/16][Ci/16][tap][16 ci][16 co]
+// into the MFMA A-operand order [Co/16][step][16 co][16 ci] of signed bytes (step = tap*Ci/16 +
+// ci block, zero padded to a multiple of 4 steps) and produces Wsum / Wtot.  It does not depend
+// on any zero point, so a model can run it once per filter (small_hip_conv2d_u8_prepare_filter)
+// and call the prepared entry point per batch.
+//
+// MFMA mapping (16x16x64): rows = output channels, columns = output pixels, and each of the four
+// 16-lane groups of the wave supplies one K-step of 16 bytes -- a pixel's whole 16-channel block
+// is one 16-byte load.  A lane ends up with 4 consecutive output channels of one pixel:
+// requantise, pack, store one dword; the wave writes 256 contiguous bytes.
+#include "common.h"
+#include "quant.h"
+
+using namespace shp;
+
+namespace
+{
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+struct QConvArgs
+{
+    const uint8_t *in;
+    const int8_t *ft;        // prepared filter [Co/16][S_pad][16][16]
+    const int32_t *wsum;     // [Co][taps]
+    const int32_t *wtot;     // [Co]
+    uint8_t *out;
+    int batch, Co, Ci, H, W, Ho, Wo, kh, kw, stride, pt, pl;
+    int32_t ZI, ZF;          // zero points + 128
+    QOut q;
+    int P, S, S_pad, n_co_groups, n_px_blocks, n_blocks, per_xcd;
+};
+
+// ---- filter pre-pass ---------------------------------------------------------------------------
+// one lane per (co, step): reads 16 ci bytes at stride 16, writes 16 contiguous signed bytes
+__global__ __launch_bounds__(256) void prep_filter_u8_kernel(const uint8_t *__restrict__ f,
+                                                             int8_t *__restrict__ ft, int Co, int CiB,
+                                                             int taps, int S_pad)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= Co * S_pad) return;
+    const int co16 = i & 15;
+    const int s = (i >> 4) % S_pad;
+    const int cob = (i >> 4) / S_pad;
+    uint32_t w[4] = {0, 0, 0, 0};
+    if (s < taps * CiB)
+    {
+        const int tap = s / CiB, cib = s - tap * CiB;
+        const uint8_t *src = f + (((size_t)cob * CiB + cib) * taps + tap) * 256 + co16;
+#pragma unroll
+        for (int ci = 0; ci < 16; ++ci) w[ci >> 2] |= (uint32_t)(src[ci * 16] ^ 0x80u) << (8 * (ci & 3));
+    }
+    reinterpret_cast<uint4 *>(ft)[(size_t)(cob * S_pad + s) * 16 + co16] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// one lane per (co, tap): Wsum[co][tap] = sum_ci (F - 128); lane tap==0 also writes Wtot
+__global__ __launch_bounds__(256) void wsum_u8_kernel(const uint8_t *__restrict__ f, int32_t *__restrict__ wsum,
+                                                      int32_t *__restrict__ wtot, int Co, int CiB, int taps)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= Co) return;
+    const int cob = i >> 4, co16 = i & 15;
+    int32_t tot = 0;
+    for (int tap = 0; tap < taps; ++tap)
+    {
+        int32_t s = 0;
+        for (int cib = 0; cib < CiB; ++cib)
+        {
+            const uint8_t *src = f + (((size_t)cob * CiB + cib) * taps + tap) * 256 + co16;
+#pragma unroll
+            for (int ci = 0; ci < 16; ++ci) s += (int32_t)src[ci * 16] - 128;
+        }
+        wsum[(size_t)i * taps + tap] = s;
+        tot += s;
+    }
+    wtot[i] = tot;
+}
+
+// ---- main kernel --------------------------------------------------------------------------------
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
+{
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;
+    const int cg = lid % a.n_co_groups;
+    const int pxb = lid / a.n_co_groups;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = lane & 15;
+    const int grp = lane >> 4;
+
+    const int HoWo = a.Ho * a.Wo;
+    const int CiB = a.Ci / CB;
+    const int CoB = a.Co / CB;
+    const size_t in_blk = (size_t)a.H * a.W * CB;
+
+    const uint8_t *in_img[PXT];
+    int ih0[PXT], iw0[PXT], rem_of[PXT], n_of[PXT];
+    bool pvalid[PXT];
+    uint32_t sumI[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = ((pxb * 4 + wave) * PXT + t) * 16 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo;
+        const int rem = pc - n * HoWo;
+        const int oh = rem / a.Wo;
+        const int ow = rem - oh * a.Wo;
+        ih0[t] = oh * a.stride - a.pt;
+        iw0[t] = ow * a.stride - a.pl;
+        in_img[t] = a.in + (size_t)n * CiB * in_blk;
+        rem_of[t] = rem;
+        n_of[t] = n;
+        sumI[t] = 0;
+    }
+    // A rows: channel block (cg*COT + c), row `col`; blocks past Co are clamped and never stored
+    const int8_t *w_row[COT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+    {
+        int cob = cg * COT + c;
+        cob = cob < CoB ? cob : CoB - 1;
+        w_row[c] = a.ft + ((size_t)cob * a.S_pad * 16 + col) * 16;
+    }
+
+    v4i acc[COT][PXT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int t = 0; t < PXT; ++t) acc[c][t] = v4i{0, 0, 0, 0};
+
+    for (int s0 = 0; s0 < a.S_pad; s0 += 4)
+    {
+        const int s = s0 + grp;
+        const bool svalid = s < a.S;
+        const int sc = svalid ? s : 0;
+        const int tap = sc / CiB;
+        const int cib = sc - tap * CiB;
+        const int ta = tap / a.kw;
+        const int tb = tap - ta * a.kw;
+        v4i B[PXT];
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = svalid && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
+            uint4 v = *reinterpret_cast<const uint4 *>(in_img[t] + off);
+            if (!ok) v = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
+            // sum of the 16 raw bytes minus 16*128 = sum of the signed bytes (0 for masked taps)
+            uint32_t sb = __builtin_amdgcn_sad_u8(v.x, 0u, 0u);
+            sb = __builtin_amdgcn_sad_u8(v.y, 0u, sb);
+            sb = __builtin_amdgcn_sad_u8(v.z, 0u, sb);
+            sb = __builtin_amdgcn_sad_u8(v.w, 0u, sb);
+            sumI[t] += sb - 2048u;
+            B[t] = v4i{(int)(v.x ^ 0x80808080u), (int)(v.y ^ 0x80808080u), (int)(v.z ^ 0x80808080u),
+                       (int)(v.w ^ 0x80808080u)};
+        }
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+        {
+            const uint4 w = *reinterpret_cast<const uint4 *>(w_row[c] + (size_t)s * 256);
+            const v4i A = v4i{(int)w.x, (int)w.y, (int)w.z, (int)w.w};
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+                acc[c][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B[t], acc[c][t], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: zero-point terms, requantise, pack, store ------------------------------------
+    const int taps = a.kh * a.kw;
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        // total over the four K groups of this pixel column
+        uint32_t si = sumI[t];
+        si += (uint32_t)__shfl_xor((int)si, 16);
+        si += (uint32_t)__shfl_xor((int)si, 32);
+        if (!pvalid[t]) continue;
+        // valid tap rectangle of this pixel
+        const int a_lo = ih0[t] < 0 ? -ih0[t] : 0;
+        const int a_hi = (a.H - ih0[t]) < a.kh ? (a.H - ih0[t]) : a.kh;
+        const int b_lo = iw0[t] < 0 ? -iw0[t] : 0;
+        const int b_hi = (a.W - iw0[t]) < a.kw ? (a.W - iw0[t]) : a.kw;
+        const int na = a_hi > a_lo ? a_hi - a_lo : 0, nb = b_hi > b_lo ? b_hi - b_lo : 0;
+        const bool full = (na == a.kh) && (nb == a.kw);
+        const uint32_t base = (uint32_t)a.ZF * si;
+        const uint32_t cnt = (uint32_t)a.ZF * (uint32_t)(a.Ci * na * nb);
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+        {
+            const int cob = cg * COT + c;
+            if (cob >= CoB) continue;
+            uint32_t packed = 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                const int co = cob * CB + 4 * grp + r;
+                uint32_t sf;
+                if (full) sf = (uint32_t)a.wtot[co];
+                else
+                {
+                    sf = 0;
+                    for (int ta = a_lo; ta < a_hi; ++ta)
+                        for (int tb = b_lo; tb < b_hi; ++tb)
+                            sf += (uint32_t)a.wsum[(size_t)co * taps + ta * a.kw + tb];
+                }
+                const uint32_t v = (uint32_t)acc[c][t][r] + base + (uint32_t)a.ZI * (sf + cnt);
+                packed |= requant_u8((int32_t)v, a.q) << (8 * r);
+            }
+            uint32_t *o = reinterpret_cast<uint32_t *>(
+                a.out + (((size_t)n_of[t] * CoB + cob) * HoWo + rem_of[t]) * CB + 4 * grp);
+            *o = packed;
+        }
+    }
+}
+
+// ---- first layers (Ci in {1,2,3}): vector ALU, direct (I + zI) * (F + zF) ----------------------------
+struct QSmallArgs
+{
+    const uint8_t *in;
+    const uint8_t *filt;
+    uint8_t *out;
+    int batch, Co, H, W, Ho, Wo, kh, kw, stride, pt, pl, P;
+    int32_t zi, zf;
+    QOut q;
+};
+
+template <int CI>
+__global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a)
+{
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= a.P) return;
+    const int cob = blockIdx.y;
+    const int HoWo = a.Ho * a.Wo;
+    const int n = p / HoWo;
+    const int rem = p - n * HoWo;
+    const int oh = rem / a.Wo;
+    const int ow = rem - oh * a.Wo;
+    const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+    const uint8_t *img = a.in + (size_t)n * a.H * a.W * CI;
+    const uint8_t *w = a.filt + (size_t)cob * a.kh * a.kw * CI * CB;
+    uint32_t acc[CB];
+#pragma unroll
+    for (int j = 0; j < CB; ++j) acc[j] = 0;
+    for (int ta = 0; ta < a.kh; ++ta)
+    {
+        const int ih = ih0 + ta;
+        if (ih < 0 || ih >= a.H) continue;
+        for (int tb = 0; tb < a.kw; ++tb)
+        {
+            const int iw = iw0 + tb;
+            if (iw < 0 || iw >= a.W) continue;
+            const uint8_t *ip = img + ((size_t)ih * a.W + iw) * CI;
+            const uint8_t *wp = w + (size_t)(ta * a.kw + tb) * CI * CB;
+#pragma unroll
+            for (int ci = 0; ci < CI; ++ci)
+            {
+                const uint32_t x = (uint32_t)((int32_t)ip[ci] + a.zi);
+#pragma unroll
+                for (int j = 0; j < CB; ++j) acc[j] += x * (uint32_t)((int32_t)wp[ci * CB + j] + a.zf);
+            }
+        }
+    }
+    uint32_t pk[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < CB; ++j) pk[j >> 2] |= requant_u8((int32_t)acc[j], a.q) << (8 * (j & 3));
+    uint4 *o = reinterpret_cast<uint4 *>(a.out + (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB);
+    *o = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+}
+
+size_t ws_ft_bytes(int Co, int S_pad) { return (size_t)Co * S_pad * 16; }
+
+size_t prepared_bytes(int kh, int kw, int Co, int Ci)
+{
+    const int S = kh * kw * (Ci / CB), S_pad = (S + 3) & ~3;
+    size_t b = ws_ft_bytes(Co, S_pad);                 // multiple of 64
+    b += (size_t)Co * kh * kw * sizeof(int32_t);       // wsum
+    b += (size_t)Co * sizeof(int32_t);                 // wtot
+    return (b + 255) & ~(size_t)255;
+}
+
+int prepare_filter(int kh, int kw, int Co, int Ci, const uint8_t *filt, void *ws, hipStream_t s)
+{
+    const int CiB = Ci / CB, taps = kh * kw, S = taps * CiB, S_pad = (S + 3) & ~3;
+    int8_t *ft = static_cast<int8_t *>(ws);
+    int32_t *wsum = reinterpret_cast<int32_t *>(ft + ws_ft_bytes(Co, S_pad));
+    int32_t *wtot = wsum + (size_t)Co * taps;
+    const int n1 = Co * S_pad;
+    hipLaunchKernelGGL(prep_filter_u8_kernel, dim3((n1 + 255) / 256), dim3(256), 0, s, filt, ft, Co, CiB, taps, S_pad);
+    SHP_LAUNCH_CHECK("prep_filter_u8_kernel");
+    hipLaunchKernelGGL(wsum_u8_kernel, dim3((Co + 255) / 256), dim3(256), 0, s, filt, wsum, wtot, Co, CiB, taps);
+    SHP_LAUNCH_CHECK("wsum_u8_kernel");
+    return SMALL_HIP_OK;
+}
+
+template <int COT, int PXT>
+void launch_q(QConvArgs &a, hipStream_t s)
+{
+    a.n_co_groups = (a.Co / CB + COT - 1) / COT;
+    a.n_px_blocks = (a.P + 16 * PXT * 4 - 1) / (16 * PXT * 4);
+    a.n_blocks = a.n_co_groups * a.n_px_blocks;
+    a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
+    hipLaunchKernelGGL((conv_mfma_u8_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+}
+
+int conv_u8_check(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+                  int Ci, int H, int W, const void *in, const void *filt, const void *out,
+                  const small_hip_quant *iq, const small_hip_quant *fq, const small_hip_quant *oq)
+{
+    const bool blocked = Ci > 0 && Ci % CB == 0;
+    const bool small_ci = Ci == 1 || Ci == 2 || Ci == 3;
+    if (!blocked && !small_ci) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (Co % CB != 0) { set_error("%s: output_channels must be a multiple of 16 (pad the filter)", op); return SMALL_HIP_EINVAL; }
+    if (!iq || !fq || !oq) { set_error("%s: null quantisation parameters", op); return SMALL_HIP_EINVAL; }
+    if (oq->rshift < 0 || oq->rshift > 31 || oq->lshift < 0 || oq->lshift > 31)
+    { set_error("%s: shift out of range", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out || !aligned16(filt) || !aligned16(out) || (blocked && !aligned16(in)))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    return SMALL_HIP_OK;
+}
+
+int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+                int Ci, int H, int W, const uint8_t *in, const small_hip_quant *iq, const void *prepared,
+                const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, hipStream_t s)
+{
+    QConvArgs a{};
+    const int CiB = Ci / CB, taps = kh * kw;
+    a.S = taps * CiB;
+    a.S_pad = (a.S + 3) & ~3;
+    a.in = in; a.out = out;
+    a.ft = static_cast<const int8_t *>(prepared);
+    a.wsum = reinterpret_cast<const int32_t *>(a.ft + ws_ft_bytes(Co, a.S_pad));
+    a.wtot = a.wsum + (size_t)Co * taps;
+    a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W; a.kh = kh; a.kw = kw;
+    a.stride = stride; a.pt = pt; a.pl = pl;
+    a.Ho = out_dim(H, pt, pb, kh, stride);
+    a.Wo = out_dim(W, pl, pr, kw, stride);
+    a.ZI = (int32_t)((uint32_t)iq->zero + 128u);
+    a.ZF = (int32_t)((uint32_t)fq->zero + 128u);
+    a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
+    const long P = (long)batch * a.Ho * a.Wo;
+    if (P == 0) return SMALL_HIP_OK;
+    if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
+    a.P = (int)P;
+    const int CoB = Co / CB;
+    if (CoB >= 4 && CoB % 4 == 0) launch_q<4, 2>(a, s);
+    else if (CoB % 2 == 0) launch_q<2, 2>(a, s);
+    else launch_q<1, 2>(a, s);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
+            int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
+            const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt, out, iq, fq, oq))
+        return rc;
+    hipStream_t s = as_stream(stream);
+    if (Ci < CB)
+    {
+        QSmallArgs a{};
+        a.in = in; a.filt = filt; a.out = out; a.batch = batch; a.Co = Co; a.H = H; a.W = W;
+        a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
+        a.Ho = out_dim(H, pt, pb, kh, stride);
+        a.Wo = out_dim(W, pl, pr, kw, stride);
+        a.zi = iq->zero; a.zf = fq->zero;
+        a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
+        const long P = (long)batch * a.Ho * a.Wo;
+        if (P == 0) return SMALL_HIP_OK;
+        if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
+        a.P = (int)P;
+        const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
+        if (Ci == 1) hipLaunchKernelGGL(conv_smallci_u8_kernel<1>, grid, dim3(256), 0, s, a);
+        else if (Ci == 2) hipLaunchKernelGGL(conv_smallci_u8_kernel<2>, grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(conv_smallci_u8_kernel<3>, grid, dim3(256), 0, s, a);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
+    void *ws = nullptr;
+    if (int rc = get_workspace(prepared_bytes(kh, kw, Co, Ci), &ws)) return rc;
+    if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
+    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, s);
+}
+
+} // namespace
+
+extern "C" {
+
+int small_hip_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
+                        int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
+                        const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq,
+                        small_hip_stream_t stream)
+{
+    return conv_u8("small_hip_conv2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, filt, fq,
+                   out, oq, stream);
+}
+
+int small_hip_dense_u8(int batch, int No, int Ni, const uint8_t *in, const small_hip_quant *iq,
+                       const uint8_t *filt, const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq,
+                       small_hip_stream_t stream)
+{
+    return conv_u8("small_hip_dense_u8", batch, 1, 1, 1, 0, 0, 0, 0, No, Ni, 1, 1, in, iq, filt, fq, out, oq,
+                   stream);
+}
+
+size_t small_hip_conv2d_u8_prepared_filter_bytes(int kh, int kw, int Co, int Ci)
+{
+    if (kh <= 0 || kw <= 0 || Co <= 0 || Co % CB != 0 || Ci <= 0 || Ci % CB != 0) return 0;
+    return prepared_bytes(kh, kw, Co, Ci);
+}
+
+int small_hip_conv2d_u8_prepare_filter(int kh, int kw, int Co, int Ci, const uint8_t *filt, void *prepared,
+                                       small_hip_stream_t stream)
+{
+    if (kh <= 0 || kw <= 0 || Co <= 0 || Co % CB != 0) return einval("small_hip_conv2d_u8_prepare_filter: bad size");
+    if (Ci <= 0 || Ci % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (!filt || !prepared || !aligned16(filt) || !aligned16(prepared))
+        return einval("small_hip_conv2d_u8_prepare_filter: null or misaligned pointer");
+    return prepare_filter(kh, kw, Co, Ci, filt, prepared, as_stream(stream));
+}
+
+int small_hip_conv2d_u8_prepared(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+                                 int Ci, int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                                 const void *prepared, const small_hip_quant *fq, uint8_t *out,
+                                 const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_conv2d_u8_prepared";
+    if (Ci <= 0 || Ci % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, prepared, out, iq, fq, oq))
+        return rc;
+    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, prepared, fq, out, oq,
+                       as_stream(stream));
+}
+
+} // extern "C"

@@ -1,0 +1,209 @@
+// DepthwiseConv2D / PartialDepthwiseConv2D (float32, optional fused bias + activation) and
+// DepthwiseConv2D (uint8).  Bandwidth-bound, no MFMA: a lane owns four channels of one output
+// pixel, so the four lanes of a (pixel, channel-block) read one 64-byte line per tap and a wave
+// covers 16 neighbouring output pixels.  Filter taps ([C/16][kh][kw][16], 576 bytes per block for
+// 3x3) are read through the vector cache; every lane of a workgroup row uses the same lines.
+#include "common.h"
+#include "quant.h"
+
+using namespace shp;
+
+namespace
+{
+
+constexpr int TPB = 256;
+
+struct Epi
+{
+    const float4 *bias;   // may be null
+    int act;
+    float slope;
+    int accumulate;
+};
+
+__device__ __forceinline__ float act1(float v, int act, float slope)
+{
+    if (act == SMALL_HIP_ACT_RELU) return v > 0.f ? v : 0.f;
+    if (act == SMALL_HIP_ACT_LEAKY) return v > 0.f ? v : v * slope;
+    return v;
+}
+
+// KH/KW == 0: run-time window size
+template <int KH, int KW>
+__global__ __launch_bounds__(TPB) void dw_f32_kernel(const float4 *__restrict__ in,
+                                                     const float4 *__restrict__ filt, float4 *out,
+                                                     size_t total4, int cblocks, Geom g, Epi e)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= total4) return;
+    const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
+    const int q = (int)(i & 3);
+    size_t pix = i >> 2;
+    const int ow = (int)(pix % (size_t)g.Wo);
+    pix /= (size_t)g.Wo;
+    const int oh = (int)(pix % (size_t)g.Ho);
+    const size_t plane = pix / (size_t)g.Ho;              // n * cblocks + cb
+    const int cbk = (int)(plane % (size_t)cblocks);
+    const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
+    const float4 *f = filt + (size_t)cbk * kh * kw * 4 + q;
+    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (e.accumulate) acc = out[i];
+    else if (e.bias) acc = e.bias[cbk * 4 + q];
+#pragma unroll
+    for (int a = 0; a < kh; ++a)
+    {
+        const int ih = ih0 + a;
+        if (ih < 0 || ih >= g.H) continue;
+#pragma unroll
+        for (int b = 0; b < kw; ++b)
+        {
+            const int iw = iw0 + b;
+            if (iw < 0 || iw >= g.W) continue;
+            const float4 v = src[((size_t)ih * g.W + iw) * 4];
+            const float4 w = f[(a * kw + b) * 4];
+            acc.x = fmaf(v.x, w.x, acc.x); acc.y = fmaf(v.y, w.y, acc.y);
+            acc.z = fmaf(v.z, w.z, acc.z); acc.w = fmaf(v.w, w.w, acc.w);
+        }
+    }
+    acc.x = act1(acc.x, e.act, e.slope); acc.y = act1(acc.y, e.act, e.slope);
+    acc.z = act1(acc.z, e.act, e.slope); acc.w = act1(acc.w, e.act, e.slope);
+    out[i] = acc;
+}
+
+__global__ __launch_bounds__(TPB) void dw_u8_kernel(const uint32_t *__restrict__ in,
+                                                    const uint32_t *__restrict__ filt,
+                                                    uint32_t *__restrict__ out, size_t total,
+                                                    int cblocks, Geom g, int32_t zi, int32_t zf, QOut qo)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= total) return;
+    const int q = (int)(i & 3);
+    size_t pix = i >> 2;
+    const int ow = (int)(pix % (size_t)g.Wo);
+    pix /= (size_t)g.Wo;
+    const int oh = (int)(pix % (size_t)g.Ho);
+    const size_t plane = pix / (size_t)g.Ho;
+    const int cbk = (int)(plane % (size_t)cblocks);
+    const uint32_t *src = in + plane * (size_t)g.H * g.W * 4 + q;
+    const uint32_t *f = filt + (size_t)cbk * g.kh * g.kw * 4 + q;
+    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    uint32_t acc[4] = {0, 0, 0, 0};
+    for (int a = 0; a < g.kh; ++a)
+    {
+        const int ih = ih0 + a;
+        if (ih < 0 || ih >= g.H) continue;
+        for (int b = 0; b < g.kw; ++b)
+        {
+            const int iw = iw0 + b;
+            if (iw < 0 || iw >= g.W) continue;
+            const uint32_t v = src[((size_t)ih * g.W + iw) * 4];
+            const uint32_t w = f[(a * g.kw + b) * 4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                acc[c] += (uint32_t)((int32_t)((v >> (8 * c)) & 0xffu) + zi) *
+                          (uint32_t)((int32_t)((w >> (8 * c)) & 0xffu) + zf);
+        }
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) packed |= requant_u8((int32_t)acc[c], qo) << (8 * c);
+    out[i] = packed;
+}
+
+int dw_check(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+             int H, int W, const void *in, const void *filt, const void *out, Geom *g)
+{
+    // interface_abstract.hpp:1013-1050: channel test first, then stride
+    if (C <= 0 || C % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out || !aligned16(in) || !aligned16(filt) || !aligned16(out))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
+    g->Ho = out_dim(H, pt, pb, kh, stride);
+    g->Wo = out_dim(W, pl, pr, kw, stride);
+    return SMALL_HIP_OK;
+}
+
+int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C, int H,
+           int W, const float *in, const float *filt, const float *bias, int act, float slope, int accumulate,
+           float *out, small_hip_stream_t stream)
+{
+    Geom g;
+    if (int rc = dw_check(op, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, filt, out, &g)) return rc;
+    if (bias && !aligned16(bias)) { set_error("%s: misaligned bias", op); return SMALL_HIP_EINVAL; }
+    if (act < SMALL_HIP_ACT_NONE || act > SMALL_HIP_ACT_LEAKY) { set_error("%s: bad activation", op); return SMALL_HIP_EINVAL; }
+    const size_t total4 = (size_t)batch * C * g.Ho * g.Wo / 4;
+    if (total4 == 0) return SMALL_HIP_OK;
+    const Epi e{reinterpret_cast<const float4 *>(bias), act, slope, accumulate};
+    const dim3 grid((unsigned)((total4 + TPB - 1) / TPB)), block(TPB);
+    auto k = (kh == 3 && kw == 3) ? dw_f32_kernel<3, 3> : dw_f32_kernel<0, 0>;
+    hipLaunchKernelGGL(k, grid, block, 0, as_stream(stream), reinterpret_cast<const float4 *>(in),
+                       reinterpret_cast<const float4 *>(filt), reinterpret_cast<float4 *>(out), total4,
+                       C / CB, g, e);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int small_hip_depthwise_conv2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                   int C, int H, int W, const float *in, const float *filt, float *out,
+                                   small_hip_stream_t stream)
+{
+    return dw_f32("small_hip_depthwise_conv2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, filt,
+                  nullptr, SMALL_HIP_ACT_NONE, 0.f, 0, out, stream);
+}
+
+int small_hip_partial_depthwise_conv2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl,
+                                           int pr, int C, int H, int W, const float *in, const float *filt,
+                                           float *out, small_hip_stream_t stream)
+{
+    return dw_f32("small_hip_partial_depthwise_conv2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in,
+                  filt, nullptr, SMALL_HIP_ACT_NONE, 0.f, 1, out, stream);
+}
+
+int small_hip_depthwise_conv2d_bias_act_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl,
+                                            int pr, int C, int H, int W, const float *in, const float *filt,
+                                            const float *bias, int act, float slope, float *out,
+                                            small_hip_stream_t stream)
+{
+    return dw_f32("small_hip_depthwise_conv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in,
+                  filt, bias, act, slope, 0, out, stream);
+}
+
+int small_hip_dense_literal_f32(int No, int Ni, const float *in, const float *filt, float *out,
+                                small_hip_stream_t stream)
+{
+    // interface_abstract.hpp:2113-2132: a 1x1 depthwise over a 1 x Ni image with No channels;
+    // no channel-count check there, but the packed layout needs whole blocks
+    if (No <= 0 || No % CB != 0) return einval("small_hip_dense_literal_f32: output_elements must be a multiple of 16");
+    return dw_f32("small_hip_dense_literal_f32", 1, 1, 1, 1, 0, 0, 0, 0, No, 1, Ni, in, filt, nullptr,
+                  SMALL_HIP_ACT_NONE, 0.f, 0, out, stream);
+}
+
+int small_hip_depthwise_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+                                  int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                                  const uint8_t *filt, const small_hip_quant *fq, uint8_t *out,
+                                  const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_depthwise_conv2d_u8";
+    if (!iq || !fq || !oq) return einval("small_hip_depthwise_conv2d_u8: null quantisation parameters");
+    Geom g;
+    if (int rc = dw_check(op, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, filt, out, &g)) return rc;
+    const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
+    if (total == 0) return SMALL_HIP_OK;
+    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    hipLaunchKernelGGL(dw_u8_kernel, dim3((unsigned)((total + TPB - 1) / TPB)), dim3(TPB), 0, as_stream(stream),
+                       reinterpret_cast<const uint32_t *>(in), reinterpret_cast<const uint32_t *>(filt),
+                       reinterpret_cast<uint32_t *>(out), total, C / CB, g, iq->zero, fq->zero, q);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,191 @@
+// MaxPool2D / AveragePool2D, float32 and uint8.  Bandwidth-bound: one lane produces four
+// channels (16 bytes of float, or 4 bytes of uint8) of one output pixel; the four lanes of a
+// pixel-block read one 64-byte line per tap, neighbouring lanes read neighbouring pixels.
+//
+// Reference semantics kept bit-for-bit:
+//   - max-pool windows that touch padding include the value 0 in the maximum
+//     (abstract_layer.hpp:514-521, 718-728 zero the tile and only max valid taps)
+//   - average-pool multiplies the sum of the valid taps by float(1.0 / (kh*kw))
+//     (abstract_layer.hpp:565-569), i.e. padded positions count in the divisor
+#include "common.h"
+#include "quant.h"
+
+using namespace shp;
+
+namespace
+{
+
+constexpr int TPB = 256;
+
+template <bool IS_MAX>
+__global__ __launch_bounds__(TPB) void pool_f32_kernel(const float4 *__restrict__ in,
+                                                       float4 *__restrict__ out, size_t total4,
+                                                       Geom g, float norm)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= total4) return;
+    const int q = (int)(i & 3);
+    size_t pix = i >> 2;
+    const int ow = (int)(pix % (size_t)g.Wo);
+    pix /= (size_t)g.Wo;
+    const int oh = (int)(pix % (size_t)g.Ho);
+    const size_t plane = pix / (size_t)g.Ho;              // n * cblocks + cb
+    const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
+    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (IS_MAX && full) acc = src[((size_t)ih0 * g.W + iw0) * 4];
+    for (int a = 0; a < g.kh; ++a)
+    {
+        const int ih = ih0 + a;
+        if (ih < 0 || ih >= g.H) continue;
+        for (int b = 0; b < g.kw; ++b)
+        {
+            const int iw = iw0 + b;
+            if (iw < 0 || iw >= g.W) continue;
+            const float4 v = src[((size_t)ih * g.W + iw) * 4];
+            if (IS_MAX)
+            {
+                acc.x = v.x > acc.x ? v.x : acc.x; acc.y = v.y > acc.y ? v.y : acc.y;
+                acc.z = v.z > acc.z ? v.z : acc.z; acc.w = v.w > acc.w ? v.w : acc.w;
+            }
+            else
+            {
+                acc.x = acc.x + v.x; acc.y = acc.y + v.y; acc.z = acc.z + v.z; acc.w = acc.w + v.w;
+            }
+        }
+    }
+    if (!IS_MAX) { acc.x *= norm; acc.y *= norm; acc.z *= norm; acc.w *= norm; }
+    out[i] = acc;
+}
+
+// uint8: a lane owns 4 channels (one dword) of one output pixel
+template <bool IS_MAX>
+__global__ __launch_bounds__(TPB) void pool_u8_kernel(const uint32_t *__restrict__ in,
+                                                      uint32_t *__restrict__ out, size_t total,
+                                                      Geom g, int32_t zi, QOut qo)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= total) return;
+    const int q = (int)(i & 3);
+    size_t pix = i >> 2;
+    const int ow = (int)(pix % (size_t)g.Wo);
+    pix /= (size_t)g.Wo;
+    const int oh = (int)(pix % (size_t)g.Ho);
+    const size_t plane = pix / (size_t)g.Ho;
+    const uint32_t *src = in + plane * (size_t)g.H * g.W * 4 + q;
+    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
+    int32_t acc[4] = {0, 0, 0, 0};
+    if (IS_MAX && full)
+    {
+        // q_abstract_layer.hpp:286-293: un-padded windows start from the first RAW byte
+        const uint32_t v = src[((size_t)ih0 * g.W + iw0) * 4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[b] = (int32_t)((v >> (8 * b)) & 0xffu);
+    }
+    for (int a = 0; a < g.kh; ++a)
+    {
+        const int ih = ih0 + a;
+        if (ih < 0 || ih >= g.H) continue;
+        for (int c = 0; c < g.kw; ++c)
+        {
+            const int iw = iw0 + c;
+            if (iw < 0 || iw >= g.W) continue;
+            const uint32_t v = src[((size_t)ih * g.W + iw) * 4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+            {
+                const int32_t x = (int32_t)((v >> (8 * b)) & 0xffu) + zi;
+                if (IS_MAX) acc[b] = x > acc[b] ? x : acc[b];
+                else acc[b] = (int32_t)((uint32_t)acc[b] + (uint32_t)x);
+            }
+        }
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) packed |= requant_u8(acc[b], qo) << (8 * b);
+    out[i] = packed;
+}
+
+int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, int pt, int pb, int pl,
+               int pr, int C, int H, int W, const void *in, const void *out, Geom *g)
+{
+    // interface_abstract.hpp:797-833 / 929-977: channel test first, then stride
+    if (C <= 0 || C % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (avg ? (stride < 1 || stride > 3) : (stride != 1 && stride != 2)) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (!in || !out || !aligned16(in) || !aligned16(out)) { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place pooling is not supported", op); return SMALL_HIP_EINVAL; }
+    g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
+    g->Ho = out_dim(H, pt, pb, kh, stride);
+    g->Wo = out_dim(W, pl, pr, kw, stride);
+    return SMALL_HIP_OK;
+}
+
+template <bool IS_MAX>
+int pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+             int H, int W, const float *in, float *out, small_hip_stream_t stream)
+{
+    Geom g;
+    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
+    const size_t total4 = (size_t)batch * C * g.Ho * g.Wo / 4;
+    if (total4 == 0) return SMALL_HIP_OK;
+    const float norm = (float)(1.0 / (1.0 * kh * kw));
+    hipLaunchKernelGGL(pool_f32_kernel<IS_MAX>, dim3((unsigned)((total4 + TPB - 1) / TPB)), dim3(TPB), 0,
+                       as_stream(stream), reinterpret_cast<const float4 *>(in),
+                       reinterpret_cast<float4 *>(out), total4, g, norm);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+template <bool IS_MAX>
+int pool_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+            int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
+            const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    if (!iq || !oq) { set_error("%s: null quantisation parameters", op); return SMALL_HIP_EINVAL; }
+    Geom g;
+    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
+    const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
+    if (total == 0) return SMALL_HIP_OK;
+    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    hipLaunchKernelGGL(pool_u8_kernel<IS_MAX>, dim3((unsigned)((total + TPB - 1) / TPB)), dim3(TPB), 0,
+                       as_stream(stream), reinterpret_cast<const uint32_t *>(in),
+                       reinterpret_cast<uint32_t *>(out), total, g, iq->zero, q);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int small_hip_maxpool2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+                            int H, int W, const float *in, float *out, small_hip_stream_t stream)
+{
+    return pool_f32<true>("small_hip_maxpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, stream);
+}
+
+int small_hip_avgpool2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+                            int H, int W, const float *in, float *out, small_hip_stream_t stream)
+{
+    return pool_f32<false>("small_hip_avgpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, stream);
+}
+
+int small_hip_maxpool2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+                           int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
+                           const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    return pool_u8<true>("small_hip_maxpool2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
+}
+
+int small_hip_avgpool2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+                           int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
+                           const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    return pool_u8<false>("small_hip_avgpool2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
+}
+
+} // extern "C"
