@@ -1,0 +1,452 @@
+"""The benchmark topologies as flat lists of `small::` layer calls on named buffers.
+
+A model is a list of Op records; executors interpret it:
+  HipExecutor (here)         device buffers + libsmall_hip.so through the C ABI
+  oracle / reference runners live with the test infrastructure, not in this package
+
+Topologies (synthetic weights; shapes as the benchmark configurations name them):
+  dscnn()        DS-CNN keyword spotting, float32, 49x10x1
+  mobilenet_v1() MobileNetV1 1.0, float32, 224x224x3
+  tiny_yolo_v2() Tiny-YOLOv2, float32, 416x416x3
+  resnet8_u8()   ResNet-8, quantised uint8, 32x32x3
+  layer_sweep()  single layers at C=256, 56x56
+"""
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+
+from . import capi, layout, synth
+
+CB = 16
+
+
+@dataclass
+class Op:
+    kind: str                      # conv dw maxpool avgpool relu leaky accum dense
+    src: str
+    dst: str
+    C: int = 0                     # input channels
+    H: int = 0
+    W: int = 0
+    Co: int = 0                    # output channels (conv/dense: padded to a multiple of 16)
+    Co_eff: int = 0                # channels that carry information (e.g. 1000 of 1008)
+    kh: int = 1
+    kw: int = 1
+    stride: int = 1
+    pads: Tuple[int, int, int, int] = (0, 0, 0, 0)   # t, b, l, r
+    weight: Optional[str] = None
+    act: Optional[str] = None      # fused activation of a conv/dw: relu | leaky
+    slope: float = 0.0
+    name: str = ""
+
+    @property
+    def Ho(self):
+        return capi.out_dim(self.H, self.pads[0], self.pads[1], self.kh, self.stride)
+
+    @property
+    def Wo(self):
+        return capi.out_dim(self.W, self.pads[2], self.pads[3], self.kw, self.stride)
+
+    def out_channels(self):
+        return self.Co if self.kind in ("conv", "dense") else self.C
+
+    def out_shape(self):
+        if self.kind == "dense":
+            return (self.Co, 1, 1)
+        if self.kind in ("relu", "leaky", "accum"):
+            return (self.C, self.H, self.W)
+        return (self.out_channels(), self.Ho, self.Wo)
+
+    # ---- algorithmic work per image ---------------------------------------------------------
+    def flops(self):
+        if self.kind in ("conv", "dense"):
+            return 2 * self.Ho * self.Wo * (self.Co_eff or self.Co) * self.C * self.kh * self.kw
+        if self.kind == "dw":
+            return 2 * self.Ho * self.Wo * self.C * self.kh * self.kw
+        return 0
+
+    def act_elems(self):
+        """(input elements, output elements) per image, each tensor once."""
+        c, h, w = self.out_shape()
+        return self.C * self.H * self.W, c * h * w
+
+    def weight_elems(self):
+        if self.kind in ("conv", "dense"):
+            return self.Co * self.C * self.kh * self.kw
+        if self.kind == "dw":
+            return self.C * self.kh * self.kw
+        return 0
+
+
+@dataclass
+class Model:
+    name: str
+    dtype: str                      # "f32" or "u8"
+    in_shape: Tuple[int, int, int]  # C, H, W
+    ops: List[Op]
+    input_kind: str = "normal"      # normal | uniform01 | u8
+    out: str = ""
+    quant: Dict[str, Tuple[int, int, int, int]] = field(default_factory=dict)   # tensor -> (zero, mult, lshift, rshift)
+
+    def flops_per_image(self):
+        return sum(o.flops() for o in self.ops)
+
+    def esize(self):
+        return 4 if self.dtype == "f32" else 1
+
+
+def same_pads(H, W, kh, kw, s):
+    t, b = capi.calc_padding(H, kh, s)
+    l, r = capi.calc_padding(W, kw, s)
+    return (t, b, l, r)
+
+
+class _Builder:
+    """Tracks the running (C, H, W) and ping-pongs between buffers."""
+
+    def __init__(self, name, dtype, in_shape, input_kind):
+        self.m = Model(name, dtype, in_shape, [], input_kind)
+        self.c, self.h, self.w = in_shape
+        self.cur = "in"
+        self.n = 0
+
+    def _next(self, avoid=()):
+        for cand in ("b0", "b1", "b2"):
+            if cand != self.cur and cand not in avoid:
+                return cand
+        raise RuntimeError("no free buffer")
+
+    def conv(self, co, k, s=1, pad="same", act=None, slope=0.0, src=None, dst=None, kw=None, co_eff=None):
+        kh, kw = (k, kw or k)
+        src = src or self.cur
+        pads = same_pads(self.h, self.w, kh, kw, s) if pad == "same" else (0, 0, 0, 0)
+        cop = layout.pad_channels(co)
+        dst = dst or self._next()
+        wname = "w%d" % self.n
+        op = Op("conv", src, dst, C=self.c, H=self.h, W=self.w, Co=cop, Co_eff=co_eff or co, kh=kh, kw=kw, stride=s,
+                pads=pads, weight=wname, act=act, slope=slope, name="conv%d_%dx%d_s%d_%d-%d" % (self.n, kh, kw, s, self.c, co))
+        self.n += 1
+        self.m.ops.append(op)
+        return op
+
+    def advance(self, op):
+        self.c, self.h, self.w = op.out_shape()
+        self.cur = op.dst
+
+    def dw(self, k, s=1, act=None):
+        pads = same_pads(self.h, self.w, k, k, s)
+        op = Op("dw", self.cur, self._next(), C=self.c, H=self.h, W=self.w, kh=k, kw=k, stride=s, pads=pads,
+                weight="w%d" % self.n, act=act, name="dw%d_%dx%d_s%d_%d" % (self.n, k, k, s, self.c))
+        self.n += 1
+        self.m.ops.append(op)
+        self.advance(op)
+        return op
+
+    def pool(self, kind, kh, kw, s, pad="valid"):
+        pads = same_pads(self.h, self.w, kh, kw, s) if pad == "same" else (0, 0, 0, 0)
+        op = Op(kind, self.cur, self._next(), C=self.c, H=self.h, W=self.w, kh=kh, kw=kw, stride=s, pads=pads,
+                name="%s_%dx%d_s%d_%d" % (kind, kh, kw, s, self.c))
+        self.m.ops.append(op)
+        self.advance(op)
+        return op
+
+    def eltwise(self, kind, src=None, dst=None, slope=0.0):
+        op = Op(kind, src or self.cur, dst or self.cur, C=self.c, H=self.h, W=self.w, slope=slope,
+                name="%s_%d" % (kind, self.c))
+        self.m.ops.append(op)
+        return op
+
+    def dense(self, no):
+        assert self.h == 1 and self.w == 1
+        nop = layout.pad_channels(no)
+        op = Op("dense", self.cur, self._next(), C=self.c, H=1, W=1, Co=nop, Co_eff=no, weight="w%d" % self.n,
+                name="dense_%d-%d" % (self.c, no))
+        self.n += 1
+        self.m.ops.append(op)
+        self.advance(op)
+        return op
+
+    def done(self):
+        self.m.out = self.cur
+        return self.m
+
+
+def dscnn():
+    """49x10x1 -> Conv 10x4 s2 same (64) + ReLU -> 4 x [DW 3x3 + ReLU, PW 1x1 + ReLU] -> AvgPool 25x5 -> Dense 12."""
+    b = _Builder("dscnn", "f32", (1, 49, 10), "normal")
+    b.advance(b.conv(64, 10, 2, "same", act="relu", kw=4))
+    for _ in range(4):
+        b.dw(3, 1, act="relu")
+        b.advance(b.conv(64, 1, 1, "valid", act="relu"))
+    b.pool("avgpool", 25, 5, 1)
+    b.dense(12)
+    return b.done()
+
+
+def mobilenet_v1():
+    """MobileNetV1 1.0 at 224x224x3: conv 3x3 s2 (32) + 13 depthwise-separable blocks + avgpool 7x7 + dense 1000."""
+    b = _Builder("mobilenet_v1", "f32", (3, 224, 224), "normal")
+    b.advance(b.conv(32, 3, 2, "same", act="relu"))
+    chans = [64, 128, 128, 256, 256, 512, 512, 512, 512, 512, 512, 1024, 1024]
+    strides = {2: 2, 4: 2, 6: 2, 12: 2}
+    for i, co in enumerate(chans, start=1):
+        b.dw(3, strides.get(i, 1), act="relu")
+        b.advance(b.conv(co, 1, 1, "valid", act="relu"))
+    b.pool("avgpool", 7, 7, 1)
+    b.dense(1000)
+    return b.done()
+
+
+def tiny_yolo_v2():
+    """Tiny-YOLOv2 at 416x416x3: 8 x (conv 3x3 + LeakyReLU 0.1) with 2x2 max-pools, then conv 1x1 -> 125."""
+    b = _Builder("tiny_yolo_v2", "f32", (3, 416, 416), "uniform01")
+    chans = [16, 32, 64, 128, 256, 512, 1024, 1024]
+    for i, co in enumerate(chans):
+        b.advance(b.conv(co, 3, 1, "same", act="leaky", slope=0.1))
+        if i < 5:
+            b.pool("maxpool", 2, 2, 2)
+        elif i == 5:
+            b.pool("maxpool", 2, 2, 1, "same")
+    b.advance(b.conv(125, 1, 1, "valid"))
+    return b.done()
+
+
+def resnet8_u8(discriminating=False, seed=7):
+    """ResNet-8 on 32x32x3 uint8: stem conv + ReLU, three residual stages (16/32/64 channels, stages 2
+    and 3 stride 2 with a 1x1 stride-2 projection shortcut), each two conv 3x3 + ReLU with an Accum add;
+    AveragePool 8x8; Dense 64->10.
+
+    Quantisation parameters travel with the buffers (as in the reference's QUInt8Buffer) and are
+    seeded: zero points in [100, 156], multiplier in [2^30, 2^31), right shift in [0, 15].  With
+    those ranges every layer saturates at 255 (added zero points make each of the >= 27 products
+    ~10^4), so a bit-exact match says little.  `discriminating=True` is the same topology with
+    parameters under which the data matters: filters and the image centred (zero point -128),
+    activation buffers with zero point 0, multiplier 2^31-1 and no shift, so that the in-place
+    ReLU and the Accum are value-preserving and each convolution output is 0, 255 or in between
+    according to the sign and size of its accumulator.
+    """
+    b = _Builder("resnet8_u8" + ("_disc" if discriminating else ""), "u8", (3, 32, 32), "u8")
+    b.advance(b.conv(16, 3, 1, "same"))
+    b.eltwise("relu")
+    for stage, co in enumerate((16, 32, 64)):
+        s = 1 if stage == 0 else 2
+        x = b.cur
+        c_in, h_in, w_in = b.c, b.h, b.w
+        # main branch: conv + ReLU, conv
+        o1 = b.conv(co, 3, s, "same", src=x, dst=b._next())
+        b.advance(o1)
+        b.eltwise("relu")
+        main = b.cur
+        if s == 1:
+            short = x
+            o2 = b.conv(co, 3, 1, "same", src=main, dst=b._next(avoid=(short,)))
+        else:
+            # projection shortcut reads the stage input
+            save = (b.c, b.h, b.w)
+            b.c, b.h, b.w = c_in, h_in, w_in
+            osc = b.conv(co, 1, 2, "valid", src=x, dst=b._next(avoid=(main, x)))
+            short = osc.dst
+            b.c, b.h, b.w = save
+            # x is dead now: re-use its buffer for the second conv
+            o2 = b.conv(co, 3, 1, "same", src=main, dst=x)
+        b.advance(o2)
+        b.eltwise("accum", src=short, dst=b.cur)
+        b.eltwise("relu")
+    b.pool("avgpool", 8, 8, 1)
+    b.dense(10)
+    m = b.done()
+    # per-tensor quantisation parameters
+    names = ["in", "b0", "b1", "b2"] + [o.weight for o in m.ops if o.weight]
+    for i, nme in enumerate(names):
+        z = synth.randint(seed * 1000 + 3 * i, 100, 156)
+        mult = synth.randint(seed * 1000 + 3 * i + 1, 1 << 30, (1 << 31) - 1)
+        rs = synth.randint(seed * 1000 + 3 * i + 2, 0, 15)
+        if discriminating:
+            if nme == "in" or nme.startswith("w"):
+                z, mult, rs = -128 + (z % 5) - 2, mult, 0
+            else:
+                z, mult, rs = 0, (1 << 31) - 1, 0
+        m.quant[nme] = (z, mult, 0, rs)
+    return m
+
+
+def layer_sweep():
+    """Single layers at C = 256, 56x56 (each its own one-op model)."""
+    out = []
+    b = _Builder("conv3x3_256", "f32", (256, 56, 56), "normal")
+    b.advance(b.conv(256, 3, 1, "same"))
+    out.append(b.done())
+    b = _Builder("dw3x3_256", "f32", (256, 56, 56), "normal")
+    b.dw(3, 1)
+    out.append(b.done())
+    b = _Builder("maxpool3x3s2_256", "f32", (256, 56, 56), "normal")
+    b.pool("maxpool", 3, 3, 2)
+    out.append(b.done())
+    b = _Builder("relu_256", "f32", (256, 56, 56), "normal")
+    op = b.eltwise("relu", src="in", dst="b0")
+    b.cur = op.dst
+    out.append(b.done())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+def make_weights(model: Model, seed=1234):
+    """name -> packed numpy array (He-normal for float32, uniform bytes for uint8)."""
+    w = {}
+    for i, op in enumerate(model.ops):
+        if not op.weight:
+            continue
+        if op.kind in ("conv", "dense"):
+            co_eff = op.Co_eff or op.Co
+            shape = (co_eff, op.C, op.kh, op.kw)
+            n = int(np.prod(shape))
+            if model.dtype == "f32":
+                flat = synth.he_normal(seed + i, n, op.C * op.kh * op.kw).reshape(shape)
+            else:
+                flat = synth.uniform_u8(seed + i, n).reshape(shape)
+            w[op.weight] = layout.pack_conv_filter(flat)
+        elif op.kind == "dw":
+            shape = (op.C, op.kh, op.kw)
+            n = int(np.prod(shape))
+            if model.dtype == "f32":
+                flat = synth.he_normal(seed + i, n, op.kh * op.kw).reshape(shape)
+            else:
+                flat = synth.uniform_u8(seed + i, n).reshape(shape)
+            w[op.weight] = layout.pack_dw_filter(flat)
+    return w
+
+
+def make_input(model: Model, batch, seed=99):
+    c, h, wd = model.in_shape
+    n = batch * c * h * wd
+    if model.input_kind == "normal":
+        x = synth.normal(seed, n)
+    elif model.input_kind == "uniform01":
+        x = synth.uniform_f32(seed, n, 0.0, 1.0)
+    else:
+        x = synth.uniform_u8(seed, n)
+    return layout.pack_activations(x.reshape(batch, c, h, wd))
+
+
+def buffer_elems(model: Model):
+    """name -> elements per image each named buffer must hold."""
+    need = {"in": int(np.prod(model.in_shape))}
+    for op in model.ops:
+        c, h, w = op.out_shape()
+        need[op.dst] = max(need.get(op.dst, 0), c * h * w)
+    return need
+
+
+class HipExecutor:
+    """Runs a Model on cuda:0 through the C ABI.  torch only owns the memory and the stream."""
+
+    def __init__(self, model: Model, batch: int, weights=None, x=None, fused=True, prepared=True):
+        import torch
+        self.torch = torch
+        self.lib = capi.load()
+        self.model, self.batch, self.fused, self.prepared = model, batch, fused, prepared
+        self.tdtype = torch.float32 if model.dtype == "f32" else torch.uint8
+        weights = weights if weights is not None else make_weights(model)
+        x = x if x is not None else make_input(model, batch)
+        self.w = {k: torch.from_numpy(v).to("cuda") for k, v in weights.items()}
+        self.buf = {k: torch.zeros(batch * n, dtype=self.tdtype, device="cuda")
+                    for k, n in buffer_elems(model).items()}
+        self.buf["in"].copy_(torch.from_numpy(x))
+        self.q = {k: capi.Quant(*v) for k, v in model.quant.items()}
+        self.prep = {}
+        if model.dtype == "u8" and prepared:
+            st = self.stream()
+            for op in model.ops:
+                if op.kind in ("conv", "dense") and op.C % CB == 0:
+                    nb = self.lib.small_hip_conv2d_u8_prepared_filter_bytes(op.kh, op.kw, op.Co, op.C)
+                    t = torch.empty(nb, dtype=torch.uint8, device="cuda")
+                    capi.check(self.lib.small_hip_conv2d_u8_prepare_filter(op.kh, op.kw, op.Co, op.C,
+                                                                           self._p(self.w[op.weight]), self._p(t), st))
+                    self.prep[op.weight] = t
+        torch.cuda.synchronize()
+
+    @staticmethod
+    def _p(t):
+        return C.c_void_p(t.data_ptr())
+
+    def stream(self):
+        return C.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def output(self):
+        op = self.model.ops[-1]
+        c, h, w = op.out_shape()
+        self.torch.cuda.synchronize()
+        return self.buf[self.model.out][: self.batch * c * h * w].cpu().numpy()
+
+    def run_op(self, op: Op, st):
+        L, p, B, b = self.lib, self._p, self.batch, self.buf
+        src, dst = b[op.src], b[op.dst]
+        act = {None: capi.ACT_NONE, "relu": capi.ACT_RELU, "leaky": capi.ACT_LEAKY}[op.act]
+        t_, b_, l_, r_ = op.pads
+        if self.model.dtype == "f32":
+            if op.kind == "conv":
+                args = (B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.Co, op.C, op.H, op.W)
+                if self.fused:
+                    rc = L.small_hip_conv2d_bias_act_f32(*args, p(src), p(self.w[op.weight]), None, act, op.slope, p(dst), st)
+                else:
+                    rc = L.small_hip_conv2d_f32(*args, p(src), p(self.w[op.weight]), p(dst), st)
+                    rc = rc or self._act_f32(op, dst, st)
+            elif op.kind == "dense":
+                rc = L.small_hip_dense_f32(B, op.Co, op.C, p(src), p(self.w[op.weight]), p(dst), st)
+            elif op.kind == "dw":
+                args = (B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.C, op.H, op.W)
+                if self.fused:
+                    rc = L.small_hip_depthwise_conv2d_bias_act_f32(*args, p(src), p(self.w[op.weight]), None, act, op.slope, p(dst), st)
+                else:
+                    rc = L.small_hip_depthwise_conv2d_f32(*args, p(src), p(self.w[op.weight]), p(dst), st)
+                    rc = rc or self._act_f32(op, dst, st)
+            elif op.kind in ("maxpool", "avgpool"):
+                fn = L.small_hip_maxpool2d_f32 if op.kind == "maxpool" else L.small_hip_avgpool2d_f32
+                rc = fn(B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.C, op.H, op.W, p(src), p(dst), st)
+            elif op.kind == "relu":
+                rc = L.small_hip_relu_f32(B, op.C, op.H, op.W, p(src), p(dst), st)
+            elif op.kind == "leaky":
+                rc = L.small_hip_leaky_relu_f32(B, op.C, op.H, op.W, p(src), op.slope, p(dst), st)
+            elif op.kind == "accum":
+                rc = L.small_hip_accum_f32(B, op.C, op.H, op.W, p(src), p(dst), st)
+            else:
+                raise ValueError(op.kind)
+        else:
+            q = self.q
+            iq, oq = C.byref(q[op.src]), C.byref(q[op.dst])
+            if op.kind in ("conv", "dense"):
+                kh, kw, s = (op.kh, op.kw, op.stride) if op.kind == "conv" else (1, 1, 1)
+                args = (B, kh, kw, s, t_, b_, l_, r_, op.Co, op.C, op.H, op.W)
+                fq = C.byref(q[op.weight])
+                if op.weight in self.prep:
+                    rc = L.small_hip_conv2d_u8_prepared(*args, p(src), iq, p(self.prep[op.weight]), fq, p(dst), oq, st)
+                else:
+                    rc = L.small_hip_conv2d_u8(*args, p(src), iq, p(self.w[op.weight]), fq, p(dst), oq, st)
+            elif op.kind == "dw":
+                rc = L.small_hip_depthwise_conv2d_u8(B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.C, op.H, op.W,
+                                                     p(src), iq, p(self.w[op.weight]), C.byref(q[op.weight]), p(dst), oq, st)
+            elif op.kind in ("maxpool", "avgpool"):
+                fn = L.small_hip_maxpool2d_u8 if op.kind == "maxpool" else L.small_hip_avgpool2d_u8
+                rc = fn(B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.C, op.H, op.W, p(src), iq, p(dst), oq, st)
+            elif op.kind == "relu":
+                rc = L.small_hip_relu_u8(B, op.C, op.H, op.W, p(src), iq, p(dst), oq, st)
+            elif op.kind == "accum":
+                rc = L.small_hip_accum_u8(B, op.C, op.H, op.W, p(src), iq, p(dst), oq, st)
+            else:
+                raise ValueError(op.kind)
+        capi.check(rc)
+
+    def _act_f32(self, op, dst, st):
+        c, h, w = op.out_shape()
+        if op.act == "relu":
+            return self.lib.small_hip_relu_f32(self.batch, c, h, w, self._p(dst), self._p(dst), st)
+        if op.act == "leaky":
+            return self.lib.small_hip_leaky_relu_f32(self.batch, c, h, w, self._p(dst), op.slope, self._p(dst), st)
+        return 0
+
+    def forward(self):
+        st = self.stream()
+        for op in self.model.ops:
+            self.run_op(op, st)

@@ -1,0 +1,139 @@
+"""Whole-model parity on the GPU: the five benchmark topologies through the C ABI against the CPU
+oracle on the same seeded inputs and weights (small batch; the oracle is scalar C)."""
+import numpy as np
+import pytest
+
+from smallframework_amd import models
+from oracle.model_exec import OracleExecutor
+from util import assert_close_f32, assert_equal_exact
+
+pytestmark = pytest.mark.gpu
+
+
+def _scale_atol(want):
+    """Whole-model bar: the 1e-5 absolute floor is meant for unit-scale tensors; after a chain of
+    layers it scales with the magnitude of the output (float32 noise of a K~10^4 reduction is
+    relative to the sum of |terms|, not to a result that cancelled to near zero)."""
+    return 1e-5 * max(1.0, float(np.abs(want).max()))
+
+
+def _layerwise(model, batch):
+    """Every op of the model on its real activations: the oracle chain supplies each op's input,
+    the HIP op must reproduce that op's output to the per-layer bar."""
+    import torch
+    w = models.make_weights(model)
+    x = models.make_input(model, batch)
+    orc = OracleExecutor(model, batch, w, x, keep=True)
+    orc.forward()
+    ex = models.HipExecutor(model, batch, w, x, fused=True)
+    st = ex.stream()
+    for op, (src, before, after) in zip(model.ops, orc.trace):
+        if op.src != op.dst:
+            ex.buf[op.src][: src.size].copy_(torch.from_numpy(src))
+        if before is not None:
+            ex.buf[op.dst][: before.size].copy_(torch.from_numpy(before))
+        elif op.src == op.dst:
+            ex.buf[op.dst][: src.size].copy_(torch.from_numpy(src))
+        ex.run_op(op, st)
+        torch.cuda.synchronize()
+        got = ex.buf[op.dst][: after.size].cpu().numpy()
+        what = "%s/%s" % (model.name, op.name)
+        if model.dtype == "u8" or op.kind in ("maxpool", "relu", "leaky", "accum"):
+            assert_equal_exact(got, after, what)
+        elif op.kind in ("conv", "dense", "dw"):
+            # against the reference's float32 sequential order and against the same op accumulated
+            # in float64; the absolute floor follows the magnitude of the layer's outputs (un-normalised
+            # activations reach ~10 in Tiny-YOLO, and float32 rounding noise of a K ~ 10^3..10^4
+            # reduction is relative to the partial sums, not to a result that cancelled to ~0)
+            assert_close_f32(got, after, atol=_scale_atol(after), what=what)
+            assert_close_f32(got, orc.apply(op, src, acc64=1), atol=_scale_atol(after),
+                             what=what + " vs float64 accumulation")
+        else:
+            assert_close_f32(got, after, what=what)
+
+
+def _run(model, batch, fused=True, prepared=True):
+    w = models.make_weights(model)
+    x = models.make_input(model, batch)
+    ex = models.HipExecutor(model, batch, w, x, fused=fused, prepared=prepared)
+    ex.forward()
+    got = ex.output()
+    want = OracleExecutor(model, batch, w, x).forward()
+    return got, want
+
+
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+def test_dscnn(fused):
+    got, want = _run(models.dscnn(), 3, fused)
+    assert_close_f32(got, want, what="dscnn")
+
+
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+def test_mobilenet_v1(fused):
+    got, want = _run(models.mobilenet_v1(), 2, fused)
+    assert np.abs(want).max() > 1e-3
+    assert_close_f32(got, want, what="mobilenet_v1")
+
+
+def test_tiny_yolo_v2():
+    got, want = _run(models.tiny_yolo_v2(), 1)
+    assert np.abs(want).max() > 1e-3
+    assert_close_f32(got, want, atol=_scale_atol(want), what="tiny_yolo_v2")
+
+
+@pytest.mark.parametrize("name,batch", [("dscnn", 2), ("mobilenet_v1", 1), ("tiny_yolo_v2", 1), ("resnet8_u8", 3)])
+def test_layerwise_on_model_activations(name, batch):
+    _layerwise(getattr(models, name)(), batch)
+
+
+def test_tiny_yolo_v2_error_is_reference_sized():
+    """Against a float64-accumulating chain the GPU is no further off than the reference's own
+    float32 arithmetic (the sequential-order oracle): whole-model differences are float32 noise."""
+    m = models.tiny_yolo_v2()
+    w = models.make_weights(m)
+    x = models.make_input(m, 1)
+    ex = models.HipExecutor(m, 1, w, x)
+    ex.forward()
+    gpu = ex.output().astype(np.float64)
+    ref32 = OracleExecutor(m, 1, w, x).forward().astype(np.float64)
+    truth = OracleExecutor(m, 1, w, x, acc64=1).forward().astype(np.float64)
+    e_gpu, e_ref = np.abs(gpu - truth), np.abs(ref32 - truth)
+    print("tiny_yolo_v2 vs float64 chain: gpu max %.3g rms %.3g | float32 oracle max %.3g rms %.3g | out max %.3g"
+          % (e_gpu.max(), np.sqrt((e_gpu ** 2).mean()), e_ref.max(), np.sqrt((e_ref ** 2).mean()), np.abs(truth).max()))
+    assert np.sqrt((e_gpu ** 2).mean()) <= 2.0 * np.sqrt((e_ref ** 2).mean()) + 1e-7
+    assert e_gpu.max() <= 2.0 * e_ref.max() + 1e-6
+
+
+@pytest.mark.parametrize("prepared", [True, False], ids=["prepared", "direct"])
+@pytest.mark.parametrize("disc", [False, True], ids=["config", "discriminating"])
+def test_resnet8_u8(disc, prepared):
+    got, want = _run(models.resnet8_u8(discriminating=disc), 5, prepared=prepared)
+    assert_equal_exact(got, want, "resnet8_u8")
+
+
+def test_resnet8_u8_discriminating_variant_depends_on_the_data():
+    """Bit-exactness on an all-255 tensor proves little: under the discriminating parameters every
+    layer's output must mix low and high values (an accumulator of the wrong sign flips a byte)."""
+    m = models.resnet8_u8(discriminating=True)
+    w = models.make_weights(m)
+    x = models.make_input(m, 2)
+    ex = OracleExecutor(m, 2, w, x, keep=True)
+    ex.forward()
+    assert len(np.unique(ex.trace[0][2])) > 50
+    for op, (_, _, after) in zip(m.ops, ex.trace):
+        if op.kind == "conv":
+            lo, hi = (after == 0).mean(), (after == 255).mean()
+            assert 0.05 < lo < 0.95 and hi < 0.95, (op.name, lo, hi)
+    # and the literal configuration does saturate, which is why the variant exists
+    lit = OracleExecutor(models.resnet8_u8(), 2, models.make_weights(models.resnet8_u8()), x, keep=True)
+    lit.forward()
+    assert (lit.trace[2][2] == 255).mean() > 0.99
+
+
+@pytest.mark.parametrize("m", models.layer_sweep(), ids=lambda m: m.name)
+def test_layer_sweep_batch1(m):
+    got, want = _run(m, 1)
+    if m.name.startswith(("maxpool", "relu")):
+        assert_equal_exact(got, want, m.name)
+    else:
+        assert_close_f32(got, want, what=m.name)
