@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the SMaLL layer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model mobilenet_v1] [--batch 64]
+
+A step is one forward pass of the model over one batch of synthetic images that are already
+resident in HBM.  The headline workload is MobileNetV1 1.0 (224x224x3, float32) at batch 64; the
+line also carries ResNet-8 uint8 at batch 64 and 256, the per-layer roofline table, the roofline
+of the dominant kernel and the reference's CPU build timed on this host.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM = 8.0e12          # B/s, MI355X HBM3E
+PEAK_MFMA_F32 = 157.3e12   # FLOP/s, dense fp32 MFMA
+PEAK_MFMA_I8 = 5.0e15      # OP/s, dense int8 MFMA
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def op_bytes(model, op, batch):
+    """Algorithmic HBM bytes of one op for `batch` images: every tensor once; in-place
+    activations count a read and a write; Accum reads both operands and writes one."""
+    es = model.esize()
+    n_in, n_out = op.act_elems()
+    w = op.weight_elems() * es
+    if op.kind == "accum":
+        return batch * 3 * n_out * es
+    return batch * (n_in + n_out) * es + w
+
+
+def op_bound(model, op, batch):
+    """-> (seconds at the roofline, 'hbm' | 'mfma')."""
+    t_hbm = op_bytes(model, op, batch) / PEAK_HBM
+    peak = PEAK_MFMA_F32 if model.dtype == "f32" else PEAK_MFMA_I8
+    on_mfma = op.kind in ("conv", "dense") and op.C % 16 == 0
+    t_mfma = batch * op.flops() / peak if on_mfma else 0.0
+    return (t_mfma, "mfma") if t_mfma > t_hbm else (t_hbm, "hbm")
+
+
+def time_forward(ex, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        ex.forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ex.forward()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_ops(ex, steps):
+    """Per-op device time (ms) from HIP events on the launch stream, averaged over `steps`."""
+    import torch
+    ops = ex.model.ops
+    tot = [0.0] * len(ops)
+    st = ex.stream()
+    for _ in range(steps):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)]
+        evs[0].record()
+        for i, op in enumerate(ops):
+            ex.run_op(op, st)
+            evs[i + 1].record()
+        torch.cuda.synchronize()
+        for i in range(len(ops)):
+            tot[i] += evs[i].elapsed_time(evs[i + 1])
+    return [t / steps for t in tot]
+
+
+def layer_table(model, batch, ms):
+    rows = []
+    for op, t in zip(model.ops, ms):
+        tb, kind = op_bound(model, op, batch)
+        rows.append({"layer": op.name, "ms": round(t, 5), "bound": kind,
+                     "roofline_frac": round(tb / (t * 1e-3), 4) if t > 0 else None,
+                     "GB/s": round(op_bytes(model, op, batch) / (t * 1e-3) / 1e9, 1) if t > 0 else None,
+                     "TFLOP/s": round(batch * op.flops() / (t * 1e-3) / 1e12, 2) if t > 0 and op.flops() else None})
+    return rows
+
+
+def cpu_reference_mobilenet(model, weights, x_one, budget_s=12.0):
+    """The reference's own ZEN2 build (AVX2 + OpenMP) on this host: images/s, batch-1 calls."""
+    from oracle.binding import have_ref
+    if not have_ref("ZEN2"):
+        return None
+    from oracle.model_exec import RefExecutor
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = min(threads, os.cpu_count() or threads)
+    os.environ["OMP_NUM_THREADS"] = str(threads)
+    ex = RefExecutor(model, weights, x_one, "ZEN2")
+    ex.forward()                     # warm-up (the reference's protocol: 1 warm-up call)
+    t0 = time.perf_counter()
+    n = 0
+    ts = []
+    while n < 64 and (time.perf_counter() - t0) < budget_s:
+        t1 = time.perf_counter()
+        ex.forward()
+        ts.append(time.perf_counter() - t1)
+        n += 1
+    mean = sum(ts) / len(ts)
+    return {"value": round(1.0 / mean, 2), "unit": "images/s", "cores": threads, "kind": "reference",
+            "sample": "%d batch-1 forward passes of %s (all layers, unfused Conv2D+ReLU as the reference's "
+                      "Layer classes issue them) on the reference's ZEN2 build, 1 warm-up; min %.2f ms mean %.2f ms"
+                      % (n, model.name, 1e3 * min(ts), 1e3 * mean)}
+
+
+def cpu_port_u8(model, batch=8):
+    """ResNet-8 uint8 on the scalar C port (1 core): the reference has no uint8 Accum/AveragePool."""
+    from smallframework_amd import models
+    from oracle.model_exec import OracleExecutor
+    w = models.make_weights(model)
+    x = models.make_input(model, batch)
+    ex = OracleExecutor(model, batch, w, x)
+    ex.forward()
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        OracleExecutor(model, batch, w, x).forward()
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(batch / dt, 1), "unit": "images/s", "cores": 1, "kind": "port",
+            "sample": "%d images x %d passes of %s on the scalar C restatement" % (batch, reps, model.name)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--model", default="mobilenet_v1",
+                    choices=["mobilenet_v1", "resnet8_u8", "tiny_yolo_v2", "dscnn"])
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="headline model only")
+    ap.add_argument("--unfused", action="store_true", help="issue Conv2D and the activation as separate calls")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build measures one GPU; the path shards by image with no collective, "
+            "so --gpus N > 1 is not run here.")
+        sys.exit(2)
+
+    import torch
+    from smallframework_amd import capi, models
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        sys.exit(1)
+    capi.load()
+    default_batch = {"mobilenet_v1": 64, "resnet8_u8": 64, "tiny_yolo_v2": 16, "dscnn": 64}
+    batch = args.batch or default_batch[args.model]
+    model = getattr(models, args.model)()
+    log("building %s batch %d ..." % (model.name, batch))
+    weights = models.make_weights(model)
+    x = models.make_input(model, batch)
+    ex = models.HipExecutor(model, batch, weights, x, fused=not args.unfused)
+
+    sec = time_forward(ex, args.steps, args.warmup)
+    ips = batch / sec
+    log("%s: %.3f ms/step, %.1f images/s" % (model.name, sec * 1e3, ips))
+
+    # per-op device times (HIP events on the launch stream) over the same number of steps
+    ms = time_ops(ex, args.steps)
+    table = layer_table(model, batch, ms)
+    for r in table:
+        log("  %-28s %9.4f ms  %-4s %6.1f%%" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0)))
+
+    # dominant kernel = the one with the largest summed time
+    def kernel_of(op):
+        if op.kind in ("conv", "dense"):
+            if op.C % 16 != 0:
+                return "conv_smallci_%s_kernel" % model.dtype
+            return "conv_mfma_%s_kernel" % model.dtype
+        return {"dw": "dw_%s_kernel" % model.dtype, "maxpool": "pool_%s_kernel" % model.dtype,
+                "avgpool": "pool_%s_kernel" % model.dtype}.get(op.kind, "ew_%s_kernel" % model.dtype)
+
+    per_kernel = {}
+    for op, t in zip(model.ops, ms):
+        k = kernel_of(op)
+        d = per_kernel.setdefault(k, {"ms": 0.0, "launches": 0, "flops": 0.0, "bytes": 0.0})
+        d["ms"] += t
+        d["launches"] += 1
+        d["flops"] += batch * op.flops()
+        d["bytes"] += op_bytes(model, op, batch)
+    dom = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    d = per_kernel[dom]
+    if "mfma" in dom:
+        peak = (PEAK_MFMA_F32 if model.dtype == "f32" else PEAK_MFMA_I8) / 1e12
+        ach = d["flops"] / (d["ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 2), "peak": round(peak, 1), "unit": "TFLOP/s",
+                "frac": round(ach / peak, 4), "traffic": None}
+    else:
+        ach = d["bytes"] / (d["ms"] * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s",
+                "frac": round(ach / 8000.0, 4), "traffic": None}
+    roof.update({"kernel": dom, "launches_per_step": d["launches"],
+                 "avg_launch_ms": round(d["ms"] / d["launches"], 5),
+                 "algorithmic_per_launch": {"GFLOP": round(d["flops"] / d["launches"] / 1e9, 3),
+                                            "MB": round(d["bytes"] / d["launches"] / 1e6, 3)}})
+
+    extras = {"per_kernel_ms": {k: round(v["ms"], 4) for k, v in per_kernel.items()},
+              "sum_of_layer_ms": round(sum(ms), 4)}
+    if not args.no_extras and args.model == "mobilenet_v1":
+        for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
+            m2 = getattr(models, name)()
+            e2 = models.HipExecutor(m2, b)
+            s2 = time_forward(e2, max(args.steps, 50), args.warmup)
+            ms2 = time_ops(e2, 10)
+            extras["%s_b%d" % (name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
+                                            "layers": layer_table(m2, b, ms2)}
+            log("%s batch %d: %.4f ms/step, %.0f images/s" % (name, b, s2 * 1e3, b / s2))
+            del e2
+        torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu:
+        try:
+            if model.dtype == "f32":
+                x1 = models.make_input(model, 1)
+                cpu = cpu_reference_mobilenet(model, weights, x1)
+            if cpu is None:
+                cpu = cpu_port_u8(model) if model.dtype == "u8" else None
+            if not args.no_extras and args.model == "mobilenet_v1":
+                extras["resnet8_u8_cpu"] = cpu_port_u8(models.resnet8_u8())
+        except Exception as e:            # the baseline leg must not take the GPU numbers down
+            log("cpu baseline failed: %r" % (e,))
+
+    out = {
+        "metric": "images/s @batch%d %s %s" % (batch, model.name, "fp32" if model.dtype == "f32" else "u8"),
+        "value": round(ips, 2), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if model.dtype == "f32" else "u8", "data": "synthetic",
+        "config": {"workload": "%s forward, batch %d, %dx%dx%d input, %s" % (
+            model.name, batch, model.in_shape[1], model.in_shape[2], model.in_shape[0],
+            "Conv2D+bias+activation fused" if not args.unfused else "unfused layer calls"),
+            "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4)},
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "layers": table,
+        "extras": extras,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
