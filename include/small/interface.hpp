@@ -1,0 +1,481 @@
+// The `small::` layer functions on the MI355X library.
+//
+// Same names, argument order and error behaviour as the reference's public API
+// (include/small/interface.hpp:49-497, definitions in include/small/interface_abstract.hpp):
+// buffers by reference, pads as uint8_t in the order top, bottom, left, right, and
+// std::invalid_argument with the reference's messages for unsupported strides / channel counts.
+// Each function forwards to one entry point of the C ABI (include/small_hip.h).
+//
+// Additions (no counterpart in the reference):
+//   - every layer also exists with a leading `int batch` argument in namespace small::batched;
+//     image n of a batched call equals the batch-1 call on image n
+//   - Conv2D_Bias_Act / DepthwiseConv2D_Bias_Act: bias + convolution + activation in one pass
+//     (the reference's Layer classes issue Bias, PartialConv2D and the activation separately)
+//   - Accum and AveragePool2D for QUInt8Buffer (the reference leaves them unimplemented)
+// Divergence: small::Dense computes y = W x (what every reference model means by a dense layer
+// and spells as Conv2D on a 1x1 image); the reference's own small::Dense body is a per-channel
+// scale with no callers and is available as small::DenseAsWritten.
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+
+#include "../small_hip.h"
+#include "Buffer.hpp"
+
+namespace small
+{
+
+enum ActivationType
+{
+    NONE = SMALL_HIP_ACT_NONE,
+    RELU = SMALL_HIP_ACT_RELU,
+    LEAKY = SMALL_HIP_ACT_LEAKY
+};
+
+namespace detail
+{
+template <class BufferT>
+struct type_tag
+{
+    static const char *name() { return std::is_same<BufferT, FloatBuffer>::value ? "float" : "quint8"; }
+};
+
+// status -> the exception the reference throws from the same place
+template <class BufferT>
+inline void raise(int status, const char *op)
+{
+    if (status == SMALL_HIP_OK) return;
+    const std::string head = std::string(op) + "<" + type_tag<BufferT>::name() + "> ERROR: ";
+    switch (status)
+    {
+    case SMALL_HIP_ESTRIDE: throw std::invalid_argument(head + "stride unsupported.");
+    case SMALL_HIP_ECHANNELS: throw std::invalid_argument(head + "in_channels unsupported.");
+    case SMALL_HIP_ESCALE: throw std::invalid_argument(head + "scale factor unsupported (only 1 or 2).");
+    case SMALL_HIP_ENOMEM: throw std::bad_alloc();
+    case SMALL_HIP_EINVAL: throw std::invalid_argument(head + small_hip_last_error());
+    default: throw std::runtime_error(head + small_hip_last_error());
+    }
+}
+
+template <class BufferT>
+using if_float = std::enable_if_t<std::is_same<FloatBuffer, BufferT>::value, bool>;
+template <class BufferT>
+using if_quint8 = std::enable_if_t<std::is_same<QUInt8Buffer, BufferT>::value, bool>;
+
+inline small_hip_stream_t st() { return current_stream(); }
+} // namespace detail
+
+// =================================================================================================
+namespace batched
+{
+
+// ---- Conv2D / PartialConv2D ------------------------------------------------------------------------
+template <class BufferT, detail::if_float<BufferT> = true>
+void Conv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+            uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels, int input_height,
+            int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_conv2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                r_pad, output_channels, input_channels, input_height,
+                                                input_width, input_buf.device_in(), filter_buf.device_in(),
+                                                output_buf.device_out(), detail::st()),
+                           "Conv2D");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void Conv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+            uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels, int input_height,
+            int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), fq = filter_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_conv2d_u8(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                               r_pad, output_channels, input_channels, input_height, input_width,
+                                               input_buf.device_in(), &iq, filter_buf.device_in(), &fq,
+                                               output_buf.device_out(), &oq, detail::st()),
+                           "Conv2D");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialConv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                   uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels, int input_height,
+                   int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_partial_conv2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad,
+                                                        l_pad, r_pad, output_channels, input_channels,
+                                                        input_height, input_width, input_buf.device_in(),
+                                                        filter_buf.device_in(), output_buf.device_out(),
+                                                        detail::st()),
+                           "PartialConv2D");
+}
+
+// bias_buf may be empty (size 0): no bias
+template <class BufferT, detail::if_float<BufferT> = true>
+void Conv2D_Bias_Act(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                     uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels, int input_height,
+                     int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                     BufferT const &bias_buf, ActivationType act, float negative_slope, BufferT &output_buf)
+{
+    detail::raise<BufferT>(
+        small_hip_conv2d_bias_act_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad,
+                                      output_channels, input_channels, input_height, input_width,
+                                      input_buf.device_in(), filter_buf.device_in(),
+                                      bias_buf.size() ? bias_buf.device_in() : nullptr, (int)act, negative_slope,
+                                      output_buf.device_out(), detail::st()),
+        "Conv2D_Bias_Act");
+}
+
+// ---- DepthwiseConv2D / PartialDepthwiseConv2D ------------------------------------------------------
+template <class BufferT, detail::if_float<BufferT> = true>
+void DepthwiseConv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                     uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                     BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_depthwise_conv2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad,
+                                                          l_pad, r_pad, input_channels, input_height, input_width,
+                                                          input_buf.device_in(), filter_buf.device_in(),
+                                                          output_buf.device_out(), detail::st()),
+                           "DepthwiseConv2D");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void DepthwiseConv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                     uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                     BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), fq = filter_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_depthwise_conv2d_u8(batch, kernel_height, kernel_width, stride, t_pad, b_pad,
+                                                         l_pad, r_pad, input_channels, input_height, input_width,
+                                                         input_buf.device_in(), &iq, filter_buf.device_in(), &fq,
+                                                         output_buf.device_out(), &oq, detail::st()),
+                           "DepthwiseConv2D");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialDepthwiseConv2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad,
+                            uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height,
+                            int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                            BufferT &output_buf)
+{
+    detail::raise<BufferT>(
+        small_hip_partial_depthwise_conv2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                               r_pad, input_channels, input_height, input_width,
+                                               input_buf.device_in(), filter_buf.device_in(),
+                                               output_buf.device_out(), detail::st()),
+        "PartialDepthwiseConv2D");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void DepthwiseConv2D_Bias_Act(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad,
+                              uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height,
+                              int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                              BufferT const &bias_buf, ActivationType act, float negative_slope,
+                              BufferT &output_buf)
+{
+    detail::raise<BufferT>(
+        small_hip_depthwise_conv2d_bias_act_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                r_pad, input_channels, input_height, input_width,
+                                                input_buf.device_in(), filter_buf.device_in(),
+                                                bias_buf.size() ? bias_buf.device_in() : nullptr, (int)act,
+                                                negative_slope, output_buf.device_out(), detail::st()),
+        "DepthwiseConv2D_Bias_Act");
+}
+
+// ---- pooling -----------------------------------------------------------------------------------------
+template <class BufferT, detail::if_float<BufferT> = true>
+void MaxPool2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+               uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+               BufferT const &input_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_maxpool2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                   r_pad, input_channels, input_height, input_width,
+                                                   input_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "MaxPool2D");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void MaxPool2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+               uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+               BufferT const &input_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_maxpool2d_u8(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                  r_pad, input_channels, input_height, input_width,
+                                                  input_buf.device_in(), &iq, output_buf.device_out(), &oq,
+                                                  detail::st()),
+                           "MaxPool2D");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void AveragePool2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                   uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                   BufferT const &input_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_avgpool2d_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                   r_pad, input_channels, input_height, input_width,
+                                                   input_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "AveragePool2D");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void AveragePool2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                   uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                   BufferT const &input_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_avgpool2d_u8(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                  r_pad, input_channels, input_height, input_width,
+                                                  input_buf.device_in(), &iq, output_buf.device_out(), &oq,
+                                                  detail::st()),
+                           "AveragePool2D");
+}
+
+// ---- activations, accumulation, bias ------------------------------------------------------------------
+template <class BufferT, detail::if_float<BufferT> = true>
+void ReLUActivation(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+                    BufferT &output_buf)
+{
+    float const *in = input_buf.device_in();
+    detail::raise<BufferT>(small_hip_relu_f32(batch, input_channels, input_height, input_width, in,
+                                              output_buf.device_out(), detail::st()),
+                           "ReLUActivation");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void ReLUActivation(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+                    BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), oq = output_buf.quant();
+    uint8_t const *in = input_buf.device_in();
+    detail::raise<BufferT>(small_hip_relu_u8(batch, input_channels, input_height, input_width, in, &iq,
+                                             output_buf.device_out(), &oq, detail::st()),
+                           "ReLUActivation");
+}
+
+// the slope arrives as a one-element buffer, as in the reference's definition
+// (interface_abstract.hpp:1616-1621)
+template <class BufferT, detail::if_float<BufferT> = true>
+void LeakyReLUActivation(int batch, int input_channels, int input_height, int input_width,
+                         BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    const float slope = filter_buf.data()[0];
+    float const *in = input_buf.device_in();
+    detail::raise<BufferT>(small_hip_leaky_relu_f32(batch, input_channels, input_height, input_width, in, slope,
+                                                    output_buf.device_out(), detail::st()),
+                           "LeakyReLUActivation");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void Accum(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+           BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_accum_f32(batch, input_channels, input_height, input_width,
+                                               input_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "Accum");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void Accum(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+           BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_accum_u8(batch, input_channels, input_height, input_width,
+                                              input_buf.device_in(), &iq, output_buf.device_out(), &oq,
+                                              detail::st()),
+                           "Accum");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void Bias(int batch, int num_channels, int output_height, int output_width, BufferT const &input_buf,
+          BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_bias_f32(batch, num_channels, output_height, output_width,
+                                              input_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "Bias");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialBias(int batch, int num_channels, int output_height, int output_width, BufferT const &input_buf,
+                 BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_partial_bias_f32(batch, num_channels, output_height, output_width,
+                                                      input_buf.device_in(), output_buf.device_out(),
+                                                      detail::st()),
+                           "PartialBias");
+}
+
+// ---- UpSample2D, Concat, Dense ----------------------------------------------------------------------------
+template <class BufferT, detail::if_float<BufferT> = true>
+void UpSample2D(int batch, int scale_factor, int input_channels, int input_height, int input_width,
+                BufferT const &input_buf, BufferT &output_buf)
+{
+    if (scale_factor == 1)
+    {
+        output_buf = input_buf;   // the reference copy-assigns the buffer (interface_abstract.hpp:1858-1861)
+        return;
+    }
+    const int status = small_hip_upsample2d_f32(batch, scale_factor, input_channels, input_height, input_width,
+                                                input_buf.device_in(), output_buf.device_out(), detail::st());
+    detail::raise<BufferT>(status, "Upsample");
+}
+
+template <class BufferT>
+void Concat(int batch, uint32_t input0_channels, uint32_t input1_channels, uint32_t input_height,
+            uint32_t input_width, BufferT const &input0_buf, BufferT const &input1_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_concat(batch, input0_channels, input1_channels, input_height, input_width,
+                                            input0_buf.device_in(), input1_buf.device_in(),
+                                            output_buf.device_out(), sizeof(typename BufferT::value_type),
+                                            detail::st()),
+                           "Concat");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void Dense(int batch, int output_elements, int input_elements, BufferT const &input_buf,
+           BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_dense_f32(batch, output_elements, input_elements, input_buf.device_in(),
+                                               filter_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "Dense");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void Dense(int batch, int output_elements, int input_elements, BufferT const &input_buf,
+           BufferT const &filter_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), fq = filter_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_dense_u8(batch, output_elements, input_elements, input_buf.device_in(), &iq,
+                                              filter_buf.device_in(), &fq, output_buf.device_out(), &oq,
+                                              detail::st()),
+                           "Dense");
+}
+
+} // namespace batched
+
+// =================================================================================================
+// The reference's batch-1 signatures (interface.hpp:49-497)
+// =================================================================================================
+template <class BufferT>
+void Conv2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+            uint8_t r_pad, int output_channels, int input_channels, int input_height, int input_width,
+            BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::Conv2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, output_channels,
+                    input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialConv2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+                   uint8_t r_pad, int output_channels, int input_channels, int input_height, int input_width,
+                   BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::PartialConv2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, output_channels,
+                           input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void DepthwiseConv2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                     uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                     BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::DepthwiseConv2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, input_channels,
+                             input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialDepthwiseConv2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                            uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                            BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::PartialDepthwiseConv2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad,
+                                    input_channels, input_height, input_width, input_buf, filter_buf,
+                                    output_buf);
+}
+
+template <class BufferT>
+void MaxPool2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+               uint8_t r_pad, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+               BufferT &output_buf)
+{
+    batched::MaxPool2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, input_channels,
+                       input_height, input_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void AveragePool2D(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+                   uint8_t r_pad, int input_channels, int input_height, int input_width,
+                   BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::AveragePool2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, input_channels,
+                           input_height, input_width, input_buf, output_buf);
+}
+
+template <typename BufferT>
+void UpSample2D(int scale_factor, int input_channels, int input_height, int input_width,
+                BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::UpSample2D(1, scale_factor, input_channels, input_height, input_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void ReLUActivation(int input_channels, int input_height, int input_width, BufferT const &input_buf,
+                    BufferT &output_buf)
+{
+    batched::ReLUActivation(1, input_channels, input_height, input_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void LeakyReLUActivation(int input_channels, int input_height, int input_width, BufferT const &input_buf,
+                         BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::LeakyReLUActivation(1, input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void Accum(int input_channels, int input_height, int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::Accum(1, input_channels, input_height, input_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void Bias(int num_channels, int output_height, int output_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::Bias(1, num_channels, output_height, output_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialBias(int num_channels, int output_height, int output_width, BufferT const &input_buf,
+                 BufferT &output_buf)
+{
+    batched::PartialBias(1, num_channels, output_height, output_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void Concat(uint32_t input0_channels, uint32_t input1_channels, uint32_t input_height, uint32_t input_width,
+            BufferT const &input0_buf, BufferT const &input1_buf, BufferT &output_buf)
+{
+    batched::Concat(1, input0_channels, input1_channels, input_height, input_width, input0_buf, input1_buf,
+                    output_buf);
+}
+
+template <class BufferT>
+void Dense(int output_elements, int input_elements, BufferT const &input_buf, BufferT const &filter_buf,
+           BufferT &output_buf)
+{
+    batched::Dense(1, output_elements, input_elements, input_buf, filter_buf, output_buf);
+}
+
+// small::Dense exactly as the reference writes it (interface_abstract.hpp:2113-2132):
+// output[o * Ni + i] = input[o * Ni + i] * filter[o]
+template <class BufferT, detail::if_float<BufferT> = true>
+void DenseAsWritten(int output_elements, int input_elements, BufferT const &input_buf,
+                    BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_dense_literal_f32(output_elements, input_elements, input_buf.device_in(),
+                                                       filter_buf.device_in(), output_buf.device_out(),
+                                                       detail::st()),
+                           "Dense");
+}
+
+} // namespace small
