@@ -32,6 +32,8 @@
 // (PartialConv2D), optional bias, optional ReLU / LeakyReLU.
 #include "common.h"
 
+#include <cstdlib>
+
 using namespace shp;
 
 namespace
@@ -62,6 +64,47 @@ __device__ __forceinline__ float act1(float v, int act, float slope)
     if (act == SMALL_HIP_ACT_RELU) return v > 0.f ? v : 0.f;
     if (act == SMALL_HIP_ACT_LEAKY) return v > 0.f ? v : v * slope;
     return v;
+}
+
+// accumulate / bias / activation in registers, then 16-byte stores: a lane holds channels
+// 8q + 4*half + {0..3} of its pixel in accumulator registers 4q .. 4q+3
+template <int COT, int PXT>
+__device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
+                                              int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+{
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+    {
+        const int co_tile = (cg * COT + c) * 32;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            if (!pvalid[t]) continue;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int co4 = co_tile + 8 * q + 4 * half;
+                if (co4 >= a.Co) continue;
+                float4 v = make_float4(acc[c][t][4 * q + 0], acc[c][t][4 * q + 1],
+                                       acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
+                float4 *o = reinterpret_cast<float4 *>(a.out + out_pix[t] +
+                                                       (size_t)(co4 / CB) * HoWo * CB + (co4 % CB));
+                if (a.accumulate)
+                {
+                    const float4 old = *o;
+                    v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+                }
+                if (a.bias)
+                {
+                    const float4 bb = *reinterpret_cast<const float4 *>(a.bias + co4);
+                    v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+                }
+                v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
+                v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
+                *o = v;
+            }
+        }
+    }
 }
 
 template <int COT, int PXT>
@@ -126,8 +169,11 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
             for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
 
     // ---- K loop state: tap (ta, tb) outer, input channel block inner ---------------------
+    // The loop below is branch-free: it always runs an even number of steps and a step past the
+    // end (`live` false) loads from valid addresses and contributes zeros through the B operand.
     int ta = 0, tb = 0, cib = 0;
     const int nsteps = taps * CiB;
+    bool live = true;
 
     auto load_step = [&](float (&A)[COT][8], float4 (&B)[PXT][2]) {
         const int tap = ta * a.kw + tb;
@@ -135,7 +181,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
         for (int t = 0; t < PXT; ++t)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
-            const bool ok = pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
             const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
             const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
             float4 v0 = p[0], v1 = p[1];
@@ -150,12 +196,15 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) A[c][kk] = w[kk * CB];
         }
-        // advance
-        if (++cib == CiB)
+        // advance; the state parks on the last step once the end is reached
+        int ncib = cib + 1, ntb = tb, nta = ta;
+        if (ncib == CiB)
         {
-            cib = 0;
-            if (++tb == a.kw) { tb = 0; ++ta; }
+            ncib = 0;
+            if (++ntb == a.kw) { ntb = 0; ++nta; }
         }
+        if (nta < a.kh) { cib = ncib; tb = ntb; ta = nta; }
+        else live = false;
     };
 
     auto compute_step = [&](const float (&A)[COT][8], const float4 (&B)[PXT][2]) {
@@ -174,55 +223,185 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
         }
     };
 
+    // register double buffer: the loads of step s+1 are in flight while step s is multiplied
     float A0[COT][8], A1[COT][8];
     float4 B0[PXT][2], B1[PXT][2];
     load_step(A0, B0);
-    for (int s = 0; s < nsteps; s += 2)
+    const int npairs = (nsteps + 1) >> 1;
+    for (int it = 0; it < npairs; ++it)
     {
-        if (s + 1 < nsteps) load_step(A1, B1);
+        load_step(A1, B1);
         compute_step(A0, B0);
-        if (s + 1 < nsteps)
-        {
-            if (s + 2 < nsteps) load_step(A0, B0);
-            compute_step(A1, B1);
-        }
+        load_step(A0, B0);
+        compute_step(A1, B1);
     }
 
-    // ---- epilogue --------------------------------------------------------------------------
+    conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    (void)co_of;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Same contraction with the filter operand staged through LDS.  The four waves of a workgroup
+// multiply the same output-channel group, so the step's [16 ci][16 co] filter tiles (COT*2 KiB)
+// are fetched once per workgroup with fully coalesced 16-byte loads, written to LDS (double
+// buffered, one barrier per K-step) and read back by every wave in MFMA operand order.  This cuts
+// the vector-cache accesses of the filter by 4x and replaces 8 strided dword loads per tile by
+// one 16-byte load per lane.  The activation operand still goes straight from global memory to
+// the MFMA register, two 16-byte loads per lane and tile.
+constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks start 16 banks apart
+
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a)
+{
+    __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
+
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
+    const int cg = lid % a.n_co_groups;
+    const int pxb = lid / a.n_co_groups;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int HoWo = a.Ho * a.Wo;
+    const int CiB = a.Ci / CB;
+    const int CoB = a.Co / CB;
+    const int taps = a.kh * a.kw;
+    const size_t in_blk = (size_t)a.H * a.W * CB;
+
+    const float *in_img[PXT];
+    int ih0[PXT], iw0[PXT];
+    bool pvalid[PXT];
+    size_t out_pix[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo;
+        const int rem = pc - n * HoWo;
+        const int oh = rem / a.Wo;
+        const int ow = rem - oh * a.Wo;
+        ih0[t] = oh * a.stride - a.pt;
+        iw0[t] = ow * a.stride - a.pl;
+        in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+    }
+
+    // ---- cooperative filter fetch: COT*2 tiles of 64 float4 each -----------------------------
+    constexpr int A_VECS = COT * 2 * 64;                 // float4 per step and workgroup
+    constexpr int A_PER_THREAD = (A_VECS + 255) / 256;   // 1 for COT <= 2, 2 for COT == 4
+    const float *a_src[A_PER_THREAD];
+    int a_dst[A_PER_THREAD];
+    bool a_on[A_PER_THREAD];
+#pragma unroll
+    for (int j = 0; j < A_PER_THREAD; ++j)
+    {
+        const int v = tid + j * 256;
+        a_on[j] = v < A_VECS;
+        const int vc = a_on[j] ? v : 0;
+        const int blk = vc >> 6, within = vc & 63;
+        int cob = cg * COT * 2 + blk;
+        cob = cob < CoB ? cob : CoB - 1;                  // rows past Co: garbage, never stored
+        a_src[j] = a.filt + (size_t)cob * CiB * taps * (CB * CB) + within * 4;
+        a_dst[j] = blk * A_TILE_FLOATS + within * 4;
+    }
+    // read position of this lane inside a staged tile pair
+    int a_rd[COT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c) a_rd[c] = (c * 2 + (col >> 4)) * A_TILE_FLOATS + half * 8 * CB + (col & 15);
+
+    floatx16 acc[COT][PXT];
 #pragma unroll
     for (int c = 0; c < COT; ++c)
-    {
-        const int co_tile = (cg * COT + c) * 32;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
+
+    int ta = 0, tb = 0, cib = 0;
+    const int nsteps = taps * CiB;
+    bool live = true;
+
+    // issues the global loads of the step at (ta, tb, cib) and advances the position
+    auto fetch = [&](float4 (&Areg)[A_PER_THREAD], float4 (&B)[PXT][2]) {
+        const int tap = ta * a.kw + tb;
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
-            if (!pvalid[t]) continue;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                const int co4 = co_tile + 8 * q + 4 * half;     // rows 8q + 4*half + {0..3}
-                if (co4 >= a.Co) continue;
-                float4 v = make_float4(acc[c][t][4 * q + 0], acc[c][t][4 * q + 1],
-                                       acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
-                float4 *o = reinterpret_cast<float4 *>(a.out + out_pix[t] +
-                                                       (size_t)(co4 / CB) * HoWo * CB + (co4 % CB));
-                if (a.accumulate)
-                {
-                    const float4 old = *o;
-                    v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
-                }
-                if (a.bias)
-                {
-                    const float4 bb = *reinterpret_cast<const float4 *>(a.bias + co4);
-                    v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
-                }
-                v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
-                v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
-                *o = v;
-            }
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
+            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
+            float4 v0 = p[0], v1 = p[1];
+            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
+            B[t][0] = v0;
+            B[t][1] = v1;
         }
+        const size_t woff = ((size_t)cib * taps + tap) * (CB * CB);
+#pragma unroll
+        for (int j = 0; j < A_PER_THREAD; ++j)
+            if (a_on[j]) Areg[j] = *reinterpret_cast<const float4 *>(a_src[j] + woff);
+        int ncib = cib + 1, ntb = tb, nta = ta;
+        if (ncib == CiB)
+        {
+            ncib = 0;
+            if (++ntb == a.kw) { ntb = 0; ++nta; }
+        }
+        if (nta < a.kh) { cib = ncib; tb = ntb; ta = nta; }
+        else live = false;
+    };
+    auto stage = [&](int buf, const float4 (&Areg)[A_PER_THREAD]) {
+#pragma unroll
+        for (int j = 0; j < A_PER_THREAD; ++j)
+            if (a_on[j]) *reinterpret_cast<float4 *>(&lds_a[buf][a_dst[j]]) = Areg[j];
+    };
+    auto multiply = [&](int buf, const float4 (&B)[PXT][2]) {
+        float A[COT][8];
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) A[c][kk] = lds_a[buf][a_rd[c] + kk * CB];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                const float4 bv = B[t][kk >> 2];
+                const float b = (kk & 3) == 0 ? bv.x : (kk & 3) == 1 ? bv.y : (kk & 3) == 2 ? bv.z : bv.w;
+#pragma unroll
+                for (int c = 0; c < COT; ++c)
+                    acc[c][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[c][kk], b, acc[c][t], 0, 0, 0);
+            }
+    };
+
+    // Schedule per step s:  multiply(s) | stage filter(s+1) into the other LDS buffer | fetch(s+2)
+    // | barrier.  The loads of a step are issued a whole step before they are consumed.
+    float4 Areg[A_PER_THREAD];
+    float4 B0[PXT][2], B1[PXT][2];
+    fetch(Areg, B0);                 // step 0
+    stage(0, Areg);
+    fetch(Areg, B1);                 // step 1
+    __syncthreads();
+    const int npairs = (nsteps + 1) >> 1;
+    for (int it = 0; it < npairs; ++it)
+    {
+        multiply(0, B0);             // step 2*it
+        stage(1, Areg);              // filter of step 2*it + 1
+        fetch(Areg, B0);             // step 2*it + 2
+        __syncthreads();
+        multiply(1, B1);             // step 2*it + 1
+        stage(0, Areg);              // filter of step 2*it + 2
+        fetch(Areg, B1);             // step 2*it + 3
+        __syncthreads();
     }
-    (void)co_of;
+
+    conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -300,7 +479,12 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    hipLaunchKernelGGL((conv_mfma_f32_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    // SMALL_HIP_CONV_LDS=0 selects the variant that reads the filter operand straight from global memory
+    static const bool use_lds = [] { const char *e = std::getenv("SMALL_HIP_CONV_LDS"); return !(e && e[0] == '0'); }();
+    if (use_lds)
+        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL((conv_mfma_f32_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
 }
 
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
@@ -344,13 +528,28 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
         return SMALL_HIP_OK;
     }
 
-    // tile choice: the largest wave tile that still gives the chip ~2 waves per SIMD
-    const long target_waves = 2L * NUM_CU * 4;
-    auto waves = [&](int cot, int pxt) {
-        return (long)((Co + 32 * cot - 1) / (32 * cot)) * ((P + 32 * pxt - 1) / (32 * pxt));
-    };
-    if (Co % 64 == 0 && waves(2, 2) >= target_waves) launch_mfma<2, 2>(a, s);
-    else if (waves(1, 2) >= target_waves) launch_mfma<1, 2>(a, s);
+    // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X: 2x2 wins only when the
+    // launch has many tiles per SIMD and a long reduction, 2x1 in the middle, 1x1 when the output is
+    // small (few tiles per SIMD: balance matters more than operand re-use).
+    const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32);
+    const long simds = 4L * NUM_CU;
+    const int nsteps = kh * kw * (Ci / CB);
+    int cot = 1, pxt = 1;
+    if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
+    else if (Co % 64 == 0 && tiles32 >= 6 * simds) { cot = 2; pxt = 1; }
+    // tuning knob: SMALL_HIP_CONV_TILE="<cot>,<pxt>" forces a wave tile (32-channel x 32-pixel units)
+    if (const char *e = std::getenv("SMALL_HIP_CONV_TILE"))
+    {
+        int c2 = 0, p2 = 0;
+        if (std::sscanf(e, "%d,%d", &c2, &p2) == 2) { cot = c2; pxt = p2; }
+    }
+    if (cot == 2 && pxt == 2) launch_mfma<2, 2>(a, s);
+    else if (cot == 1 && pxt == 2) launch_mfma<1, 2>(a, s);
+    else if (cot == 2 && pxt == 1) launch_mfma<2, 1>(a, s);
+    else if (cot == 4 && pxt == 1) launch_mfma<4, 1>(a, s);
+    else if (cot == 4 && pxt == 2) launch_mfma<4, 2>(a, s);
+    else if (cot == 2 && pxt == 4) launch_mfma<2, 4>(a, s);
+    else if (cot == 1 && pxt == 4) launch_mfma<1, 4>(a, s);
     else launch_mfma<1, 1>(a, s);
     SHP_LAUNCH_CHECK(op);
     return SMALL_HIP_OK;
