@@ -405,6 +405,164 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a
 }
 
 // ---------------------------------------------------------------------------------------------
+// Small outputs (few 32x32 tiles per SIMD: fully connected layers, 7x7 / 13x13 feature maps,
+// batch 1): the four waves of a workgroup take the SAME output tile and one quarter of the K-steps
+// each, then waves 1..3 hand their partial accumulators to wave 0 through LDS, which adds them in
+// the fixed order 0+1+2+3 (deterministic) and runs the epilogue.  Operands go straight from global
+// memory to the MFMA registers (nothing is shared between the waves until the reduction).
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a)
+{
+    __shared__ float red[3][COT * PXT][16][64];
+
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;
+    const int cg = lid % a.n_co_groups;
+    const int pxb = lid / a.n_co_groups;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int HoWo = a.Ho * a.Wo;
+    const int CiB = a.Ci / CB;
+    const int CoB = a.Co / CB;
+    const int taps = a.kh * a.kw;
+    const size_t in_blk = (size_t)a.H * a.W * CB;
+
+    const float *in_img[PXT];
+    int ih0[PXT], iw0[PXT];
+    bool pvalid[PXT];
+    size_t out_pix[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = (pxb * PXT + t) * 32 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo;
+        const int rem = pc - n * HoWo;
+        const int oh = rem / a.Wo;
+        const int ow = rem - oh * a.Wo;
+        ih0[t] = oh * a.stride - a.pt;
+        iw0[t] = ow * a.stride - a.pl;
+        in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+    }
+    const float *w_row[COT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+    {
+        const int co = (cg * COT + c) * 32 + col;
+        const int cc = co < a.Co ? co : a.Co - 1;
+        w_row[c] = a.filt + (size_t)(cc / CB) * CiB * taps * (CB * CB) + (cc % CB) + half * 8 * CB;
+    }
+
+    floatx16 acc[COT][PXT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
+
+    // this wave's K range: steps [s_lo, s_hi) of the (tap outer, channel block inner) order
+    const int nsteps = taps * CiB;
+    const int per = (nsteps + 3) >> 2;
+    const int s_lo = wave * per;
+    const int s_hi = (s_lo + per < nsteps) ? s_lo + per : nsteps;
+    const int mine = s_hi > s_lo ? s_hi - s_lo : 0;
+    int tap0 = (s_lo < nsteps ? s_lo : 0) / CiB;
+    int cib = (s_lo < nsteps ? s_lo : 0) - tap0 * CiB;
+    int ta = tap0 / a.kw, tb = tap0 - (tap0 / a.kw) * a.kw;
+    int left = mine;                 // steps still to be loaded
+
+    auto load_step = [&](float (&A)[COT][8], float4 (&B)[PXT][2]) {
+        const bool live = left > 0;
+        const int tap = ta * a.kw + tb;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
+            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
+            float4 v0 = p[0], v1 = p[1];
+            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
+            B[t][0] = v0;
+            B[t][1] = v1;
+        }
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+        {
+            const float *w = w_row[c] + ((size_t)cib * taps + tap) * (CB * CB);
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) A[c][kk] = w[kk * CB];
+        }
+        if (left > 1)                // stay on a valid position after the last step
+        {
+            if (++cib == CiB)
+            {
+                cib = 0;
+                if (++tb == a.kw) { tb = 0; ++ta; }
+            }
+        }
+        --left;
+    };
+    auto compute_step = [&](const float (&A)[COT][8], const float4 (&B)[PXT][2]) {
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                const float4 bv = B[t][kk >> 2];
+                const float b = (kk & 3) == 0 ? bv.x : (kk & 3) == 1 ? bv.y : (kk & 3) == 2 ? bv.z : bv.w;
+#pragma unroll
+                for (int c = 0; c < COT; ++c)
+                    acc[c][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[c][kk], b, acc[c][t], 0, 0, 0);
+            }
+    };
+
+    float A0[COT][8], A1[COT][8];
+    float4 B0[PXT][2], B1[PXT][2];
+    load_step(A0, B0);
+    const int npairs = (per + 1) >> 1;           // uniform over the workgroup
+    for (int it = 0; it < npairs; ++it)
+    {
+        load_step(A1, B1);
+        compute_step(A0, B0);
+        load_step(A0, B0);
+        compute_step(A1, B1);
+    }
+
+    // ---- reduction over the four K quarters --------------------------------------------------
+    if (wave > 0)
+    {
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[wave - 1][c * PXT + t][r][lane] = acc[c][t][r];
+    }
+    __syncthreads();
+    if (wave == 0)
+    {
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int c = 0; c < COT; ++c)
+#pragma unroll
+                for (int t = 0; t < PXT; ++t)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[c][t][r] += red[w][c * PXT + t][r][lane];
+        conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // first layers: Ci in {1,2,3}; input block is [H][W][Ci], filter [Co/16][kh][kw][Ci][16]
 // grid.x over pixels, grid.y = output channel block (uniform per workgroup -> scalar weight loads)
 template <int CI>
@@ -473,6 +631,16 @@ __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
 }
 
 template <int COT, int PXT>
+void launch_splitk(ConvArgs &a, hipStream_t s)
+{
+    a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
+    a.n_px_blocks = (a.P + 32 * PXT - 1) / (32 * PXT);
+    a.n_blocks = a.n_co_groups * a.n_px_blocks;
+    a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
+    hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+}
+
+template <int COT, int PXT>
 void launch_mfma(ConvArgs &a, hipStream_t s)
 {
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
@@ -537,6 +705,15 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     int cot = 1, pxt = 1;
     if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
     else if (Co % 64 == 0 && tiles32 >= 6 * simds) { cot = 2; pxt = 1; }
+    // few tiles and a long reduction: split K over the four waves of a workgroup
+    bool splitk = tiles32 < 2 * simds && nsteps >= 16;
+    if (const char *e = std::getenv("SMALL_HIP_CONV_SPLITK")) splitk = e[0] == '1';
+    if (splitk)
+    {
+        launch_splitk<1, 1>(a, s);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
     // tuning knob: SMALL_HIP_CONV_TILE="<cot>,<pxt>" forces a wave tile (32-channel x 32-pixel units)
     if (const char *e = std::getenv("SMALL_HIP_CONV_TILE"))
     {
