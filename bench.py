@@ -215,9 +215,22 @@ def main():
             e2 = models.HipExecutor(m2, b)
             s2 = time_forward(e2, max(args.steps, 50), args.warmup)
             ms2 = time_ops(e2, 10)
+            # the same forward pass replayed from a HIP graph (21 launches, no host work in between)
+            e2.capture()
+            for _ in range(args.warmup):
+                e2.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(max(args.steps, 50)):
+                e2.replay()
+            torch.cuda.synchronize()
+            s3 = (time.perf_counter() - t0) / max(args.steps, 50)
             extras["%s_b%d" % (name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
+                                            "hip_graph_images_per_s": round(b / s3, 1),
+                                            "hip_graph_ms_per_step": round(s3 * 1e3, 4),
                                             "layers": layer_table(m2, b, ms2)}
-            log("%s batch %d: %.4f ms/step, %.0f images/s" % (name, b, s2 * 1e3, b / s2))
+            log("%s batch %d: eager %.4f ms/step %.0f images/s | HIP graph %.4f ms/step %.0f images/s"
+                % (name, b, s2 * 1e3, b / s2, s3 * 1e3, b / s3))
             del e2
         torch.cuda.empty_cache()
 

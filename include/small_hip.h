@@ -197,6 +197,28 @@ int small_hip_conv2d_u8_prepared(int batch, int kernel_height, int kernel_width,
                                  const void *prepared, const small_hip_quant *filter_q,
                                  uint8_t *output, const small_hip_quant *output_q,
                                  small_hip_stream_t stream);
+/* Convolution with the element-wise tail of a residual block applied in the same pass, in place on
+ * the convolution's output buffer and with that buffer's quantisation parameters -- bit-identical
+ * to Conv2D(in, filter, out); [Accum(accum_input, out);] [ReLUActivation(out, out);].
+ * accum_input may be NULL (no Accum); relu != 0 applies the ReLU.  No counterpart in the reference
+ * (its residual blocks issue the layers separately, include/small/models/Resnet8Tiny.hpp:262-296). */
+int small_hip_conv2d_accum_relu_u8(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                                   int b_pad, int l_pad, int r_pad, int output_channels,
+                                   int input_channels, int input_height, int input_width,
+                                   const uint8_t *input, const small_hip_quant *input_q,
+                                   const uint8_t *filter, const small_hip_quant *filter_q,
+                                   const uint8_t *accum_input, const small_hip_quant *accum_input_q,
+                                   int relu, uint8_t *output, const small_hip_quant *output_q,
+                                   small_hip_stream_t stream);
+int small_hip_conv2d_accum_relu_u8_prepared(int batch, int kernel_height, int kernel_width, int stride,
+                                            int t_pad, int b_pad, int l_pad, int r_pad,
+                                            int output_channels, int input_channels, int input_height,
+                                            int input_width, const uint8_t *input,
+                                            const small_hip_quant *input_q, const void *prepared,
+                                            const small_hip_quant *filter_q, const uint8_t *accum_input,
+                                            const small_hip_quant *accum_input_q, int relu,
+                                            uint8_t *output, const small_hip_quant *output_q,
+                                            small_hip_stream_t stream);
 /* small::DepthwiseConv2D<QUInt8Buffer>  interface_abstract.hpp:1059-1116 */
 int small_hip_depthwise_conv2d_u8(int batch, int kernel_height, int kernel_width, int stride,
                                   int t_pad, int b_pad, int l_pad, int r_pad, int input_channels,

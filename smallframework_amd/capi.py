@@ -73,6 +73,8 @@ SIGNATURES = {
     "small_hip_conv2d_u8_prepared_filter_bytes": (_sz, [_i] * 4),
     "small_hip_conv2d_u8_prepare_filter": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_conv2d_u8_prepared": (_i, _conv + [_p, _q, _p, _q, _p, _q, _p]),
+    "small_hip_conv2d_accum_relu_u8": (_i, _conv + [_p, _q, _p, _q, _p, _q, _i, _p, _q, _p]),
+    "small_hip_conv2d_accum_relu_u8_prepared": (_i, _conv + [_p, _q, _p, _q, _p, _q, _i, _p, _q, _p]),
     "small_hip_depthwise_conv2d_u8": (_i, _win + [_p, _q, _p, _q, _p, _q, _p]),
     "small_hip_maxpool2d_u8": (_i, _win + [_p, _q, _p, _q, _p]),
     "small_hip_relu_u8": (_i, [_i] * 4 + [_p, _q, _p, _q, _p]),

@@ -11,6 +11,16 @@
 //     SI  = sum_valid I'                 (v_sad_u8 on the bytes the lane loads anyway)
 //     SF  = sum over the valid taps of Wsum[co][tap],  Wsum = sum_ci F'   (filter pre-pass)
 //     nv  = number of valid taps,  ZI = zI + 128,  ZF = zF + 128
+//   The valid taps of a pixel form a rectangle [a_lo,a_hi) x [b_lo,b_hi) of the filter window, so
+//   SF is read from a 2-D prefix-sum table P[(kh+1)*(kw+1)][Co] with four 16-byte loads per lane
+//   (P[hi][hi] - P[lo][hi] - P[hi][lo] + P[lo][lo], exact in wrap-around int32) whatever the
+//   border position; interior pixels are the same formula with the full rectangle.
+//
+// The epilogue can also apply the two element-wise layers that follow a convolution in a residual
+// block, both in place on the convolution's output buffer and both with its quantisation parameters:
+//   Accum(shortcut, out):  out = requant((shortcut + zS) + (out + zO))
+//   ReLUActivation(out, out):  out = requant(max(out + zO, 0))
+// which is bit-identical to issuing the three layers one after the other.
 //
 // A filter pre-pass (one small kernel) turns the packed filter [Co/16][Ci/16][tap][16 ci][16 co]
 // into the MFMA A-operand order [Co/16][step][16 co][16 ci] of signed bytes (step = tap*Ci/16 +
@@ -36,11 +46,13 @@ struct QConvArgs
 {
     const uint8_t *in;
     const int8_t *ft;        // prepared filter [Co/16][S_pad][16][16]
-    const int32_t *wsum;     // [Co][taps]
-    const int32_t *wtot;     // [Co]
+    const int32_t *wpre;     // prefix sums of the per-tap filter sums: [(kh+1)*(kw+1)][Co]
+    const uint8_t *accum_src; // optional shortcut tensor added after the convolution (same shape as out)
     uint8_t *out;
     int batch, Co, Ci, H, W, Ho, Wo, kh, kw, stride, pt, pl;
     int32_t ZI, ZF;          // zero points + 128
+    int32_t zS, zO;          // zero points of the shortcut and of the output buffer (fused Accum / ReLU)
+    int relu;
     QOut q;
     int P, S, S_pad, n_co_groups, n_px_blocks, n_blocks, per_xcd;
 };
@@ -67,27 +79,34 @@ __global__ __launch_bounds__(256) void prep_filter_u8_kernel(const uint8_t *__re
     reinterpret_cast<uint4 *>(ft)[(size_t)(cob * S_pad + s) * 16 + co16] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// one lane per (co, tap): Wsum[co][tap] = sum_ci (F - 128); lane tap==0 also writes Wtot
-__global__ __launch_bounds__(256) void wsum_u8_kernel(const uint8_t *__restrict__ f, int32_t *__restrict__ wsum,
-                                                      int32_t *__restrict__ wtot, int Co, int CiB, int taps)
+// one lane per output channel: per-tap sums Wsum[a][b] = sum_ci (F - 128), then the inclusive 2-D
+// prefix table P[a][b] = sum_{a' < a, b' < b} Wsum[a'][b'] stored as [(kh+1)*(kw+1)][Co]
+__global__ __launch_bounds__(256) void wprefix_u8_kernel(const uint8_t *__restrict__ f, int32_t *__restrict__ wpre,
+                                                         int Co, int CiB, int kh, int kw)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= Co) return;
     const int cob = i >> 4, co16 = i & 15;
-    int32_t tot = 0;
-    for (int tap = 0; tap < taps; ++tap)
+    const int taps = kh * kw;
+    for (int b = 0; b <= kw; ++b) wpre[(size_t)b * Co + i] = 0;
+    for (int a = 0; a < kh; ++a)
     {
-        int32_t s = 0;
-        for (int cib = 0; cib < CiB; ++cib)
+        wpre[(size_t)((a + 1) * (kw + 1)) * Co + i] = 0;
+        uint32_t row = 0;
+        for (int b = 0; b < kw; ++b)
         {
-            const uint8_t *src = f + (((size_t)cob * CiB + cib) * taps + tap) * 256 + co16;
+            int32_t sum = 0;
+            for (int cib = 0; cib < CiB; ++cib)
+            {
+                const uint8_t *src = f + (((size_t)cob * CiB + cib) * taps + a * kw + b) * 256 + co16;
 #pragma unroll
-            for (int ci = 0; ci < 16; ++ci) s += (int32_t)src[ci * 16] - 128;
+                for (int ci = 0; ci < 16; ++ci) sum += (int32_t)src[ci * 16] - 128;
+            }
+            row += (uint32_t)sum;
+            wpre[(size_t)((a + 1) * (kw + 1) + b + 1) * Co + i] =
+                (int32_t)((uint32_t)wpre[(size_t)(a * (kw + 1) + b + 1) * Co + i] + row);
         }
-        wsum[(size_t)i * taps + tap] = s;
-        tot += s;
     }
-    wtot[i] = tot;
 }
 
 // ---- main kernel --------------------------------------------------------------------------------
@@ -185,8 +204,8 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
         }
     }
 
-    // ---- epilogue: zero-point terms, requantise, pack, store ------------------------------------
-    const int taps = a.kh * a.kw;
+    // ---- epilogue: zero-point terms, requantise, optional Accum / ReLU, pack, store ----------------
+    const int pw = a.kw + 1;
 #pragma unroll
     for (int t = 0; t < PXT; ++t)
     {
@@ -197,37 +216,50 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
         if (!pvalid[t]) continue;
         // valid tap rectangle of this pixel
         const int a_lo = ih0[t] < 0 ? -ih0[t] : 0;
-        const int a_hi = (a.H - ih0[t]) < a.kh ? (a.H - ih0[t]) : a.kh;
+        int a_hi = (a.H - ih0[t]) < a.kh ? (a.H - ih0[t]) : a.kh;
         const int b_lo = iw0[t] < 0 ? -iw0[t] : 0;
-        const int b_hi = (a.W - iw0[t]) < a.kw ? (a.W - iw0[t]) : a.kw;
-        const int na = a_hi > a_lo ? a_hi - a_lo : 0, nb = b_hi > b_lo ? b_hi - b_lo : 0;
-        const bool full = (na == a.kh) && (nb == a.kw);
+        int b_hi = (a.W - iw0[t]) < a.kw ? (a.W - iw0[t]) : a.kw;
+        a_hi = a_hi > a_lo ? a_hi : a_lo;
+        b_hi = b_hi > b_lo ? b_hi : b_lo;
         const uint32_t base = (uint32_t)a.ZF * si;
-        const uint32_t cnt = (uint32_t)a.ZF * (uint32_t)(a.Ci * na * nb);
+        const uint32_t cnt = (uint32_t)a.ZF * (uint32_t)(a.Ci * (a_hi - a_lo) * (b_hi - b_lo));
+        const int32_t *p_hh = a.wpre + (size_t)(a_hi * pw + b_hi) * a.Co;
+        const int32_t *p_lh = a.wpre + (size_t)(a_lo * pw + b_hi) * a.Co;
+        const int32_t *p_hl = a.wpre + (size_t)(a_hi * pw + b_lo) * a.Co;
+        const int32_t *p_ll = a.wpre + (size_t)(a_lo * pw + b_lo) * a.Co;
 #pragma unroll
         for (int c = 0; c < COT; ++c)
         {
             const int cob = cg * COT + c;
             if (cob >= CoB) continue;
+            const int co4 = cob * CB + 4 * grp;
+            const uint4 hh = *reinterpret_cast<const uint4 *>(p_hh + co4);
+            const uint4 lh = *reinterpret_cast<const uint4 *>(p_lh + co4);
+            const uint4 hl = *reinterpret_cast<const uint4 *>(p_hl + co4);
+            const uint4 ll = *reinterpret_cast<const uint4 *>(p_ll + co4);
+            const uint32_t sf4[4] = {hh.x - lh.x - hl.x + ll.x, hh.y - lh.y - hl.y + ll.y,
+                                     hh.z - lh.z - hl.z + ll.z, hh.w - lh.w - hl.w + ll.w};
+            uint32_t *o = reinterpret_cast<uint32_t *>(
+                a.out + (((size_t)n_of[t] * CoB + cob) * HoWo + rem_of[t]) * CB + 4 * grp);
+            uint32_t sc = 0;
+            if (a.accum_src)
+                sc = *reinterpret_cast<const uint32_t *>(
+                    a.accum_src + (((size_t)n_of[t] * CoB + cob) * HoWo + rem_of[t]) * CB + 4 * grp);
             uint32_t packed = 0;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
             {
-                const int co = cob * CB + 4 * grp + r;
-                uint32_t sf;
-                if (full) sf = (uint32_t)a.wtot[co];
-                else
+                const uint32_t v = (uint32_t)acc[c][t][r] + base + (uint32_t)a.ZI * (sf4[r] + cnt);
+                uint32_t y = requant_u8((int32_t)v, a.q);
+                if (a.accum_src)
+                    y = requant_u8((int32_t)(((sc >> (8 * r)) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
+                if (a.relu)
                 {
-                    sf = 0;
-                    for (int ta = a_lo; ta < a_hi; ++ta)
-                        for (int tb = b_lo; tb < b_hi; ++tb)
-                            sf += (uint32_t)a.wsum[(size_t)co * taps + ta * a.kw + tb];
+                    const int32_t z = (int32_t)y + a.zO;
+                    y = requant_u8(z > 0 ? z : 0, a.q);
                 }
-                const uint32_t v = (uint32_t)acc[c][t][r] + base + (uint32_t)a.ZI * (sf + cnt);
-                packed |= requant_u8((int32_t)v, a.q) << (8 * r);
+                packed |= y << (8 * r);
             }
-            uint32_t *o = reinterpret_cast<uint32_t *>(
-                a.out + (((size_t)n_of[t] * CoB + cob) * HoWo + rem_of[t]) * CB + 4 * grp);
             *o = packed;
         }
     }
@@ -241,6 +273,9 @@ struct QSmallArgs
     uint8_t *out;
     int batch, Co, H, W, Ho, Wo, kh, kw, stride, pt, pl, P;
     int32_t zi, zf;
+    const uint8_t *accum_src;
+    int32_t zS, zO;
+    int relu;
     QOut q;
 };
 
@@ -280,11 +315,25 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
             }
         }
     }
+    const size_t opos = (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB;
+    uint4 sc4 = make_uint4(0, 0, 0, 0);
+    if (a.accum_src) sc4 = *reinterpret_cast<const uint4 *>(a.accum_src + opos);
+    const uint32_t scw[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
     uint32_t pk[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < CB; ++j) pk[j >> 2] |= requant_u8((int32_t)acc[j], a.q) << (8 * (j & 3));
-    uint4 *o = reinterpret_cast<uint4 *>(a.out + (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB);
-    *o = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    for (int j = 0; j < CB; ++j)
+    {
+        uint32_t y = requant_u8((int32_t)acc[j], a.q);
+        if (a.accum_src)
+            y = requant_u8((int32_t)(((scw[j >> 2] >> (8 * (j & 3))) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
+        if (a.relu)
+        {
+            const int32_t z = (int32_t)y + a.zO;
+            y = requant_u8(z > 0 ? z : 0, a.q);
+        }
+        pk[j >> 2] |= y << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint4 *>(a.out + opos) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 }
 
 size_t ws_ft_bytes(int Co, int S_pad) { return (size_t)Co * S_pad * 16; }
@@ -293,8 +342,7 @@ size_t prepared_bytes(int kh, int kw, int Co, int Ci)
 {
     const int S = kh * kw * (Ci / CB), S_pad = (S + 3) & ~3;
     size_t b = ws_ft_bytes(Co, S_pad);                 // multiple of 64
-    b += (size_t)Co * kh * kw * sizeof(int32_t);       // wsum
-    b += (size_t)Co * sizeof(int32_t);                 // wtot
+    b += (size_t)Co * (kh + 1) * (kw + 1) * sizeof(int32_t);   // prefix sums of the per-tap filter sums
     return (b + 255) & ~(size_t)255;
 }
 
@@ -302,13 +350,12 @@ int prepare_filter(int kh, int kw, int Co, int Ci, const uint8_t *filt, void *ws
 {
     const int CiB = Ci / CB, taps = kh * kw, S = taps * CiB, S_pad = (S + 3) & ~3;
     int8_t *ft = static_cast<int8_t *>(ws);
-    int32_t *wsum = reinterpret_cast<int32_t *>(ft + ws_ft_bytes(Co, S_pad));
-    int32_t *wtot = wsum + (size_t)Co * taps;
+    int32_t *wpre = reinterpret_cast<int32_t *>(ft + ws_ft_bytes(Co, S_pad));
     const int n1 = Co * S_pad;
     hipLaunchKernelGGL(prep_filter_u8_kernel, dim3((n1 + 255) / 256), dim3(256), 0, s, filt, ft, Co, CiB, taps, S_pad);
     SHP_LAUNCH_CHECK("prep_filter_u8_kernel");
-    hipLaunchKernelGGL(wsum_u8_kernel, dim3((Co + 255) / 256), dim3(256), 0, s, filt, wsum, wtot, Co, CiB, taps);
-    SHP_LAUNCH_CHECK("wsum_u8_kernel");
+    hipLaunchKernelGGL(wprefix_u8_kernel, dim3((Co + 255) / 256), dim3(256), 0, s, filt, wpre, Co, CiB, kh, kw);
+    SHP_LAUNCH_CHECK("wprefix_u8_kernel");
     return SMALL_HIP_OK;
 }
 
@@ -342,9 +389,17 @@ int conv_u8_check(const char *op, int batch, int kh, int kw, int stride, int pt,
     return SMALL_HIP_OK;
 }
 
+struct Fuse
+{
+    const uint8_t *accum_src = nullptr;
+    int32_t zS = 0;
+    int relu = 0;
+};
+
 int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
                 int Ci, int H, int W, const uint8_t *in, const small_hip_quant *iq, const void *prepared,
-                const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, hipStream_t s)
+                const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, const Fuse &fz,
+                hipStream_t s)
 {
     QConvArgs a{};
     const int CiB = Ci / CB, taps = kh * kw;
@@ -352,8 +407,11 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     a.S_pad = (a.S + 3) & ~3;
     a.in = in; a.out = out;
     a.ft = static_cast<const int8_t *>(prepared);
-    a.wsum = reinterpret_cast<const int32_t *>(a.ft + ws_ft_bytes(Co, a.S_pad));
-    a.wtot = a.wsum + (size_t)Co * taps;
+    a.wpre = reinterpret_cast<const int32_t *>(a.ft + ws_ft_bytes(Co, a.S_pad));
+    a.accum_src = fz.accum_src;
+    a.zS = fz.zS;
+    a.zO = oq->zero;
+    a.relu = fz.relu;
     a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W; a.kh = kh; a.kw = kw;
     a.stride = stride; a.pt = pt; a.pl = pl;
     a.Ho = out_dim(H, pt, pb, kh, stride);
@@ -375,7 +433,8 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
 
 int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
             int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
-            const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, small_hip_stream_t stream)
+            const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, const Fuse &fz,
+            small_hip_stream_t stream)
 {
     if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt, out, iq, fq, oq))
         return rc;
@@ -388,6 +447,7 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         a.Ho = out_dim(H, pt, pb, kh, stride);
         a.Wo = out_dim(W, pl, pr, kw, stride);
         a.zi = iq->zero; a.zf = fq->zero;
+        a.accum_src = fz.accum_src; a.zS = fz.zS; a.zO = oq->zero; a.relu = fz.relu;
         a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
         const long P = (long)batch * a.Ho * a.Wo;
         if (P == 0) return SMALL_HIP_OK;
@@ -403,7 +463,22 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
     void *ws = nullptr;
     if (int rc = get_workspace(prepared_bytes(kh, kw, Co, Ci), &ws)) return rc;
     if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
-    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, s);
+    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s);
+}
+
+int fuse_check(const char *op, const uint8_t *accum_input, const small_hip_quant *accum_q, const void *out, Fuse *fz,
+               int relu)
+{
+    fz->relu = relu ? 1 : 0;
+    if (accum_input)
+    {
+        if (!accum_q) { set_error("%s: accum_input without quantisation parameters", op); return SMALL_HIP_EINVAL; }
+        if (!aligned16(accum_input) || accum_input == out)
+        { set_error("%s: misaligned or aliased accum_input", op); return SMALL_HIP_EINVAL; }
+        fz->accum_src = accum_input;
+        fz->zS = accum_q->zero;
+    }
+    return SMALL_HIP_OK;
 }
 
 } // namespace
@@ -416,7 +491,7 @@ int small_hip_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, i
                         small_hip_stream_t stream)
 {
     return conv_u8("small_hip_conv2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, filt, fq,
-                   out, oq, stream);
+                   out, oq, Fuse{}, stream);
 }
 
 int small_hip_dense_u8(int batch, int No, int Ni, const uint8_t *in, const small_hip_quant *iq,
@@ -424,7 +499,7 @@ int small_hip_dense_u8(int batch, int No, int Ni, const uint8_t *in, const small
                        small_hip_stream_t stream)
 {
     return conv_u8("small_hip_dense_u8", batch, 1, 1, 1, 0, 0, 0, 0, No, Ni, 1, 1, in, iq, filt, fq, out, oq,
-                   stream);
+                   Fuse{}, stream);
 }
 
 size_t small_hip_conv2d_u8_prepared_filter_bytes(int kh, int kw, int Co, int Ci)
@@ -453,6 +528,35 @@ int small_hip_conv2d_u8_prepared(int batch, int kh, int kw, int stride, int pt, 
     if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, prepared, out, iq, fq, oq))
         return rc;
     return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, prepared, fq, out, oq,
+                       Fuse{}, as_stream(stream));
+}
+
+int small_hip_conv2d_accum_relu_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
+                                   int Ci, int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                                   const uint8_t *filt, const small_hip_quant *fq, const uint8_t *accum_input,
+                                   const small_hip_quant *accum_q, int relu, uint8_t *out,
+                                   const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_conv2d_accum_relu_u8";
+    Fuse fz;
+    if (int rc = fuse_check(op, accum_input, accum_q, out, &fz, relu)) return rc;
+    return conv_u8(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, filt, fq, out, oq, fz, stream);
+}
+
+int small_hip_conv2d_accum_relu_u8_prepared(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                            int Co, int Ci, int H, int W, const uint8_t *in,
+                                            const small_hip_quant *iq, const void *prepared,
+                                            const small_hip_quant *fq, const uint8_t *accum_input,
+                                            const small_hip_quant *accum_q, int relu, uint8_t *out,
+                                            const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_conv2d_accum_relu_u8_prepared";
+    if (Ci <= 0 || Ci % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, prepared, out, iq, fq, oq))
+        return rc;
+    Fuse fz;
+    if (int rc = fuse_check(op, accum_input, accum_q, out, &fz, relu)) return rc;
+    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, prepared, fq, out, oq, fz,
                        as_stream(stream));
 }
 

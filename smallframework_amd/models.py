@@ -365,6 +365,22 @@ class HipExecutor:
                     capi.check(self.lib.small_hip_conv2d_u8_prepare_filter(op.kh, op.kw, op.Co, op.C,
                                                                            self._p(self.w[op.weight]), self._p(t), st))
                     self.prep[op.weight] = t
+        # uint8 residual blocks: Conv2D [+ Accum onto its output] [+ in-place ReLU] run as one launch
+        self.plan = []
+        ops = model.ops
+        i = 0
+        while i < len(ops):
+            op = ops[i]
+            acc_op, relu, j = None, False, i + 1
+            if fused and model.dtype == "u8" and op.kind == "conv":
+                if j < len(ops) and ops[j].kind == "accum" and ops[j].dst == op.dst and ops[j].src != op.dst:
+                    acc_op = ops[j]
+                    j += 1
+                if j < len(ops) and ops[j].kind == "relu" and ops[j].src == op.dst and ops[j].dst == op.dst:
+                    relu = True
+                    j += 1
+            self.plan.append((op, acc_op, relu))
+            i = j
         torch.cuda.synchronize()
 
     @staticmethod
@@ -379,6 +395,22 @@ class HipExecutor:
         c, h, w = op.out_shape()
         self.torch.cuda.synchronize()
         return self.buf[self.model.out][: self.batch * c * h * w].cpu().numpy()
+
+    def run_fused_u8(self, op, acc_op, relu, st):
+        """Conv2D + optional Accum + optional in-place ReLU in one launch (bit-identical to the sequence)."""
+        L, p, B, b, q = self.lib, self._p, self.batch, self.buf, self.q
+        t_, b_, l_, r_ = op.pads
+        args = (B, op.kh, op.kw, op.stride, t_, b_, l_, r_, op.Co, op.C, op.H, op.W)
+        iq, fq, oq = C.byref(q[op.src]), C.byref(q[op.weight]), C.byref(q[op.dst])
+        acc_p = p(b[acc_op.src]) if acc_op else None
+        acc_q = C.byref(q[acc_op.src]) if acc_op else None
+        if op.weight in self.prep:
+            rc = L.small_hip_conv2d_accum_relu_u8_prepared(*args, p(b[op.src]), iq, p(self.prep[op.weight]), fq,
+                                                           acc_p, acc_q, int(relu), p(b[op.dst]), oq, st)
+        else:
+            rc = L.small_hip_conv2d_accum_relu_u8(*args, p(b[op.src]), iq, p(self.w[op.weight]), fq,
+                                                  acc_p, acc_q, int(relu), p(b[op.dst]), oq, st)
+        capi.check(rc)
 
     def run_op(self, op: Op, st):
         L, p, B, b = self.lib, self._p, self.batch, self.buf
@@ -448,5 +480,23 @@ class HipExecutor:
 
     def forward(self):
         st = self.stream()
-        for op in self.model.ops:
-            self.run_op(op, st)
+        for op, acc_op, relu in self.plan:
+            if acc_op is not None or relu:
+                self.run_fused_u8(op, acc_op, relu, st)
+            else:
+                self.run_op(op, st)
+
+    def capture(self):
+        """Record one forward pass into a HIP graph (the launches go to the capture stream through the
+        same C ABI calls).  Needs the prepared-filter path for uint8 models: capture must not allocate."""
+        torch = self.torch
+        self.forward()                      # warm up outside the capture (lazy module loading)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.forward()
+        self.graph = g
+        return g
+
+    def replay(self):
+        self.graph.replay()

@@ -104,10 +104,13 @@ def test_tiny_yolo_v2_error_is_reference_sized():
     assert e_gpu.max() <= 2.0 * e_ref.max() + 1e-6
 
 
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
 @pytest.mark.parametrize("prepared", [True, False], ids=["prepared", "direct"])
 @pytest.mark.parametrize("disc", [False, True], ids=["config", "discriminating"])
-def test_resnet8_u8(disc, prepared):
-    got, want = _run(models.resnet8_u8(discriminating=disc), 5, prepared=prepared)
+def test_resnet8_u8(disc, prepared, fused):
+    """fused: Conv2D + Accum + ReLU of a residual block in one launch; the oracle always runs the
+    layers one after the other."""
+    got, want = _run(models.resnet8_u8(discriminating=disc), 5, fused=fused, prepared=prepared)
     assert_equal_exact(got, want, "resnet8_u8")
 
 
@@ -137,3 +140,31 @@ def test_layer_sweep_batch1(m):
         assert_equal_exact(got, want, m.name)
     else:
         assert_close_f32(got, want, what=m.name)
+
+
+@pytest.mark.parametrize("name,batch", [("resnet8_u8", 4), ("dscnn", 2)])
+def test_hip_graph_replays_match_eager(name, batch):
+    """A captured forward pass must reproduce the eager result on every replay, with eager work and
+    synchronisations between the replays."""
+    import torch
+    m = getattr(models, name)(discriminating=True) if name == "resnet8_u8" else getattr(models, name)()
+    w = models.make_weights(m)
+    x = models.make_input(m, batch)
+    ex = models.HipExecutor(m, batch, w, x)
+    ex.forward()
+    eager = ex.output().copy()
+    ex.capture()
+    for rep in range(4):
+        # different input every replay so a stale result cannot pass
+        xr = models.make_input(m, batch, seed=200 + rep)
+        ex.buf["in"].copy_(torch.from_numpy(xr))
+        ex.replay()
+        got = ex.output().copy()
+        ex.forward()                      # eager pass on the same input, in between replays
+        want = ex.output().copy()
+        if m.dtype == "u8":
+            assert_equal_exact(got, want, "graph replay %d" % rep)
+        else:
+            assert_equal_exact(got, want, "graph replay %d" % rep)
+        torch.cuda.synchronize()
+    assert eager.shape == got.shape

@@ -372,3 +372,31 @@ def test_dense_u8(lib, oracle):
     assert lib.small_hip_dense_u8(batch, No, Ni, hu.ptr(dx), hu.qref(iq), hu.ptr(dw), hu.qref(fq), hu.ptr(do),
                                   hu.qref(oq), hu.stream()) == 0
     assert_equal_exact(hu.host(do), oracle.dense_u8(batch, CB, No, Ni, x, _oq(iq), w, _oq(fq), _oq(oq))[1], "dense_u8")
+
+
+@pytest.mark.parametrize("qp", QPARAMS[:4], ids=str)
+@pytest.mark.parametrize("mode", ["relu", "accum", "accum_relu"])
+def test_conv2d_accum_relu_u8_equals_sequence(lib, oracle, qp, mode):
+    """The fused entry point against the oracle's Conv2D -> Accum -> ReLU sequence, bit for bit."""
+    zi, zf, mul, ls, rs = qp
+    for (batch, kh, kw, s, (pt, pb, pl, pr), Co, Ci, H, W) in [(2, 3, 3, 1, (1, 1, 1, 1), 32, 16, 9, 10),
+                                                                (2, 3, 3, 2, (0, 1, 0, 1), 16, 3, 12, 12)]:
+        x = synth.uniform_u8(71, batch * Ci * H * W)
+        f = synth.uniform_u8(72, Co * Ci * kh * kw)
+        Ho, Wo = oracle.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
+        sc = synth.uniform_u8(73, batch * Co * Ho * Wo)
+        iq, fq, oq, sq = hu.q(zi), hu.q(zf), hu.q(-9, mul, ls, rs), hu.q(11)
+        dx, df, dsc = hu.dev(x), hu.dev(f), hu.dev(sc)
+        do = hu.dev_empty(batch * Co * Ho * Wo, np.uint8)
+        use_acc, use_relu = mode != "relu", mode != "accum"
+        rc = lib.small_hip_conv2d_accum_relu_u8(batch, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, hu.ptr(dx),
+                                                hu.qref(iq), hu.ptr(df), hu.qref(fq),
+                                                hu.ptr(dsc) if use_acc else None, hu.qref(sq) if use_acc else None,
+                                                int(use_relu), hu.ptr(do), hu.qref(oq), hu.stream())
+        assert rc == 0, lib.small_hip_last_error()
+        _, want = oracle.conv2d_u8(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, _oq(iq), f, _oq(fq), _oq(oq))
+        if use_acc:
+            _, want = oracle.accum_u8(batch, CB, Co, Ho, Wo, sc, _oq(sq), want, _oq(oq))
+        if use_relu:
+            _, want = oracle.relu_u8(batch, CB, Co, Ho, Wo, want, _oq(oq), _oq(oq))
+        assert_equal_exact(hu.host(do), want, "fused %s Ci=%d" % (mode, Ci))
