@@ -108,6 +108,97 @@ __global__ __launch_bounds__(TPB) void pool_u8_kernel(const uint32_t *__restrict
     out[i] = packed;
 }
 
+// Global pooling (the window is the whole un-padded image, one output pixel per channel): one wave
+// per (image, channel block).  Lane = (pixel slot, channel quad): the 16 slots stride over the
+// pixels with 16-byte (float) / 4-byte (uint8) accesses, i.e. the wave reads whole kilobytes /
+// 256-byte runs, then the slots are combined with a wavefront xor-shuffle reduction.
+template <bool IS_MAX>
+__global__ __launch_bounds__(TPB) void global_pool_f32_kernel(const float4 *__restrict__ in,
+                                                              float4 *__restrict__ out, int planes, int hw,
+                                                              float norm)
+{
+    const int plane = blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
+    if (plane >= planes) return;                     // whole waves leave together
+    const int lane = threadIdx.x & 63, q = lane & 3, slot = lane >> 2;
+    const float4 *src = in + (size_t)plane * hw * 4 + q;
+    // every slot starts from pixel 0 for max (any element of the window is a valid start value)
+    float4 acc = IS_MAX ? src[0] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int p = slot; p < hw; p += 16)
+    {
+        const float4 v = src[(size_t)p * 4];
+        if (IS_MAX)
+        {
+            acc.x = v.x > acc.x ? v.x : acc.x; acc.y = v.y > acc.y ? v.y : acc.y;
+            acc.z = v.z > acc.z ? v.z : acc.z; acc.w = v.w > acc.w ? v.w : acc.w;
+        }
+        else { acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w; }
+    }
+#pragma unroll
+    for (int m = 4; m < 64; m <<= 1)
+    {
+        const float ox = __shfl_xor(acc.x, m), oy = __shfl_xor(acc.y, m);
+        const float oz = __shfl_xor(acc.z, m), ow = __shfl_xor(acc.w, m);
+        if (IS_MAX)
+        {
+            acc.x = ox > acc.x ? ox : acc.x; acc.y = oy > acc.y ? oy : acc.y;
+            acc.z = oz > acc.z ? oz : acc.z; acc.w = ow > acc.w ? ow : acc.w;
+        }
+        else { acc.x += ox; acc.y += oy; acc.z += oz; acc.w += ow; }
+    }
+    if (!IS_MAX) { acc.x *= norm; acc.y *= norm; acc.z *= norm; acc.w *= norm; }
+    if (slot == 0) out[(size_t)plane * 4 + q] = acc;
+}
+
+template <bool IS_MAX>
+__global__ __launch_bounds__(TPB) void global_pool_u8_kernel(const uint32_t *__restrict__ in,
+                                                             uint32_t *__restrict__ out, int planes, int hw,
+                                                             int32_t zi, QOut qo)
+{
+    const int plane = blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
+    if (plane >= planes) return;
+    const int lane = threadIdx.x & 63, q = lane & 3, slot = lane >> 2;
+    const uint32_t *src = in + (size_t)plane * hw * 4 + q;
+    int32_t acc[4];
+    {
+        // un-padded max windows start from the first RAW byte (q_abstract_layer.hpp:286-293)
+        const uint32_t v0 = src[0];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[b] = IS_MAX ? (int32_t)((v0 >> (8 * b)) & 0xffu) : 0;
+    }
+    for (int p = slot; p < hw; p += 16)
+    {
+        const uint32_t v = src[(size_t)p * 4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+        {
+            const int32_t x = (int32_t)((v >> (8 * b)) & 0xffu) + zi;
+            if (IS_MAX) acc[b] = x > acc[b] ? x : acc[b];
+            else acc[b] = (int32_t)((uint32_t)acc[b] + (uint32_t)x);
+        }
+    }
+#pragma unroll
+    for (int m = 4; m < 64; m <<= 1)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+        {
+            const int32_t o = __shfl_xor(acc[b], m);
+            if (IS_MAX) acc[b] = o > acc[b] ? o : acc[b];
+            else acc[b] = (int32_t)((uint32_t)acc[b] + (uint32_t)o);
+        }
+    if (slot == 0)
+    {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) packed |= requant_u8(acc[b], qo) << (8 * b);
+        out[(size_t)plane * 4 + q] = packed;
+    }
+}
+
+inline bool is_global(const Geom &g, int pt, int pb, int pl, int pr)
+{
+    return g.kh == g.H && g.kw == g.W && pt == 0 && pb == 0 && pl == 0 && pr == 0 && g.H * g.W >= 16;
+}
+
 int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, int pt, int pb, int pl,
                int pr, int C, int H, int W, const void *in, const void *out, Geom *g)
 {
@@ -133,6 +224,15 @@ int pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     const size_t total4 = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total4 == 0) return SMALL_HIP_OK;
     const float norm = (float)(1.0 / (1.0 * kh * kw));
+    if (is_global(g, pt, pb, pl, pr))
+    {
+        const int planes = batch * (C / CB);
+        hipLaunchKernelGGL(global_pool_f32_kernel<IS_MAX>, dim3((planes + TPB / 64 - 1) / (TPB / 64)), dim3(TPB), 0,
+                           as_stream(stream), reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out),
+                           planes, H * W, norm);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
     hipLaunchKernelGGL(pool_f32_kernel<IS_MAX>, dim3((unsigned)((total4 + TPB - 1) / TPB)), dim3(TPB), 0,
                        as_stream(stream), reinterpret_cast<const float4 *>(in),
                        reinterpret_cast<float4 *>(out), total4, g, norm);
@@ -151,6 +251,15 @@ int pool_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
     const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total == 0) return SMALL_HIP_OK;
     const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    if (is_global(g, pt, pb, pl, pr))
+    {
+        const int planes = batch * (C / CB);
+        hipLaunchKernelGGL(global_pool_u8_kernel<IS_MAX>, dim3((planes + TPB / 64 - 1) / (TPB / 64)), dim3(TPB), 0,
+                           as_stream(stream), reinterpret_cast<const uint32_t *>(in),
+                           reinterpret_cast<uint32_t *>(out), planes, H * W, iq->zero, q);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
     hipLaunchKernelGGL(pool_u8_kernel<IS_MAX>, dim3((unsigned)((total + TPB - 1) / TPB)), dim3(TPB), 0,
                        as_stream(stream), reinterpret_cast<const uint32_t *>(in),
                        reinterpret_cast<uint32_t *>(out), total, g, iq->zero, q);
