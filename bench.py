@@ -24,6 +24,12 @@ PEAK_HBM = 8.0e12          # B/s, MI355X HBM3E
 PEAK_MFMA_F32 = 157.3e12   # FLOP/s, dense fp32 MFMA
 PEAK_MFMA_I8 = 5.0e15      # OP/s, dense int8 MFMA
 
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs) over this same benchmark and scaled by what the counters read for an
+# in-place ReLU of known size (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); the summary is
+# profiles/mobilenet_v1_b64_traffic_and_mfma.md.  Keyed by (model, batch, kernel family).
+MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_kernel"): 94.3}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -202,6 +208,9 @@ def main():
         ach = d["bytes"] / (d["ms"] * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s",
                 "frac": round(ach / 8000.0, 4), "traffic": None}
+    mt = MEASURED_TRAFFIC_MB_PER_LAUNCH.get((model.name, batch, dom))
+    if mt is not None and not args.unfused:
+        roof["traffic"] = round(mt * 1e6)      # bytes per launch, like algorithmic_per_launch
     roof.update({"kernel": dom, "launches_per_step": d["launches"],
                  "avg_launch_ms": round(d["ms"] / d["launches"], 5),
                  "algorithmic_per_launch": {"GFLOP": round(d["flops"] / d["launches"] / 1e9, 3),
