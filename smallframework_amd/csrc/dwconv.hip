@@ -1,10 +1,14 @@
 // DepthwiseConv2D / PartialDepthwiseConv2D (float32, optional fused bias + activation) and
 // DepthwiseConv2D (uint8).  Bandwidth-bound, no MFMA: a lane owns four channels of one output
-// pixel, so the four lanes of a (pixel, channel-block) read one 64-byte line per tap and a wave
-// covers 16 neighbouring output pixels.  Filter taps ([C/16][kh][kw][16], 576 bytes per block for
-// 3x3) are read through the vector cache; every lane of a workgroup row uses the same lines.
+// pixel, so the four lanes of a (pixel, channel-block) touch one 64-byte line per tap and a wave
+// covers 16 neighbouring output pixels.  Three float32 kernels, picked by shape:
+//   - 3x3 on images of at least 14x14 (28x28 at stride 2) outputs: input tile staged in LDS
+//   - other 3x3: a lane loads a strip of rows into registers
+//   - any other window: one output per lane, taps read through the vector cache
 #include "common.h"
 #include "quant.h"
+
+#include <cstdlib>
 
 using namespace shp;
 
@@ -152,6 +156,125 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
     }
 }
 
+// 3x3 depthwise through LDS.  A workgroup owns a TW x TH tile of output pixels of one (image,
+// channel block) plane.  The input pixels under it (64 bytes each) are fetched from memory exactly
+// once, in row-contiguous 16-byte pieces with every load in flight together, and parked in LDS with
+// zeros where the tile hangs over the image; the nine filter taps of the block go to LDS too.  A
+// lane then owns one output column, four channels and R consecutive rows.  At stride 1 it slides a
+// three-row register window down the staged tile (three 16-byte LDS reads per output); at stride 2
+// it reads its nine taps per output.  The strip kernel issued 4.5 (stride 1) to 7 (stride 2)
+// vector-cache loads per output plus nine tap loads per lane, and that cache, not HBM, was its limit.
+template <int S, int TW, int R>
+__global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__restrict__ in,
+                                                             const float4 *__restrict__ filt, float4 *out,
+                                                             int cblocks, int tiles_x, int tiles_y,
+                                                             int nblocks, int per_xcd, Geom g, Epi e)
+{
+    constexpr int SR = 64 / TW;                              // rows of lane slots
+    constexpr int TH = SR * R;                               // output rows per tile
+    constexpr int IW = (TW - 1) * S + 3, IH = (TH - 1) * S + 3;  // staged input tile, in pixels
+    constexpr int ROW4 = IW * 4;                             // float4 per staged row
+    constexpr int E = IH * ROW4;
+    constexpr int NLD = (E + TPB - 1) / TPB;
+    __shared__ float4 sX[E];
+    __shared__ float4 sW[36];
+
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * per_xcd + bid / NUM_XCD;
+    if (lid >= nblocks) return;              // the whole workgroup leaves, before any barrier
+    const int tiles = tiles_x * tiles_y;
+    const int plane = lid / tiles, tile = lid - plane * tiles;
+    const int tyi = tile / tiles_x, txi = tile - tyi * tiles_x;
+    const int cbk = plane % cblocks;
+    const int oh0 = tyi * TH, ow0 = txi * TW;
+    const int ih0 = oh0 * S - g.pt, iw0 = ow0 * S - g.pl;
+    const float4 *src = in + (size_t)plane * g.H * g.W * 4;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int tid = threadIdx.x;
+
+    float4 v[NLD];
+#pragma unroll
+    for (int k = 0; k < NLD; ++k)
+    {
+        const int el = tid + k * TPB;
+        const int r = el / ROW4, c4 = el - r * ROW4;
+        const int ih = ih0 + r, iw = iw0 + (c4 >> 2);
+        const bool ok = el < E && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+        v[k] = src[ok ? ((size_t)ih * g.W + iw) * 4 + (c4 & 3) : 0];
+        if (!ok) v[k] = zero;
+    }
+    if (tid < 36) sW[tid] = filt[(size_t)cbk * 36 + tid];
+#pragma unroll
+    for (int k = 0; k < NLD; ++k)
+    {
+        const int el = tid + k * TPB;
+        if (el < E) sX[el] = v[k];
+    }
+    __syncthreads();
+
+    const int q = tid & 3, slot = tid >> 2;
+    const int tx = slot % TW, sy = slot / TW;
+    const int ow = ow0 + tx;
+    float4 w[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w[t] = sW[t * 4 + q];
+    float4 bias = zero;
+    if (e.bias) bias = e.bias[cbk * 4 + q];
+    const float4 *xs = sX + ((sy * R * S) * IW + tx * S) * 4 + q;
+    float4 *dst = out + (size_t)plane * g.Ho * g.Wo * 4 + (size_t)ow * 4 + q;
+    const bool col_ok = ow < g.Wo;
+
+    float4 win[3][3];
+    if (S == 1)
+    {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[a][c] = xs[(a * IW + c) * 4];
+    }
+#pragma unroll
+    for (int o = 0; o < R; ++o)
+    {
+        if (S == 1)
+        {
+            // rows o, o+1, o+2 of the lane's window live in win[o%3], win[(o+1)%3], win[(o+2)%3]
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[(o + 2) % 3][c] = xs[((o + 2) * IW + c) * 4];
+        }
+        else
+        {
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int c = 0; c < 3; ++c) win[(o + a) % 3][c] = xs[((o * S + a) * IW + c) * 4];
+        }
+        const int oh = oh0 + sy * R + o;
+        const bool ok = col_ok && oh < g.Ho;
+        float4 acc = bias;
+        if (e.accumulate) { acc = zero; if (ok) acc = dst[(size_t)oh * g.Wo * 4]; }
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+            {
+                const float4 x = win[(o + a) % 3][c];
+                const float4 k = w[a * 3 + c];
+                acc.x = fmaf(x.x, k.x, acc.x); acc.y = fmaf(x.y, k.y, acc.y);
+                acc.z = fmaf(x.z, k.z, acc.z); acc.w = fmaf(x.w, k.w, acc.w);
+            }
+        if (e.accumulate && e.bias) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }
+        acc.x = act1(acc.x, e.act, e.slope); acc.y = act1(acc.y, e.act, e.slope);
+        acc.z = act1(acc.z, e.act, e.slope); acc.w = act1(acc.w, e.act, e.slope);
+        if (ok) dst[(size_t)oh * g.Wo * 4] = acc;
+    }
+}
+
+// tile shapes of the LDS kernel: (TW, R) -> a TW x (64/TW)*R tile of output pixels
+struct TileShape { int tw, th; };
+constexpr TileShape TILE_SHAPES_S1[] = {{16, 16}, {8, 56}, {16, 28}, {32, 8}};
+constexpr TileShape TILE_SHAPES_S2[] = {{8, 8}, {4, 16}, {16, 4}};
+
+
 __global__ __launch_bounds__(TPB) void dw_u8_kernel(const uint32_t *__restrict__ in,
                                                     const uint32_t *__restrict__ filt,
                                                     uint32_t *__restrict__ out, size_t total,
@@ -223,6 +346,44 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
     if (kh == 3 && kw == 3)
     {
         constexpr int R1 = 4, R2 = 3;      // output rows per lane at stride 1 / stride 2
+        static const bool tile_off = [] { const char *v = std::getenv("SMALL_HIP_DW_TILE"); return v && v[0] == '0'; }();
+        // measured: the strip kernel wins below 14x14 outputs at stride 1 and below 28x28 at stride 2
+        const int min_side = stride == 1 ? 14 : 28;
+        if (g.Ho >= min_side && g.Wo >= min_side && !tile_off)
+        {
+            // the tile shape that wastes the fewest lanes on this image; ties go to the first
+            const TileShape *shapes = stride == 1 ? TILE_SHAPES_S1 : TILE_SHAPES_S2;
+            int best = -1;
+            double best_util = 0.7;        // below that the strip kernel is the better choice
+            const int nshapes = stride == 1 ? 4 : 3;
+            for (int t = 0; t < nshapes; ++t)
+            {
+                const int tx = (g.Wo + shapes[t].tw - 1) / shapes[t].tw;
+                const int ty = (g.Ho + shapes[t].th - 1) / shapes[t].th;
+                const double util = (double)g.Wo * g.Ho / ((double)tx * shapes[t].tw * ty * shapes[t].th);
+                if (util > best_util + 1e-9) { best_util = util; best = t; }
+            }
+            if (best >= 0)
+            {
+                const int tiles_x = (g.Wo + shapes[best].tw - 1) / shapes[best].tw;
+                const int tiles_y = (g.Ho + shapes[best].th - 1) / shapes[best].th;
+                const size_t nb = (size_t)batch * (C / CB) * tiles_x * tiles_y;
+                if (nb > 0x7fffffff / 2) { set_error("%s: too many blocks for one launch", op); return SMALL_HIP_EINVAL; }
+                const int nblocks = (int)nb, per_xcd = (nblocks + NUM_XCD - 1) / NUM_XCD;
+                decltype(&dw3x3_f32_tile_kernel<1, 16, 4>) tk;
+                if (stride == 1)
+                    tk = best == 0 ? dw3x3_f32_tile_kernel<1, 16, 4> : best == 1 ? dw3x3_f32_tile_kernel<1, 8, 7>
+                       : best == 2 ? dw3x3_f32_tile_kernel<1, 16, 7> : dw3x3_f32_tile_kernel<1, 32, 4>;
+                else
+                    tk = best == 0 ? dw3x3_f32_tile_kernel<2, 8, 1> : best == 1 ? dw3x3_f32_tile_kernel<2, 4, 1>
+                                                                   : dw3x3_f32_tile_kernel<2, 16, 1>;
+                hipLaunchKernelGGL(tk, dim3(per_xcd * NUM_XCD), dim3(TPB), 0, as_stream(stream),
+                                   reinterpret_cast<const float4 *>(in), reinterpret_cast<const float4 *>(filt),
+                                   reinterpret_cast<float4 *>(out), C / CB, tiles_x, tiles_y, nblocks, per_xcd, g, e);
+                SHP_LAUNCH_CHECK(op);
+                return SMALL_HIP_OK;
+            }
+        }
         const int rows = stride == 1 ? R1 : R2;
         const size_t ncols4 = (size_t)batch * C * g.Wo / 4;
         const int nstrips = (g.Ho + rows - 1) / rows;

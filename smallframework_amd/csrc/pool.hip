@@ -59,6 +59,61 @@ __global__ __launch_bounds__(TPB) void pool_f32_kernel(const float4 *__restrict_
     out[i] = acc;
 }
 
+// Fixed-window variant (2x2 and 3x3 cover the networks in use): the taps are unrolled and every
+// load is issued before the first use, out-of-image taps read a clamped address and are replaced
+// by 0.  For max that is the reference rule itself (a window that touches padding includes 0, an
+// interior window has no replaced tap); for average, adding +0 leaves the running sum unchanged.
+template <bool IS_MAX, int KH, int KW>
+__global__ __launch_bounds__(TPB) void pool_win_f32_kernel(const float4 *__restrict__ in,
+                                                           float4 *__restrict__ out, size_t total4,
+                                                           Geom g, float norm)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= total4) return;
+    const int q = (int)(i & 3);
+    size_t pix = i >> 2;
+    const int ow = (int)(pix % (size_t)g.Wo);
+    pix /= (size_t)g.Wo;
+    const int oh = (int)(pix % (size_t)g.Ho);
+    const size_t plane = pix / (size_t)g.Ho;
+    const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
+    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    float4 v[KH * KW];
+#pragma unroll
+    for (int a = 0; a < KH; ++a)
+#pragma unroll
+        for (int b = 0; b < KW; ++b)
+        {
+            const int ih = ih0 + a, iw = iw0 + b;
+            const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 1);
+            v[a * KW + b] = src[((size_t)ihc * g.W + iwc) * 4];
+        }
+    const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + KH <= g.H && iw0 + KW <= g.W;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (IS_MAX && full) acc = v[0];
+#pragma unroll
+    for (int a = 0; a < KH; ++a)
+#pragma unroll
+        for (int b = 0; b < KW; ++b)
+        {
+            const int ih = ih0 + a, iw = iw0 + b;
+            const bool ok = ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+            float4 t = v[a * KW + b];
+            if (!ok) t = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (IS_MAX)
+            {
+                acc.x = t.x > acc.x ? t.x : acc.x; acc.y = t.y > acc.y ? t.y : acc.y;
+                acc.z = t.z > acc.z ? t.z : acc.z; acc.w = t.w > acc.w ? t.w : acc.w;
+            }
+            else
+            {
+                acc.x = acc.x + t.x; acc.y = acc.y + t.y; acc.z = acc.z + t.z; acc.w = acc.w + t.w;
+            }
+        }
+    if (!IS_MAX) { acc.x *= norm; acc.y *= norm; acc.z *= norm; acc.w *= norm; }
+    out[i] = acc;
+}
+
 // uint8: a lane owns 4 channels (one dword) of one output pixel
 template <bool IS_MAX>
 __global__ __launch_bounds__(TPB) void pool_u8_kernel(const uint32_t *__restrict__ in,
@@ -233,7 +288,10 @@ int pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }
-    hipLaunchKernelGGL(pool_f32_kernel<IS_MAX>, dim3((unsigned)((total4 + TPB - 1) / TPB)), dim3(TPB), 0,
+    auto kern = pool_f32_kernel<IS_MAX>;
+    if (kh == 2 && kw == 2) kern = pool_win_f32_kernel<IS_MAX, 2, 2>;
+    if (kh == 3 && kw == 3) kern = pool_win_f32_kernel<IS_MAX, 3, 3>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((total4 + TPB - 1) / TPB)), dim3(TPB), 0,
                        as_stream(stream), reinterpret_cast<const float4 *>(in),
                        reinterpret_cast<float4 *>(out), total4, g, norm);
     SHP_LAUNCH_CHECK(op);

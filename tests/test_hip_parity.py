@@ -125,6 +125,22 @@ WIN_CASES = [
     (2, 7, 7, 1, (0, 0, 0, 0), 64, 7, 7),
     (1, 25, 5, 1, (0, 0, 0, 0), 64, 25, 5),
     (1, 3, 3, 2, (0, 0, 0, 0), 256, 56, 56),
+    # stride-1 3x3 at sizes that select each tile shape of the LDS depthwise kernel, whole and ragged
+    (2, 3, 3, 1, (1, 1, 1, 1), 32, 16, 16),
+    (1, 3, 3, 1, (1, 1, 1, 1), 16, 56, 56),
+    (2, 3, 3, 1, (1, 1, 1, 1), 32, 28, 28),
+    (1, 3, 3, 1, (1, 1, 1, 1), 16, 24, 32),
+    (2, 3, 3, 1, (0, 1, 0, 1), 16, 15, 30),
+    (1, 3, 3, 1, (0, 0, 0, 0), 16, 30, 30),
+    (1, 3, 3, 1, (1, 1, 1, 1), 16, 56, 15),
+    (1, 3, 3, 1, (1, 1, 1, 1), 16, 23, 63),
+    (3, 3, 3, 1, (1, 1, 1, 1), 48, 14, 14),
+    # stride 2 through the same kernel: 56x56, 28x28 (4x16 tiles), ragged 8x8 tiles, 28x32 (16x4 tiles); 14x52 stays on the strip kernel
+    (1, 3, 3, 2, (0, 1, 0, 1), 16, 112, 112),
+    (2, 3, 3, 2, (0, 1, 0, 1), 32, 56, 56),
+    (1, 3, 3, 2, (1, 1, 1, 1), 16, 27, 103),
+    (1, 3, 3, 2, (0, 1, 0, 1), 16, 62, 32),
+    (2, 3, 3, 2, (0, 1, 0, 1), 16, 56, 64),
 ]
 
 
