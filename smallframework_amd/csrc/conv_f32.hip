@@ -57,6 +57,7 @@ struct ConvArgs
     int n_px_blocks;     // ceil(P / (32*PXT*4))
     int n_blocks;        // n_co_groups * n_px_blocks
     int per_xcd;         // ceil(n_blocks / 8)
+    int n_main;          // hybrid kernel: workgroups that run whole tiles (multiple of the CU count)
 };
 
 __device__ __forceinline__ float act1(float v, int act, float slope)
@@ -251,16 +252,9 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
 constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks start 16 banks apart
 
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a)
+__device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
+                                              const int cg, const int pxb)
 {
-    __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
-
-    const int bid = blockIdx.x;
-    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
-    if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
-    const int cg = lid % a.n_co_groups;
-    const int pxb = lid / a.n_co_groups;
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -404,6 +398,16 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a
     conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a)
+{
+    __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
+    conv_lds_tile<COT, PXT>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Small outputs (few 32x32 tiles per SIMD: fully connected layers, 7x7 / 13x13 feature maps,
 // batch 1): the four waves of a workgroup take the SAME output tile and one quarter of the K-steps
@@ -411,16 +415,9 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a
 // the fixed order 0+1+2+3 (deterministic) and runs the epilogue.  Operands go straight from global
 // memory to the MFMA registers (nothing is shared between the waves until the reduction).
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a)
+__device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)[3][COT * PXT][16][64],
+                                                 const int cg, const int pxb)
 {
-    __shared__ float red[3][COT * PXT][16][64];
-
-    const int bid = blockIdx.x;
-    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
-    if (lid >= a.n_blocks) return;
-    const int cg = lid % a.n_co_groups;
-    const int pxb = lid / a.n_co_groups;
-
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = lane & 31;
@@ -562,6 +559,48 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
     }
 }
 
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a)
+{
+    __shared__ float red[3][COT * PXT][16][64];
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
+    if (lid >= a.n_blocks) return;
+    conv_splitk_tile<COT, PXT>(a, red, lid % a.n_co_groups, lid / a.n_co_groups);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Whole rounds + balanced tail in one launch.  The MFMA pipes are the bound, so a launch whose
+// workgroup count is not a multiple of the CU count ends with a round in which a few CUs work and
+// the rest idle for a whole workgroup time.  Here the first n_main workgroups (a multiple of the
+// CU count) run the LDS-staged kernel on their COT x (4*PXT) tiles; what is left over is cut into
+// single 32x32 tiles, each multiplied by one workgroup whose four waves split the reduction, i.e.
+// 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
+// The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_mfma_f32_hybrid_kernel(const ConvArgs a)
+{
+    __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
+    __shared__ float red[3][1][16][64];
+    const int bid = blockIdx.x;
+    if (bid < a.n_main)
+    {
+        // n_main is a multiple of NUM_XCD: consecutive logical ids share an XCD
+        const int lid = (bid % NUM_XCD) * (a.n_main / NUM_XCD) + bid / NUM_XCD;
+        conv_lds_tile<COT, PXT>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+        return;
+    }
+    constexpr int SUB = 4 * COT * PXT;            // 32x32 tiles per whole workgroup tile
+    const int j = bid - a.n_main;
+    const int lid = a.n_main + j / SUB;
+    if (lid >= a.n_blocks) return;
+    const int sub = j % SUB;
+    const int co32 = (lid % a.n_co_groups) * COT + sub % COT;
+    const int px32 = (lid / a.n_co_groups) * (4 * PXT) + sub / COT;
+    if (co32 * 32 >= a.Co || px32 * 32 >= a.P) return;     // uniform over the workgroup
+    conv_splitk_tile<1, 1>(a, red, co32, px32);
+}
+
 // ---------------------------------------------------------------------------------------------
 // first layers: Ci in {1,2,3}; input block is [H][W][Ci], filter [Co/16][kh][kw][Ci][16]
 // grid.x over pixels, grid.y = output channel block (uniform per workgroup -> scalar weight loads)
@@ -649,7 +688,15 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
     // SMALL_HIP_CONV_LDS=0 selects the variant that reads the filter operand straight from global memory
     static const bool use_lds = [] { const char *e = std::getenv("SMALL_HIP_CONV_LDS"); return !(e && e[0] == '0'); }();
-    if (use_lds)
+    static const bool use_tail = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return !(e && e[0] == '0'); }();
+    const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
+    if (use_lds && use_tail && rest > 0 && a.kh * a.kw * (a.Ci / CB) >= 8)
+    {
+        a.n_main = n_main;
+        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT), dim3(256),
+                           0, s, a);
+    }
+    else if (use_lds)
         hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
     else
         hipLaunchKernelGGL((conv_mfma_f32_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
@@ -696,15 +743,15 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
         return SMALL_HIP_OK;
     }
 
-    // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X: 2x2 wins only when the
-    // launch has many tiles per SIMD and a long reduction, 2x1 in the middle, 1x1 when the output is
-    // small (few tiles per SIMD: balance matters more than operand re-use).
+    // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X with the balanced tail in
+    // place: 2x2 wins from about 12 tiles per SIMD when the reduction is not trivially short, 2x1
+    // from 3 tiles per SIMD, 1x1 below (few tiles: balance matters more than operand re-use).
     const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32);
     const long simds = 4L * NUM_CU;
     const int nsteps = kh * kw * (Ci / CB);
     int cot = 1, pxt = 1;
-    if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
-    else if (Co % 64 == 0 && tiles32 >= 6 * simds) { cot = 2; pxt = 1; }
+    if (Co % 64 == 0 && tiles32 >= 12 * simds && nsteps >= 8) { cot = 2; pxt = 2; }
+    else if (Co % 64 == 0 && tiles32 >= 3 * simds) { cot = 2; pxt = 1; }
     // few tiles and a long reduction: split K over the four waves of a workgroup
     bool splitk = tiles32 < 2 * simds && nsteps >= 16;
     if (const char *e = std::getenv("SMALL_HIP_CONV_SPLITK")) splitk = e[0] == '1';

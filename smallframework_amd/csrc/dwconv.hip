@@ -2,7 +2,7 @@
 // DepthwiseConv2D (uint8).  Bandwidth-bound, no MFMA: a lane owns four channels of one output
 // pixel, so the four lanes of a (pixel, channel-block) touch one 64-byte line per tap and a wave
 // covers 16 neighbouring output pixels.  Three float32 kernels, picked by shape:
-//   - 3x3 on images of at least 14x14 (28x28 at stride 2) outputs: input tile staged in LDS
+//   - 3x3 on images of at least 7x7 (28x28 at stride 2) outputs: input tile staged in LDS
 //   - other 3x3: a lane loads a strip of rows into registers
 //   - any other window: one output per lane, taps read through the vector cache
 #include "common.h"
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
 
 // tile shapes of the LDS kernel: (TW, R) -> a TW x (64/TW)*R tile of output pixels
 struct TileShape { int tw, th; };
-constexpr TileShape TILE_SHAPES_S1[] = {{16, 16}, {8, 56}, {16, 28}, {32, 8}};
+constexpr TileShape TILE_SHAPES_S1[] = {{16, 16}, {8, 56}, {16, 28}, {32, 8}, {8, 8}};
 constexpr TileShape TILE_SHAPES_S2[] = {{8, 8}, {4, 16}, {16, 4}};
 
 
@@ -347,15 +347,15 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
     {
         constexpr int R1 = 4, R2 = 3;      // output rows per lane at stride 1 / stride 2
         static const bool tile_off = [] { const char *v = std::getenv("SMALL_HIP_DW_TILE"); return v && v[0] == '0'; }();
-        // measured: the strip kernel wins below 14x14 outputs at stride 1 and below 28x28 at stride 2
-        const int min_side = stride == 1 ? 14 : 28;
+        // measured: the strip kernel wins below 7x7 outputs at stride 1 and below 28x28 at stride 2
+        const int min_side = stride == 1 ? 7 : 28;
         if (g.Ho >= min_side && g.Wo >= min_side && !tile_off)
         {
             // the tile shape that wastes the fewest lanes on this image; ties go to the first
             const TileShape *shapes = stride == 1 ? TILE_SHAPES_S1 : TILE_SHAPES_S2;
             int best = -1;
             double best_util = 0.7;        // below that the strip kernel is the better choice
-            const int nshapes = stride == 1 ? 4 : 3;
+            const int nshapes = stride == 1 ? 5 : 3;
             for (int t = 0; t < nshapes; ++t)
             {
                 const int tx = (g.Wo + shapes[t].tw - 1) / shapes[t].tw;
@@ -373,7 +373,8 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 decltype(&dw3x3_f32_tile_kernel<1, 16, 4>) tk;
                 if (stride == 1)
                     tk = best == 0 ? dw3x3_f32_tile_kernel<1, 16, 4> : best == 1 ? dw3x3_f32_tile_kernel<1, 8, 7>
-                       : best == 2 ? dw3x3_f32_tile_kernel<1, 16, 7> : dw3x3_f32_tile_kernel<1, 32, 4>;
+                       : best == 2 ? dw3x3_f32_tile_kernel<1, 16, 7> : best == 3 ? dw3x3_f32_tile_kernel<1, 32, 4>
+                                                                     : dw3x3_f32_tile_kernel<1, 8, 1>;
                 else
                     tk = best == 0 ? dw3x3_f32_tile_kernel<2, 8, 1> : best == 1 ? dw3x3_f32_tile_kernel<2, 4, 1>
                                                                    : dw3x3_f32_tile_kernel<2, 16, 1>;

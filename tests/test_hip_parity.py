@@ -135,6 +135,8 @@ WIN_CASES = [
     (1, 3, 3, 1, (1, 1, 1, 1), 16, 56, 15),
     (1, 3, 3, 1, (1, 1, 1, 1), 16, 23, 63),
     (3, 3, 3, 1, (1, 1, 1, 1), 48, 14, 14),
+    (3, 3, 3, 1, (1, 1, 1, 1), 32, 7, 7),
+    (2, 3, 3, 1, (0, 0, 0, 0), 16, 10, 9),
     # stride 2 through the same kernel: 56x56, 28x28 (4x16 tiles), ragged 8x8 tiles, 28x32 (16x4 tiles); 14x52 stays on the strip kernel
     (1, 3, 3, 2, (0, 1, 0, 1), 16, 112, 112),
     (2, 3, 3, 2, (0, 1, 0, 1), 32, 56, 56),
