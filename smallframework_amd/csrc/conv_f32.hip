@@ -669,6 +669,94 @@ __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
     }
 }
 
+// Ci in {1,2,3} on the matrix cores.  The reduction index k = (tap, ci) is only kh*kw*Ci long
+// (27 for a 3x3 RGB stem) and the filter block [kh][kw][Ci][16] is already a [K][16] matrix, so a
+// K-step of the 32x32x2 MFMA takes k = 2s (lanes 0..31) and k = 2s+1 (lanes 32..63): one dword of
+// the lane's pixel and one filter dword per step, no repacking.  A wave multiplies PXT tiles of
+// 32 pixels by one tile of 32 output channels; the vector ALU only does the address arithmetic.
+// NS = number of K-steps, ceil(kh*kw*Ci / 2), a compile-time bound so that every load of the
+// reduction is issued before the first MFMA.
+template <int CI, int NS, int PXT>
+__global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvArgs a)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int cg = blockIdx.y;                       // tile of 32 output channels
+    const int HoWo = a.Ho * a.Wo;
+    const int CoB = a.Co / CB;
+    const int K = a.kh * a.kw * CI;
+
+    const float *img[PXT];
+    int ih0[PXT], iw0[PXT];
+    bool pvalid[PXT];
+    size_t out_pix[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = ((blockIdx.x * 4 + wave) * PXT + t) * 32 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo;
+        const int rem = pc - n * HoWo;
+        const int oh = rem / a.Wo;
+        const int ow = rem - oh * a.Wo;
+        ih0[t] = oh * a.stride - a.pt;
+        iw0[t] = ow * a.stride - a.pl;
+        img[t] = a.in + (size_t)n * a.H * a.W * CI;
+        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+    }
+    // filter row of this lane: channel co = cg*32 + col, element k at w_row[k * 16]
+    const int co = cg * 32 + col;
+    const bool co_ok = co < a.Co;
+    const int cc = co_ok ? co : a.Co - 1;
+    const float *w_row = a.filt + (size_t)(cc / CB) * K * CB + (cc % CB);
+
+    // position of k = 2s + half inside the window, advanced by two elements per step; the element
+    // offset of a tap relative to the window origin is shared by the PXT tiles (32-bit: one image
+    // holds fewer than 2^31 elements, checked by the launcher)
+    int ci = half % CI, tb = half / CI, ta = 0;
+    if (tb >= a.kw) { tb -= a.kw; ++ta; }          // only Ci == 1 with a one-column window
+    int base[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t) base[t] = (ih0[t] * a.W + iw0[t]) * CI;
+    float av[NS], bv[NS][PXT];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        const int k = 2 * s + half;
+        const bool k_ok = k < K;
+        const float wv = w_row[(k_ok ? k : 0) * CB];
+        av[s] = k_ok && co_ok ? wv : 0.f;
+        const int delta = (ta * a.W + tb) * CI + ci;
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const bool ok = k_ok && pvalid[t] && (unsigned)(ih0[t] + ta) < (unsigned)a.H &&
+                            (unsigned)(iw0[t] + tb) < (unsigned)a.W;
+            const float v = img[t][ok ? base[t] + delta : 0];
+            bv[s][t] = ok ? v : 0.f;
+        }
+        // k += 2, branch-free: Ci <= 3, so ci wraps at most twice (Ci == 1) and tb at most twice
+        if (CI == 1) tb += 2;
+        else if (CI == 2) tb += 1;
+        else { const bool wrap = ci >= 1; ci = wrap ? ci - 1 : 2; tb += wrap ? 1 : 0; }
+        { const bool w1 = tb >= a.kw; tb -= w1 ? a.kw : 0; ta += w1 ? 1 : 0; }
+        if (CI == 1) { const bool w2 = tb >= a.kw; tb -= w2 ? a.kw : 0; ta += w2 ? 1 : 0; }
+    }
+
+    floatx16 acc[1][PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][t][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+            acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s], bv[s][t], acc[0][t], 0, 0, 0);
+    conv_epilogue<1, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+}
+
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
@@ -736,6 +824,22 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     if (small_ci)
     {
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
+        static const bool smallci_valu = [] { const char *e = std::getenv("SMALL_HIP_SMALLCI_VALU"); return e && e[0] == '1'; }();
+        const int nsteps = (kh * kw * Ci + 1) / 2;
+        // measured: with 16 output channels half of every 32-row MFMA tile is idle and the vector-ALU
+        // kernel is faster
+        if (!smallci_valu && Co >= 32 && nsteps <= 20 && (long)H * W * Ci < 0x7fffffffL)
+        {
+            constexpr int PXT = 2;
+            const dim3 gm((unsigned)((a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4)), (unsigned)((Co + 31) / 32));
+            void (*km)(const ConvArgs) = nullptr;
+            if (Ci == 1) km = nsteps <= 5 ? conv_smallci_mfma_f32_kernel<1, 5, PXT> : nsteps <= 14 ? conv_smallci_mfma_f32_kernel<1, 14, PXT> : conv_smallci_mfma_f32_kernel<1, 20, PXT>;
+            else if (Ci == 2) km = nsteps <= 9 ? conv_smallci_mfma_f32_kernel<2, 9, PXT> : conv_smallci_mfma_f32_kernel<2, 20, PXT>;
+            else km = nsteps <= 14 ? conv_smallci_mfma_f32_kernel<3, 14, PXT> : conv_smallci_mfma_f32_kernel<3, 20, PXT>;
+            hipLaunchKernelGGL(km, gm, dim3(256), 0, s, a);
+            SHP_LAUNCH_CHECK(op);
+            return SMALL_HIP_OK;
+        }
         if (Ci == 1) hipLaunchKernelGGL(conv_smallci_f32_kernel<1>, grid, dim3(256), 0, s, a);
         else if (Ci == 2) hipLaunchKernelGGL(conv_smallci_f32_kernel<2>, grid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL(conv_smallci_f32_kernel<3>, grid, dim3(256), 0, s, a);

@@ -48,6 +48,8 @@ CONV_CASES = [
     (2, 3, 3, 2, (0, 1, 0, 1), 32, 3, 16, 16),
     (1, 3, 3, 1, (0, 0, 0, 0), 16, 1, 9, 11),
     (1, 3, 3, 1, (0, 0, 0, 0), 16, 2, 9, 11),
+    (1, 3, 3, 1, (1, 1, 1, 1), 64, 2, 9, 11),
+    (2, 3, 3, 2, (0, 1, 0, 1), 48, 1, 16, 16),
     (2, 10, 4, 2, (4, 5, 1, 1), 64, 1, 49, 10),   # DS-CNN stem: >= 2 padded rows per side
 ]
 
