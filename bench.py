@@ -26,9 +26,9 @@ PEAK_MFMA_I8 = 5.0e15      # OP/s, dense int8 MFMA
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (two runs) over this same benchmark and scaled by what the counters read for an
-# in-place ReLU of known size (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); the summary is
+# in-place ReLU of 822 MB (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); the summary is
 # profiles/mobilenet_v1_b64_traffic_and_mfma.md.  Keyed by (model, batch, kernel family).
-MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_kernel"): 94.3}
+MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_*"): 94.5}
 
 
 def log(*a):
@@ -139,13 +139,50 @@ def cpu_port_u8(model, batch=8):
             "sample": "%d images x %d passes of %s on the scalar C restatement" % (batch, reps, model.name)}
 
 
+def sweep_only(args, torch, models):
+    """--model layer_sweep: the four single layers at C = 256, 56x56 (Conv2D 3x3, DepthwiseConv2D 3x3,
+    MaxPool2D 3x3 stride 2, ReLU), each run `steps` times at --batch (default 64).  The JSON line is
+    about the Conv2D layer; the others are in "layers"."""
+    batch = args.batch or 64
+    rows, head = [], None
+    for m in models.layer_sweep():
+        ex = models.HipExecutor(m, batch)
+        sec = time_forward(ex, args.steps, args.warmup)
+        ms = time_ops(ex, args.steps)
+        r = layer_table(m, batch, ms)[0]
+        r["layer"] = m.name
+        r["images_per_s"] = round(batch / (r["ms"] * 1e-3), 1)
+        rows.append(r)
+        log("%-20s batch %d: %.4f ms  %.0f images/s  %s %.1f%% of roofline" % (
+            m.name, batch, r["ms"], r["images_per_s"], r["bound"], 100 * (r["roofline_frac"] or 0)))
+        if head is None:
+            head = (m, sec, r)
+        del ex
+        torch.cuda.empty_cache()
+    m, sec, r = head
+    op = m.ops[0]
+    out = {"metric": "images/s @batch%d %s fp32" % (batch, m.name), "value": round(batch / sec, 2),
+           "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "single layers at C=256, 56x56, batch %d: Conv2D 3x3 s1 same, DepthwiseConv2D "
+                                  "3x3 s1, MaxPool2D 3x3 s2 valid, ReLU" % batch, "batch": batch},
+           "roofline": {"bound": "mfma", "achieved": r["TFLOP/s"], "peak": round(PEAK_MFMA_F32 / 1e12, 1),
+                        "unit": "TFLOP/s", "frac": r["roofline_frac"], "traffic": None,
+                        "kernel": "conv_mfma_f32_*", "launches_per_step": 1, "avg_launch_ms": r["ms"],
+                        "algorithmic_per_launch": {"GFLOP": round(batch * op.flops() / 1e9, 3),
+                                                   "MB": round(op_bytes(m, op, batch) / 1e6, 3)}},
+           "cpu_baseline": None, "layers": rows}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--model", default="mobilenet_v1",
-                    choices=["mobilenet_v1", "resnet8_u8", "tiny_yolo_v2", "dscnn"])
+                    choices=["mobilenet_v1", "resnet8_u8", "tiny_yolo_v2", "dscnn", "layer_sweep"])
     ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="headline model only")
@@ -162,6 +199,8 @@ def main():
         log("bench.py: no GPU visible")
         sys.exit(1)
     capi.load()
+    if args.model == "layer_sweep":
+        return sweep_only(args, torch, models)
     default_batch = {"mobilenet_v1": 64, "resnet8_u8": 64, "tiny_yolo_v2": 16, "dscnn": 64}
     batch = args.batch or default_batch[args.model]
     model = getattr(models, args.model)()
@@ -185,7 +224,7 @@ def main():
         if op.kind in ("conv", "dense"):
             if op.C % 16 != 0:
                 return "conv_smallci_%s_kernel" % model.dtype
-            return "conv_mfma_%s_kernel" % model.dtype
+            return "conv_mfma_%s_*" % model.dtype
         return {"dw": "dw_%s_kernel" % model.dtype, "maxpool": "pool_%s_kernel" % model.dtype,
                 "avgpool": "pool_%s_kernel" % model.dtype}.get(op.kind, "ew_%s_kernel" % model.dtype)
 
@@ -242,6 +281,27 @@ def main():
                 % (name, b, s2 * 1e3, b / s2, s3 * 1e3, b / s3))
             del e2
         torch.cuda.empty_cache()
+        # the other float32 configurations: whole models and the single-layer sweep at C = 256, 56x56
+        others = [(models.tiny_yolo_v2(), 16), (models.dscnn(), 1), (models.dscnn(), 64)]
+        others += [(m, b) for b in (1, 64) for m in models.layer_sweep()]
+        for m2, b in others:
+            e2 = models.HipExecutor(m2, b)
+            s2 = time_forward(e2, args.steps, args.warmup)
+            ms2 = time_ops(e2, 10)
+            tab = layer_table(m2, b, ms2)
+            extras["%s_b%d" % (m2.name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
+                                               "layers": tab}
+            if len(m2.ops) == 1:
+                log("%-20s batch %2d: %.4f ms  %.0f images/s  %s %.1f%% of roofline" % (
+                    m2.name, b, tab[0]["ms"], b / (tab[0]["ms"] * 1e-3), tab[0]["bound"],
+                    100 * (tab[0]["roofline_frac"] or 0)))
+            else:
+                log("%s batch %d: %.4f ms/step %.0f images/s" % (m2.name, b, s2 * 1e3, b / s2))
+                for r in tab:
+                    log("  %-28s %9.4f ms  %-4s %6.1f%%" % (r["layer"], r["ms"], r["bound"],
+                                                           100 * (r["roofline_frac"] or 0)))
+            del e2
+            torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:

@@ -363,6 +363,7 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 const double util = (double)g.Wo * g.Ho / ((double)tx * shapes[t].tw * ty * shapes[t].th);
                 if (util > best_util + 1e-9) { best_util = util; best = t; }
             }
+            if (const char *v = std::getenv("SMALL_HIP_DW_SHAPE")) best = std::atoi(v);
             if (best >= 0)
             {
                 const int tiles_x = (g.Wo + shapes[best].tw - 1) / shapes[best].tw;
