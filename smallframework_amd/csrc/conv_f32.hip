@@ -60,6 +60,11 @@ struct ConvArgs
     int n_main;          // hybrid kernel: workgroups that run whole tiles (multiple of the CU count)
 };
 
+// 64 bytes of zeros.  A masked tap (padding, a pixel past the end, a step past the last) loads from
+// here instead of being zeroed after the load: a select on the loaded value sits in the step that
+// issued the load and makes the wave wait for data it only needs a step later.
+__device__ __align__(64) float g_zero_block[CB];
+
 __device__ __forceinline__ float act1(float v, int act, float slope)
 {
     if (act == SMALL_HIP_ACT_RELU) return v > 0.f ? v : 0.f;
@@ -128,6 +133,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
     const int CoB = a.Co / CB;
     const int taps = a.kh * a.kw;
     const size_t in_blk = (size_t)a.H * a.W * CB;     // floats per input channel block
+    const float *zero_half = g_zero_block + half * 8;
 
     // ---- per-lane pixel columns --------------------------------------------------------
     const float *in_img[PXT];   // image base + half offset
@@ -183,12 +189,10 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
             const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
-            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
-            float4 v0 = p[0], v1 = p[1];
-            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
-            B[t][0] = v0;
-            B[t][1] = v1;
+            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
+            const float4 *p = reinterpret_cast<const float4 *>(ok ? in_img[t] + off : zero_half);
+            B[t][0] = p[0];
+            B[t][1] = p[1];
         }
 #pragma unroll
         for (int c = 0; c < COT; ++c)
@@ -266,6 +270,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     const int CoB = a.Co / CB;
     const int taps = a.kh * a.kw;
     const size_t in_blk = (size_t)a.H * a.W * CB;
+    const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
     int ih0[PXT], iw0[PXT];
@@ -290,15 +295,17 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // ---- cooperative filter fetch: COT*2 tiles of 64 float4 each -----------------------------
     constexpr int A_VECS = COT * 2 * 64;                 // float4 per step and workgroup
     constexpr int A_PER_THREAD = (A_VECS + 255) / 256;   // 1 for COT <= 2, 2 for COT == 4
+    // Every thread loads and stores (no predicate): with fewer vectors than threads (COT == 1) the
+    // upper threads repeat a lower thread's vector and write the same value to the same place.  A
+    // predicated load would put the wait of the staging store inside a branch, and the compiler
+    // would then have to wait at the top of the loop for loads issued only a step earlier.
+    static_assert(A_VECS >= 256 ? A_VECS % 256 == 0 : 256 % A_VECS == 0, "filter vectors vs workgroup size");
     const float *a_src[A_PER_THREAD];
     int a_dst[A_PER_THREAD];
-    bool a_on[A_PER_THREAD];
 #pragma unroll
     for (int j = 0; j < A_PER_THREAD; ++j)
     {
-        const int v = tid + j * 256;
-        a_on[j] = v < A_VECS;
-        const int vc = a_on[j] ? v : 0;
+        const int vc = (tid + j * 256) % A_VECS;
         const int blk = vc >> 6, within = vc & 63;
         int cob = cg * COT * 2 + blk;
         cob = cob < CoB ? cob : CoB - 1;                  // rows past Co: garbage, never stored
@@ -325,22 +332,21 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // issues the global loads of the step at (ta, tb, cib) and advances the position
     auto fetch = [&](float4 (&Areg)[A_PER_THREAD], float4 (&B)[PXT][2]) {
         const int tap = ta * a.kw + tb;
+        // filter first: its staging store is the first consumer, so it can wait for these loads
+        // alone and leave the activation loads of the same step in flight
+        const size_t woff = ((size_t)cib * taps + tap) * (CB * CB);
+#pragma unroll
+        for (int j = 0; j < A_PER_THREAD; ++j) Areg[j] = *reinterpret_cast<const float4 *>(a_src[j] + woff);
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
             const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
-            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
-            float4 v0 = p[0], v1 = p[1];
-            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
-            B[t][0] = v0;
-            B[t][1] = v1;
+            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
+            const float4 *p = reinterpret_cast<const float4 *>(ok ? in_img[t] + off : zero_half);
+            B[t][0] = p[0];
+            B[t][1] = p[1];
         }
-        const size_t woff = ((size_t)cib * taps + tap) * (CB * CB);
-#pragma unroll
-        for (int j = 0; j < A_PER_THREAD; ++j)
-            if (a_on[j]) Areg[j] = *reinterpret_cast<const float4 *>(a_src[j] + woff);
         int ncib = cib + 1, ntb = tb, nta = ta;
         if (ncib == CiB)
         {
@@ -352,8 +358,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     };
     auto stage = [&](int buf, const float4 (&Areg)[A_PER_THREAD]) {
 #pragma unroll
-        for (int j = 0; j < A_PER_THREAD; ++j)
-            if (a_on[j]) *reinterpret_cast<float4 *>(&lds_a[buf][a_dst[j]]) = Areg[j];
+        for (int j = 0; j < A_PER_THREAD; ++j) *reinterpret_cast<float4 *>(&lds_a[buf][a_dst[j]]) = Areg[j];
     };
     auto multiply = [&](int buf, const float4 (&B)[PXT][2]) {
         float A[COT][8];
@@ -428,6 +433,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     const int CoB = a.Co / CB;
     const int taps = a.kh * a.kw;
     const size_t in_blk = (size_t)a.H * a.W * CB;
+    const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
     int ih0[PXT], iw0[PXT];
@@ -484,12 +490,10 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
             const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
-            const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + off);
-            float4 v0 = p[0], v1 = p[1];
-            if (!ok) { v0 = make_float4(0.f, 0.f, 0.f, 0.f); v1 = v0; }
-            B[t][0] = v0;
-            B[t][1] = v1;
+            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
+            const float4 *p = reinterpret_cast<const float4 *>(ok ? in_img[t] + off : zero_half);
+            B[t][0] = p[0];
+            B[t][1] = p[1];
         }
 #pragma unroll
         for (int c = 0; c < COT; ++c)
@@ -847,14 +851,15 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
         return SMALL_HIP_OK;
     }
 
-    // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X with the balanced tail in
-    // place: 2x2 wins from about 12 tiles per SIMD when the reduction is not trivially short, 2x1
-    // from 3 tiles per SIMD, 1x1 below (few tiles: balance matters more than operand re-use).
+    // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X inside whole-model runs with
+    // the balanced tail in place: 2x2 only pays with many tiles per SIMD and a long reduction (big
+    // 3x3 layers), 2x1 from 3 tiles per SIMD, 1x1 below (few tiles: balance matters more than
+    // operand re-use).
     const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32);
     const long simds = 4L * NUM_CU;
     const int nsteps = kh * kw * (Ci / CB);
     int cot = 1, pxt = 1;
-    if (Co % 64 == 0 && tiles32 >= 12 * simds && nsteps >= 8) { cot = 2; pxt = 2; }
+    if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
     else if (Co % 64 == 0 && tiles32 >= 3 * simds) { cot = 2; pxt = 1; }
     // few tiles and a long reduction: split K over the four waves of a workgroup
     bool splitk = tiles32 < 2 * simds && nsteps >= 16;
