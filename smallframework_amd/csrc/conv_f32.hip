@@ -673,25 +673,51 @@ __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
     }
 }
 
-// Ci in {1,2,3} on the matrix cores.  The reduction index k = (tap, ci) is only kh*kw*Ci long
-// (27 for a 3x3 RGB stem) and the filter block [kh][kw][Ci][16] is already a [K][16] matrix, so a
-// K-step of the 32x32x2 MFMA takes k = 2s (lanes 0..31) and k = 2s+1 (lanes 32..63): one dword of
-// the lane's pixel and one filter dword per step, no repacking.  A wave multiplies PXT tiles of
-// 32 pixels by one tile of 32 output channels; the vector ALU only does the address arithmetic.
-// NS = number of K-steps, ceil(kh*kw*Ci / 2), a compile-time bound so that every load of the
-// reduction is issued before the first MFMA.
-template <int CI, int NS, int PXT>
+// Ci in {1,2,3} on the matrix cores.  The reduction index (tap, ci) is only kh*kw*Ci long (27 for
+// a 3x3 RGB stem) and the filter block [kh][kw][Ci][16] is already a [K][16] matrix, so a K-step
+// of the 32x32x2 MFMA takes one reduction element in lanes 0..31 and another in lanes 32..63: one
+// input dword and one filter dword per lane and step, no repacking.  The order of the reduction is
+// free, and it is chosen so that every step's window positions are compile-time constants:
+//   Ci == 2: step s = tap s, the wave halves take ci 0 / 1
+//   Ci == 3: steps 0..taps-1 the same with ci 0 / 1, then ci 2 of taps 2j / 2j+1 in step taps+j
+//   Ci == 1: step s = taps 2s / 2s+1
+// Row and column validity of the window is computed once per pixel; every load is issued before the
+// first MFMA, masked positions load from the zero block.  A wave multiplies PXT tiles of 32 pixels
+// by one tile of 32 output channels.
+template <int CI, int KH, int KW>
+struct SmallCiSteps
+{
+    static constexpr int TAPS = KH * KW;
+    static constexpr int NS = CI == 1 ? (TAPS + 1) / 2 : CI == 2 ? TAPS : TAPS + (TAPS + 1) / 2;
+    // window tap and channel of (step, wave half); tap == TAPS means "nothing" (contributes zero)
+    static constexpr int tap(int s, int h)
+    {
+        if (CI == 1) return 2 * s + h < TAPS ? 2 * s + h : TAPS;
+        if (CI == 2) return s;
+        if (s < TAPS) return s;
+        return 2 * (s - TAPS) + h < TAPS ? 2 * (s - TAPS) + h : TAPS;
+    }
+    static constexpr int ci(int s, int h)
+    {
+        if (CI == 1) return 0;
+        if (CI == 2) return h;
+        return s < TAPS ? h : 2;
+    }
+};
+
+template <int CI, int KH, int KW, int PXT>
 __global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvArgs a)
 {
+    using St = SmallCiSteps<CI, KH, KW>;
+    constexpr int NS = St::NS, TAPS = St::TAPS;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 31, half = lane >> 5;
     const int cg = blockIdx.y;                       // tile of 32 output channels
     const int HoWo = a.Ho * a.Wo;
     const int CoB = a.Co / CB;
-    const int K = a.kh * a.kw * CI;
 
-    const float *img[PXT];
-    int ih0[PXT], iw0[PXT];
+    const float *img[PXT];                           // window origin of the lane's pixel (may lie outside)
+    bool rowok[PXT][KH], colok[PXT][KW];
     bool pvalid[PXT];
     size_t out_pix[PXT];
 #pragma unroll
@@ -704,48 +730,42 @@ __global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvAr
         const int rem = pc - n * HoWo;
         const int oh = rem / a.Wo;
         const int ow = rem - oh * a.Wo;
-        ih0[t] = oh * a.stride - a.pt;
-        iw0[t] = ow * a.stride - a.pl;
-        img[t] = a.in + (size_t)n * a.H * a.W * CI;
+        const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+#pragma unroll
+        for (int r = 0; r < KH; ++r) rowok[t][r] = pvalid[t] && (unsigned)(ih0 + r) < (unsigned)a.H;
+#pragma unroll
+        for (int c = 0; c < KW; ++c) colok[t][c] = (unsigned)(iw0 + c) < (unsigned)a.W;
+        // 32-bit element offsets inside one image (the launcher checks H*W*Ci < 2^31)
+        img[t] = a.in + (size_t)n * a.H * a.W * CI + (ih0 * a.W + iw0) * CI;
         out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
     }
-    // filter row of this lane: channel co = cg*32 + col, element k at w_row[k * 16]
+    // filter row of this lane: channel co = cg*32 + col, reduction element k at w_row[k * 16]
     const int co = cg * 32 + col;
     const bool co_ok = co < a.Co;
     const int cc = co_ok ? co : a.Co - 1;
-    const float *w_row = a.filt + (size_t)(cc / CB) * K * CB + (cc % CB);
+    const float *w_row = a.filt + (size_t)(cc / CB) * (TAPS * CI) * CB + (cc % CB);
 
-    // position of k = 2s + half inside the window, advanced by two elements per step; the element
-    // offset of a tap relative to the window origin is shared by the PXT tiles (32-bit: one image
-    // holds fewer than 2^31 elements, checked by the launcher)
-    int ci = half % CI, tb = half / CI, ta = 0;
-    if (tb >= a.kw) { tb -= a.kw; ++ta; }          // only Ci == 1 with a one-column window
-    int base[PXT];
-#pragma unroll
-    for (int t = 0; t < PXT; ++t) base[t] = (ih0[t] * a.W + iw0[t]) * CI;
     float av[NS], bv[NS][PXT];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        const int k = 2 * s + half;
-        const bool k_ok = k < K;
-        const float wv = w_row[(k_ok ? k : 0) * CB];
-        av[s] = k_ok && co_ok ? wv : 0.f;
-        const int delta = (ta * a.W + tb) * CI + ci;
+        const int t0 = St::tap(s, 0), t1 = St::tap(s, 1);
+        const int c0 = St::ci(s, 0), c1 = St::ci(s, 1);
+        const bool e0 = t0 < TAPS, e1 = t1 < TAPS;       // compile-time after unrolling
+        const int k0 = e0 ? t0 * CI + c0 : 0, k1 = e1 ? t1 * CI + c1 : 0;
+        const bool exists = half ? e1 : e0;
+        const float *wp = exists && co_ok ? w_row + (half ? k1 : k0) * CB : g_zero_block;
+        av[s] = *wp;
+        const int r0 = e0 ? t0 / KW : 0, q0 = e0 ? t0 % KW : 0;
+        const int r1 = e1 ? t1 / KW : 0, q1 = e1 ? t1 % KW : 0;
+        const int d0 = (r0 * a.W + q0) * CI + c0, d1 = (r1 * a.W + q1) * CI + c1;
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
-            const bool ok = k_ok && pvalid[t] && (unsigned)(ih0[t] + ta) < (unsigned)a.H &&
-                            (unsigned)(iw0[t] + tb) < (unsigned)a.W;
-            const float v = img[t][ok ? base[t] + delta : 0];
-            bv[s][t] = ok ? v : 0.f;
+            const bool ok = half ? (e1 && rowok[t][r1] && colok[t][q1]) : (e0 && rowok[t][r0] && colok[t][q0]);
+            const float *bp = ok ? img[t] + (half ? d1 : d0) : g_zero_block;
+            bv[s][t] = *bp;
         }
-        // k += 2, branch-free: Ci <= 3, so ci wraps at most twice (Ci == 1) and tb at most twice
-        if (CI == 1) tb += 2;
-        else if (CI == 2) tb += 1;
-        else { const bool wrap = ci >= 1; ci = wrap ? ci - 1 : 2; tb += wrap ? 1 : 0; }
-        { const bool w1 = tb >= a.kw; tb -= w1 ? a.kw : 0; ta += w1 ? 1 : 0; }
-        if (CI == 1) { const bool w2 = tb >= a.kw; tb -= w2 ? a.kw : 0; ta += w2 ? 1 : 0; }
     }
 
     floatx16 acc[1][PXT];
@@ -829,20 +849,24 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     {
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
         static const bool smallci_valu = [] { const char *e = std::getenv("SMALL_HIP_SMALLCI_VALU"); return e && e[0] == '1'; }();
-        const int nsteps = (kh * kw * Ci + 1) / 2;
         // measured: with 16 output channels half of every 32-row MFMA tile is idle and the vector-ALU
         // kernel is faster
-        if (!smallci_valu && Co >= 32 && nsteps <= 20 && (long)H * W * Ci < 0x7fffffffL)
+        if (!smallci_valu && Co >= 32 && (long)H * W * Ci < 0x7fffffffL)
         {
             constexpr int PXT = 2;
             const dim3 gm((unsigned)((a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4)), (unsigned)((Co + 31) / 32));
             void (*km)(const ConvArgs) = nullptr;
-            if (Ci == 1) km = nsteps <= 5 ? conv_smallci_mfma_f32_kernel<1, 5, PXT> : nsteps <= 14 ? conv_smallci_mfma_f32_kernel<1, 14, PXT> : conv_smallci_mfma_f32_kernel<1, 20, PXT>;
-            else if (Ci == 2) km = nsteps <= 9 ? conv_smallci_mfma_f32_kernel<2, 9, PXT> : conv_smallci_mfma_f32_kernel<2, 20, PXT>;
-            else km = nsteps <= 14 ? conv_smallci_mfma_f32_kernel<3, 14, PXT> : conv_smallci_mfma_f32_kernel<3, 20, PXT>;
-            hipLaunchKernelGGL(km, gm, dim3(256), 0, s, a);
-            SHP_LAUNCH_CHECK(op);
-            return SMALL_HIP_OK;
+            if (kh == 3 && kw == 3)
+                km = Ci == 1 ? conv_smallci_mfma_f32_kernel<1, 3, 3, PXT> : Ci == 2 ? conv_smallci_mfma_f32_kernel<2, 3, 3, PXT>
+                                                                           : conv_smallci_mfma_f32_kernel<3, 3, 3, PXT>;
+            else if (kh == 10 && kw == 4 && Ci == 1)          // the keyword-spotting stem
+                km = conv_smallci_mfma_f32_kernel<1, 10, 4, PXT>;
+            if (km)
+            {
+                hipLaunchKernelGGL(km, gm, dim3(256), 0, s, a);
+                SHP_LAUNCH_CHECK(op);
+                return SMALL_HIP_OK;
+            }
         }
         if (Ci == 1) hipLaunchKernelGGL(conv_smallci_f32_kernel<1>, grid, dim3(256), 0, s, a);
         else if (Ci == 2) hipLaunchKernelGGL(conv_smallci_f32_kernel<2>, grid, dim3(256), 0, s, a);
