@@ -35,6 +35,8 @@
 #include "common.h"
 #include "quant.h"
 
+#include <cstdlib>
+
 using namespace shp;
 
 namespace
@@ -110,6 +112,11 @@ __global__ __launch_bounds__(256) void wprefix_u8_kernel(const uint8_t *__restri
 }
 
 // ---- main kernel --------------------------------------------------------------------------------
+// 16 bytes of 0x80, the re-biased zero: masked taps load from here instead of being patched after
+// the load (a select on the loaded value would make the wave wait for the data where it was issued)
+__device__ __align__(16) uint8_t g_bias_block[16] = {0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80,
+                                                    0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80};
+
 template <int COT, int PXT>
 __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
 {
@@ -166,8 +173,14 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
 #pragma unroll
         for (int t = 0; t < PXT; ++t) acc[c][t] = v4i{0, 0, 0, 0};
 
-    for (int s0 = 0; s0 < a.S_pad; s0 += 4)
-    {
+    // Software pipeline of depth D over the K loop (4 K-steps per iteration, one per 16-lane group):
+    // the loads of iteration i+D are issued right after iteration i has been multiplied, so D
+    // iterations' worth of loads are always in flight.  These layers are small and latency-bound:
+    // without it every iteration paid a full memory round trip.  Branch-free: iterations past the
+    // end load the 0x80 block (re-biased zero, contributes nothing to the product or to sumI).
+    constexpr int D = 3;
+    uint4 Bq[D][PXT], Wq[D][COT];
+    auto load = [&](int s0, uint4 (&Bv)[PXT], uint4 (&Wv)[COT]) {
         const int s = s0 + grp;
         const bool svalid = s < a.S;
         const int sc = svalid ? s : 0;
@@ -175,15 +188,24 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
         const int cib = sc - tap * CiB;
         const int ta = tap / a.kw;
         const int tb = tap - ta * a.kw;
-        v4i B[PXT];
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
             const bool ok = svalid && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = ok ? ((size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB) : 0;
-            uint4 v = *reinterpret_cast<const uint4 *>(in_img[t] + off);
-            if (!ok) v = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
+            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
+            Bv[t] = *reinterpret_cast<const uint4 *>(ok ? in_img[t] + off : g_bias_block);
+        }
+        const int sw = s < a.S_pad ? s : 0;          // past the end: any valid filter step (B is zero)
+#pragma unroll
+        for (int c = 0; c < COT; ++c) Wv[c] = *reinterpret_cast<const uint4 *>(w_row[c] + (size_t)sw * 256);
+    };
+    auto consume = [&](const uint4 (&Bv)[PXT], const uint4 (&Wv)[COT]) {
+        v4i B[PXT];
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const uint4 v = Bv[t];
             // sum of the 16 raw bytes minus 16*128 = sum of the signed bytes (0 for masked taps)
             uint32_t sb = __builtin_amdgcn_sad_u8(v.x, 0u, 0u);
             sb = __builtin_amdgcn_sad_u8(v.y, 0u, sb);
@@ -196,11 +218,21 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
 #pragma unroll
         for (int c = 0; c < COT; ++c)
         {
-            const uint4 w = *reinterpret_cast<const uint4 *>(w_row[c] + (size_t)s * 256);
-            const v4i A = v4i{(int)w.x, (int)w.y, (int)w.z, (int)w.w};
+            const v4i A = v4i{(int)Wv[c].x, (int)Wv[c].y, (int)Wv[c].z, (int)Wv[c].w};
 #pragma unroll
             for (int t = 0; t < PXT; ++t)
                 acc[c][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B[t], acc[c][t], 0, 0, 0);
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load(4 * d, Bq[d], Wq[d]);
+    for (int s0 = 0; s0 < a.S_pad; s0 += 4 * D)
+    {
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+        {
+            consume(Bq[d], Wq[d]);
+            load(s0 + 4 * (d + D), Bq[d], Wq[d]);
         }
     }
 
@@ -279,7 +311,10 @@ struct QSmallArgs
     QOut q;
 };
 
-template <int CI>
+// M24: both zero points are small enough (|z| < 2^22) that (byte + z) fits 24 signed bits; the
+// products then use the full-rate 24-bit multiply-add (its low 32 bits equal those of the 32-bit
+// wrap-around product), four times the rate of the 32-bit integer multiply.
+template <int CI, bool M24>
 __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a)
 {
     const int p = blockIdx.x * 256 + threadIdx.x;
@@ -309,9 +344,14 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
 #pragma unroll
             for (int ci = 0; ci < CI; ++ci)
             {
-                const uint32_t x = (uint32_t)((int32_t)ip[ci] + a.zi);
+                const int32_t xs = (int32_t)ip[ci] + a.zi;
 #pragma unroll
-                for (int j = 0; j < CB; ++j) acc[j] += x * (uint32_t)((int32_t)wp[ci * CB + j] + a.zf);
+                for (int j = 0; j < CB; ++j)
+                {
+                    const int32_t ws = (int32_t)wp[ci * CB + j] + a.zf;
+                    if (M24) acc[j] += (uint32_t)__mul24(xs, ws);
+                    else acc[j] += (uint32_t)xs * (uint32_t)ws;
+                }
             }
         }
     }
@@ -424,9 +464,15 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     a.P = (int)P;
     const int CoB = Co / CB;
-    if (CoB >= 4 && CoB % 4 == 0) launch_q<4, 2>(a, s);
-    else if (CoB % 2 == 0) launch_q<2, 2>(a, s);
-    else launch_q<1, 2>(a, s);
+    // The largest wave tile (COT channel blocks x PXT pixel groups of 16) that still leaves at least
+    // `want` workgroups: these layers are small and latency-bound, so filling the chip with waves
+    // comes before operand re-use.
+    static const long want = [] { const char *e = std::getenv("SMALL_HIP_CONVQ_MIN_WG"); return e ? std::atol(e) : 512L; }();
+    auto nwg = [&](int cot, int pxt) { return (long)((CoB + cot - 1) / cot) * ((P + 64 * pxt - 1) / (64 * pxt)); };
+    if (CoB % 4 == 0 && nwg(4, 2) >= want) launch_q<4, 2>(a, s);
+    else if (CoB % 2 == 0 && nwg(2, 2) >= want) launch_q<2, 2>(a, s);
+    else if (nwg(1, 2) >= want) launch_q<1, 2>(a, s);
+    else launch_q<1, 1>(a, s);
     SHP_LAUNCH_CHECK(op);
     return SMALL_HIP_OK;
 }
@@ -454,9 +500,11 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
         a.P = (int)P;
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
-        if (Ci == 1) hipLaunchKernelGGL(conv_smallci_u8_kernel<1>, grid, dim3(256), 0, s, a);
-        else if (Ci == 2) hipLaunchKernelGGL(conv_smallci_u8_kernel<2>, grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL(conv_smallci_u8_kernel<3>, grid, dim3(256), 0, s, a);
+        void (*k)(const QSmallArgs) = nullptr;
+        const auto small = [](int32_t z) { return z > -(1 << 22) && z < (1 << 22); };
+        if (small(a.zi) && small(a.zf)) k = Ci == 1 ? conv_smallci_u8_kernel<1, true> : Ci == 2 ? conv_smallci_u8_kernel<2, true> : conv_smallci_u8_kernel<3, true>;
+        else k = Ci == 1 ? conv_smallci_u8_kernel<1, false> : Ci == 2 ? conv_smallci_u8_kernel<2, false> : conv_smallci_u8_kernel<3, false>;
+        hipLaunchKernelGGL(k, grid, dim3(256), 0, s, a);
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }

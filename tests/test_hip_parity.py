@@ -349,6 +349,8 @@ QPARAMS = [
     (100, 156, (1 << 31) - 1, 0, 15),
     (-3, 5, 1234567890, 1, 4),
     (-120, -131, 2000000000, 0, 0),
+    # zero points beyond 24 bits: int32 wrap-around arithmetic, the 32-bit multiply path of the stem kernel
+    (-(1 << 24) - 77, (1 << 23) + 5, 1518500250, 0, 3),
 ]
 
 
