@@ -96,30 +96,48 @@ def layer_table(model, batch, ms):
     return rows
 
 
-def cpu_reference_mobilenet(model, weights, x_one, budget_s=12.0):
-    """The reference's own ZEN2 build (AVX2 + OpenMP) on this host: images/s, batch-1 calls."""
-    from oracle.binding import have_ref
-    if not have_ref("ZEN2"):
-        return None
-    from oracle.model_exec import RefExecutor
+def cpu_threads():
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     threads = min(threads, os.cpu_count() or threads)
     os.environ["OMP_NUM_THREADS"] = str(threads)
+    return threads
+
+
+def cpu_reference_model(model, weights, x_one, budget_s=12.0, max_passes=64):
+    """The reference's own ZEN2 build (AVX2 + OpenMP) on this host, batch-1 calls.
+    -> (cpu_baseline object, per-layer mean milliseconds per image)."""
+    from oracle.binding import have_ref
+    if not have_ref("ZEN2"):
+        return None, None
+    from oracle.model_exec import RefExecutor
+    threads = cpu_threads()
     ex = RefExecutor(model, weights, x_one, "ZEN2")
     ex.forward()                     # warm-up (the reference's protocol: 1 warm-up call)
+    per_op = [0.0] * len(model.ops)
     t0 = time.perf_counter()
     n = 0
     ts = []
-    while n < 64 and (time.perf_counter() - t0) < budget_s:
+    while n < max_passes and (time.perf_counter() - t0) < budget_s:
         t1 = time.perf_counter()
-        ex.forward()
+        ex.forward(per_op)
         ts.append(time.perf_counter() - t1)
         n += 1
     mean = sum(ts) / len(ts)
-    return {"value": round(1.0 / mean, 2), "unit": "images/s", "cores": threads, "kind": "reference",
+    base = {"value": round(1.0 / mean, 2), "unit": "images/s", "cores": threads, "kind": "reference",
             "sample": "%d batch-1 forward passes of %s (all layers, unfused Conv2D+ReLU as the reference's "
                       "Layer classes issue them) on the reference's ZEN2 build, 1 warm-up; min %.2f ms mean %.2f ms"
                       % (n, model.name, 1e3 * min(ts), 1e3 * mean)}
+    return base, [1e3 * t / n for t in per_op]
+
+
+def add_cpu_column(table, cpu_ms, batch):
+    """Per layer: the reference CPU build's milliseconds per image and the GPU/CPU throughput ratio."""
+    if cpu_ms is None:
+        return
+    for row, c in zip(table, cpu_ms):
+        row["cpu_ref_ms_per_image"] = round(c, 4)
+        if row.get("ms"):
+            row["gpu_over_cpu"] = round(c / (row["ms"] / batch), 1)
 
 
 def cpu_port_u8(model, batch=8):
@@ -306,13 +324,25 @@ def main():
     cpu = None
     if not args.no_cpu:
         try:
-            if model.dtype == "f32":
+            if model.dtype == "f32" and model.name != "dscnn":   # the reference cannot run the 10x4 stem
                 x1 = models.make_input(model, 1)
-                cpu = cpu_reference_mobilenet(model, weights, x1)
+                cpu, cpu_ms = cpu_reference_model(model, weights, x1)
+                add_cpu_column(table, cpu_ms, batch)
             if cpu is None:
                 cpu = cpu_port_u8(model) if model.dtype == "u8" else None
             if not args.no_extras and args.model == "mobilenet_v1":
                 extras["resnet8_u8_cpu"] = cpu_port_u8(models.resnet8_u8())
+                # reference CPU build beside the other float32 configurations (bounded samples)
+                for m2 in [models.tiny_yolo_v2()] + models.layer_sweep():
+                    w2 = models.make_weights(m2)
+                    c2, ms2 = cpu_reference_model(m2, w2, models.make_input(m2, 1), budget_s=3.0, max_passes=8)
+                    if c2 is None:
+                        continue
+                    extras["%s_cpu" % m2.name] = c2
+                    for key, e in extras.items():
+                        if key.startswith(m2.name + "_b") and "layers" in e:
+                            add_cpu_column(e["layers"], ms2, int(key.rsplit("_b", 1)[1]))
+                    log("%s on the reference ZEN2 build, %d threads: %.2f images/s" % (m2.name, c2["cores"], c2["value"]))
         except Exception as e:            # the baseline leg must not take the GPU numbers down
             log("cpu baseline failed: %r" % (e,))
 

@@ -110,9 +110,12 @@ class RefExecutor:
             if op.act == "leaky" or op.kind == "leaky":
                 self.slopes[op.slope] = self.ref.fbuf(1, np.float32([op.slope]))
 
-    def forward(self):
+    def forward(self, op_seconds=None):
+        """One forward pass; op_seconds (a list with one slot per op) accumulates each layer's wall
+        time including its activation call."""
         L, buf, w = self.ref.lib, self.buf, self.w
-        for op in self.model.ops:
+        for i, op in enumerate(self.model.ops):
+            t0 = time.perf_counter()
             t, b, l, r = op.pads
             s, d = buf[op.src].h, buf[op.dst].h
             if op.kind == "conv":
@@ -141,6 +144,8 @@ class RefExecutor:
                 else:
                     rc = L.sref_leaky_relu_f32(c, h, wd, d, self.slopes[op.slope].h, d)
                 assert rc == 0, (op.name, self.ref.err())
+            if op_seconds is not None:
+                op_seconds[i] += time.perf_counter() - t0
 
     def output(self):
         op = self.model.ops[-1]
