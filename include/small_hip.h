@@ -13,8 +13,10 @@
  *       dw filter    [C/16][kh][kw][16]
  *       bias         [C] (channel order == packed order)
  *     (reference: include/small/abstract_layer.hpp:1419-1432, include/small/buffers.hpp:33-120)
- *   - `batch` independent images lie back to back; image n of a batched call equals the
- *     reference's (batch-1) call on image n.  The reference has no batch argument.
+ *   - `batch` independent images lie back to back; image n of a batched call is the
+ *     reference's (batch-1) call on image n: bit for bit on the uint8 path, within float32
+ *     rounding on the float path (the kernel variant, and with it the summation order, is chosen
+ *     from the launch shape).  The reference has no batch argument.
  *   - Pads are given in the reference's public order: top, bottom, left, right.
  *   - Output height/width follow include/small/utils.hpp:159-165 applied to the padded input.
  *   - `stream` is a hipStream_t (NULL = the default stream).  Calls are asynchronous with
