@@ -55,6 +55,7 @@ struct QConvArgs
     int32_t ZI, ZF;          // zero points + 128
     int32_t zS, zO;          // zero points of the shortcut and of the output buffer (fused Accum / ReLU)
     int relu;
+    int use_table;       // tabulate the Accum / ReLU requantisation per workgroup (pays when the launch is ALU-bound)
     QOut q;
     int P, S, S_pad, n_co_groups, n_px_blocks, n_blocks, per_xcd;
 };
@@ -111,6 +112,32 @@ __global__ __launch_bounds__(256) void wprefix_u8_kernel(const uint8_t *__restri
     }
 }
 
+// The Accum and ReLU stages that follow a convolution in a residual block requantise values from a
+// tiny domain (a sum of two bytes, a byte), so a workgroup tabulates them once instead of running
+// the 64-bit requantisation per element: post[t], t = accumulated byte + convolution byte (0..510)
+// or, without Accum, t = convolution byte (0..255), holds the byte the op-by-op sequence produces.
+struct PostArgs
+{
+    int has_accum, relu;
+    int32_t zS, zO;
+    QOut q;
+};
+
+__device__ __forceinline__ void build_post_table(uint8_t (&post)[512], const PostArgs pa)
+{
+    for (int t = threadIdx.x; t < (pa.has_accum ? 511 : 256); t += blockDim.x)
+    {
+        uint32_t y = (uint32_t)t;
+        if (pa.has_accum) y = requant_u8((int32_t)((uint32_t)t + (uint32_t)pa.zS + (uint32_t)pa.zO), pa.q);
+        if (pa.relu)
+        {
+            const int32_t z = (int32_t)y + pa.zO;
+            y = requant_u8(z > 0 ? z : 0, pa.q);
+        }
+        post[t] = (uint8_t)y;
+    }
+}
+
 // ---- main kernel --------------------------------------------------------------------------------
 // 16 bytes of 0x80, the re-biased zero: masked taps load from here instead of being patched after
 // the load (a select on the loaded value would make the wave wait for the data where it was issued)
@@ -130,6 +157,9 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
     const int wave = threadIdx.x >> 6;
     const int col = lane & 15;
     const int grp = lane >> 4;
+
+    __shared__ uint8_t post[512];
+    const bool use_post = a.use_table && (a.accum_src != nullptr || a.relu);     // uniform
 
     const int HoWo = a.Ho * a.Wo;
     const int CiB = a.Ci / CB;
@@ -226,6 +256,12 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) load(4 * d, Bq[d], Wq[d]);
+    // tabulate the post-ops while the first loads are in flight
+    if (use_post)
+    {
+        build_post_table(post, PostArgs{a.accum_src != nullptr, a.relu, a.zS, a.zO, a.q});
+        __syncthreads();                  // use_post is uniform over the launch
+    }
     for (int s0 = 0; s0 < a.S_pad; s0 += 4 * D)
     {
 #pragma unroll
@@ -283,12 +319,16 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
             {
                 const uint32_t v = (uint32_t)acc[c][t][r] + base + (uint32_t)a.ZI * (sf4[r] + cnt);
                 uint32_t y = requant_u8((int32_t)v, a.q);
-                if (a.accum_src)
-                    y = requant_u8((int32_t)(((sc >> (8 * r)) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
-                if (a.relu)
+                if (use_post) y = post[y + ((sc >> (8 * r)) & 0xffu)];      // sc is 0 without Accum
+                else
                 {
-                    const int32_t z = (int32_t)y + a.zO;
-                    y = requant_u8(z > 0 ? z : 0, a.q);
+                    if (a.accum_src)
+                        y = requant_u8((int32_t)(((sc >> (8 * r)) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
+                    if (a.relu)
+                    {
+                        const int32_t z = (int32_t)y + a.zO;
+                        y = requant_u8(z > 0 ? z : 0, a.q);
+                    }
                 }
                 packed |= y << (8 * r);
             }
@@ -308,6 +348,7 @@ struct QSmallArgs
     const uint8_t *accum_src;
     int32_t zS, zO;
     int relu;
+    int use_table;       // tabulate the Accum / ReLU requantisation per workgroup (pays when the launch is ALU-bound)
     QOut q;
 };
 
@@ -317,8 +358,11 @@ struct QSmallArgs
 template <int CI, bool M24>
 __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a)
 {
-    const int p = blockIdx.x * 256 + threadIdx.x;
-    if (p >= a.P) return;
+    __shared__ uint8_t post[512];
+    const bool use_post = a.use_table && (a.accum_src != nullptr || a.relu);     // uniform
+    const int p0 = blockIdx.x * 256 + threadIdx.x;
+    const bool live = p0 < a.P;                                 // lanes past the end compute nothing, store nothing
+    const int p = live ? p0 : 0;
     const int cob = blockIdx.y;
     const int HoWo = a.Ho * a.Wo;
     const int n = p / HoWo;
@@ -331,7 +375,7 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
     uint32_t acc[CB];
 #pragma unroll
     for (int j = 0; j < CB; ++j) acc[j] = 0;
-    for (int ta = 0; ta < a.kh; ++ta)
+    for (int ta = 0; ta < (live ? a.kh : 0); ++ta)
     {
         const int ih = ih0 + ta;
         if (ih < 0 || ih >= a.H) continue;
@@ -355,25 +399,41 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
             }
         }
     }
+    if (use_post)
+    {
+        build_post_table(post, PostArgs{a.accum_src != nullptr, a.relu, a.zS, a.zO, a.q});
+        __syncthreads();                  // use_post is uniform over the launch
+    }
     const size_t opos = (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB;
     uint4 sc4 = make_uint4(0, 0, 0, 0);
-    if (a.accum_src) sc4 = *reinterpret_cast<const uint4 *>(a.accum_src + opos);
+    if (a.accum_src && live) sc4 = *reinterpret_cast<const uint4 *>(a.accum_src + opos);
     const uint32_t scw[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
     uint32_t pk[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < CB; ++j)
     {
         uint32_t y = requant_u8((int32_t)acc[j], a.q);
-        if (a.accum_src)
-            y = requant_u8((int32_t)(((scw[j >> 2] >> (8 * (j & 3))) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
-        if (a.relu)
+        if (use_post) y = post[y + ((scw[j >> 2] >> (8 * (j & 3))) & 0xffu)];   // scw is 0 without Accum
+        else
         {
-            const int32_t z = (int32_t)y + a.zO;
-            y = requant_u8(z > 0 ? z : 0, a.q);
+            if (a.accum_src)
+                y = requant_u8((int32_t)(((scw[j >> 2] >> (8 * (j & 3))) & 0xffu) + (uint32_t)a.zS + y + (uint32_t)a.zO), a.q);
+            if (a.relu)
+            {
+                const int32_t z = (int32_t)y + a.zO;
+                y = requant_u8(z > 0 ? z : 0, a.q);
+            }
         }
         pk[j >> 2] |= y << (8 * (j & 3));
     }
-    *reinterpret_cast<uint4 *>(a.out + opos) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    if (live) *reinterpret_cast<uint4 *>(a.out + opos) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+}
+
+// workgroups from which the post-op table pays (below, the launch is latency-bound and the table only adds a barrier)
+long table_min_wg()
+{
+    static const long v = [] { const char *e = std::getenv("SMALL_HIP_CONVQ_TABLE_MIN_WG"); return e ? std::atol(e) : 2L * NUM_CU; }();
+    return v;
 }
 
 size_t ws_ft_bytes(int Co, int S_pad) { return (size_t)Co * S_pad * 16; }
@@ -406,6 +466,7 @@ void launch_q(QConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 16 * PXT * 4 - 1) / (16 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
+    a.use_table = a.n_blocks >= table_min_wg();
     hipLaunchKernelGGL((conv_mfma_u8_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
 }
 
@@ -500,6 +561,7 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
         a.P = (int)P;
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
+        a.use_table = (long)grid.x * grid.y >= table_min_wg();
         void (*k)(const QSmallArgs) = nullptr;
         const auto small = [](int32_t z) { return z > -(1 << 22) && z < (1 << 22); };
         if (small(a.zi) && small(a.zf)) k = Ci == 1 ? conv_smallci_u8_kernel<1, true> : Ci == 2 ? conv_smallci_u8_kernel<2, true> : conv_smallci_u8_kernel<3, true>;
