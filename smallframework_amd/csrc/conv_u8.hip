@@ -44,6 +44,18 @@ namespace
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
+// n / d for 0 <= n < 2^31, d >= 1, with rcp = 1.0 / d: a double product is within one of the
+// quotient, the remainder test fixes it.  A handful of full-rate instructions instead of the
+// ~25 of the generic 32-bit division; these kernels are small enough for that to show.
+__device__ __forceinline__ int udiv_rcp(int n, int d, double rcp)
+{
+    int q = (int)((double)n * rcp);
+    const int r = n - q * d;
+    q += r >= d ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}
+
 struct QConvArgs
 {
     const uint8_t *in;
@@ -58,6 +70,7 @@ struct QConvArgs
     int use_table;       // tabulate the Accum / ReLU requantisation per workgroup (pays when the launch is ALU-bound)
     QOut q;
     int P, S, S_pad, n_co_groups, n_px_blocks, n_blocks, per_xcd;
+    double r_howo, r_wo, r_cib, r_kw;   // reciprocals of Ho*Wo, Wo, Ci/16, kw for udiv_rcp
 };
 
 // ---- filter pre-pass ---------------------------------------------------------------------------
@@ -176,9 +189,9 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
         const int p = ((pxb * 4 + wave) * PXT + t) * 16 + col;
         pvalid[t] = p < a.P;
         const int pc = pvalid[t] ? p : 0;
-        const int n = pc / HoWo;
+        const int n = udiv_rcp(pc, HoWo, a.r_howo);
         const int rem = pc - n * HoWo;
-        const int oh = rem / a.Wo;
+        const int oh = udiv_rcp(rem, a.Wo, a.r_wo);
         const int ow = rem - oh * a.Wo;
         ih0[t] = oh * a.stride - a.pt;
         iw0[t] = ow * a.stride - a.pl;
@@ -206,23 +219,24 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
     // Software pipeline of depth D over the K loop (4 K-steps per iteration, one per 16-lane group):
     // the loads of iteration i+D are issued right after iteration i has been multiplied, so D
     // iterations' worth of loads are always in flight.  These layers are small and latency-bound:
-    // without it every iteration paid a full memory round trip.  Branch-free: iterations past the
-    // end load the 0x80 block (re-biased zero, contributes nothing to the product or to sumI).
+    // without it every iteration paid a full memory round trip.  Masked taps load the 0x80 block
+    // (re-biased zero, contributes nothing to the product or to sumI).
     constexpr int D = 3;
     uint4 Bq[D][PXT], Wq[D][COT];
     auto load = [&](int s0, uint4 (&Bv)[PXT], uint4 (&Wv)[COT]) {
+        if (s0 >= a.S_pad) return;        // uniform: nothing left to fetch, the registers are not consumed again
         const int s = s0 + grp;
         const bool svalid = s < a.S;
         const int sc = svalid ? s : 0;
-        const int tap = sc / CiB;
+        const int tap = udiv_rcp(sc, CiB, a.r_cib);
         const int cib = sc - tap * CiB;
-        const int ta = tap / a.kw;
+        const int ta = udiv_rcp(tap, a.kw, a.r_kw);
         const int tb = tap - ta * a.kw;
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
-            const bool ok = svalid && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+            const bool ok = svalid && pvalid[t] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
             const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
             Bv[t] = *reinterpret_cast<const uint4 *>(ok ? in_img[t] + off : g_bias_block);
         }
@@ -267,6 +281,7 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
 #pragma unroll
         for (int d = 0; d < D; ++d)
         {
+            if (s0 + 4 * d >= a.S_pad) break;        // uniform
             consume(Bq[d], Wq[d]);
             load(s0 + 4 * (d + D), Bq[d], Wq[d]);
         }
@@ -506,6 +521,7 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     const int CiB = Ci / CB, taps = kh * kw;
     a.S = taps * CiB;
     a.S_pad = (a.S + 3) & ~3;
+    a.r_cib = 1.0 / CiB; a.r_kw = 1.0 / kw;
     a.in = in; a.out = out;
     a.ft = static_cast<const int8_t *>(prepared);
     a.wpre = reinterpret_cast<const int32_t *>(a.ft + ws_ft_bytes(Co, a.S_pad));
@@ -517,6 +533,7 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     a.stride = stride; a.pt = pt; a.pl = pl;
     a.Ho = out_dim(H, pt, pb, kh, stride);
     a.Wo = out_dim(W, pl, pr, kw, stride);
+    a.r_howo = 1.0 / ((double)a.Ho * a.Wo); a.r_wo = 1.0 / a.Wo;
     a.ZI = (int32_t)((uint32_t)iq->zero + 128u);
     a.ZF = (int32_t)((uint32_t)fq->zero + 128u);
     a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
