@@ -61,6 +61,52 @@ struct Geom
     int H, W, Ho, Wo, kh, kw, stride, pt, pl;
 };
 
+// Position of a flat pixel index in [planes][Ho][Wo].  Tensors of fewer than 2^32 pixels (all that
+// fit in practice) take the 32-bit division, a quarter of the instructions of the 64-bit one.
+struct PixelPos
+{
+    int ow, oh;
+    size_t plane;
+};
+
+#ifdef __HIPCC__
+__device__ __forceinline__ PixelPos split_pixel(size_t pix, int Wo, int Ho)
+{
+    PixelPos r;
+    if (pix <= 0xffffffffull)
+    {
+        const uint32_t p = (uint32_t)pix;
+        const uint32_t row = p / (uint32_t)Wo;
+        r.ow = (int)(p - row * (uint32_t)Wo);
+        const uint32_t pl = row / (uint32_t)Ho;
+        r.oh = (int)(row - pl * (uint32_t)Ho);
+        r.plane = pl;
+    }
+    else
+    {
+        r.ow = (int)(pix % (size_t)Wo);
+        pix /= (size_t)Wo;
+        r.oh = (int)(pix % (size_t)Ho);
+        r.plane = pix / (size_t)Ho;
+    }
+    return r;
+}
+
+// pix / d and pix % d for a row-less split (columns of planes)
+__device__ __forceinline__ size_t split_col(size_t col, int Wo, int *ow)
+{
+    if (col <= 0xffffffffull)
+    {
+        const uint32_t c = (uint32_t)col;
+        const uint32_t pl = c / (uint32_t)Wo;
+        *ow = (int)(c - pl * (uint32_t)Wo);
+        return pl;
+    }
+    *ow = (int)(col % (size_t)Wo);
+    return col / (size_t)Wo;
+}
+#endif
+
 // Library-owned device scratch for the calling thread's current device: grows on demand and is
 // re-used by later calls.  Work that uses it is ordered by the stream it is launched on, so
 // calls that share a device must not overlap on different streams.

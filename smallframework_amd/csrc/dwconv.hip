@@ -42,12 +42,10 @@ __global__ __launch_bounds__(TPB) void dw_f32_kernel(const float4 *__restrict__ 
     if (i >= total4) return;
     const int kh = KH ? KH : g.kh, kw = KW ? KW : g.kw;
     const int q = (int)(i & 3);
-    size_t pix = i >> 2;
-    const int ow = (int)(pix % (size_t)g.Wo);
-    pix /= (size_t)g.Wo;
-    const int oh = (int)(pix % (size_t)g.Ho);
-    const size_t plane = pix / (size_t)g.Ho;              // n * cblocks + cb
-    const int cbk = (int)(plane % (size_t)cblocks);
+    const PixelPos pp = split_pixel(i >> 2, g.Wo, g.Ho);
+    const int ow = pp.ow, oh = pp.oh;
+    const size_t plane = pp.plane;                        // n * cblocks + cb
+    const int cbk = (int)((uint32_t)plane % (uint32_t)cblocks);   // planes < 2^31 (checked by the launcher)
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
     const float4 *f = filt + (size_t)cbk * kh * kw * 4 + q;
     const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
@@ -98,10 +96,9 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
     const size_t i = (size_t)(lid / nstrips) * TPB + threadIdx.x;  // (plane, ow, quad)
     if (i >= ncols4) return;
     const int q = (int)(i & 3);
-    size_t col = i >> 2;
-    const int ow = (int)(col % (size_t)g.Wo);
-    const size_t plane = col / (size_t)g.Wo;                        // n * cblocks + cb
-    const int cbk = (int)(plane % (size_t)cblocks);
+    int ow;
+    const size_t plane = split_col(i >> 2, g.Wo, &ow);              // n * cblocks + cb
+    const int cbk = (int)((uint32_t)plane % (uint32_t)cblocks);     // planes < 2^31 (checked by the launcher)
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
     float4 *dst = out + plane * (size_t)g.Ho * g.Wo * 4 + (size_t)ow * 4 + q;
     const float4 *f = filt + (size_t)cbk * 36 + q;
@@ -283,12 +280,10 @@ __global__ __launch_bounds__(TPB) void dw_u8_kernel(const uint32_t *__restrict__
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= total) return;
     const int q = (int)(i & 3);
-    size_t pix = i >> 2;
-    const int ow = (int)(pix % (size_t)g.Wo);
-    pix /= (size_t)g.Wo;
-    const int oh = (int)(pix % (size_t)g.Ho);
-    const size_t plane = pix / (size_t)g.Ho;
-    const int cbk = (int)(plane % (size_t)cblocks);
+    const PixelPos pp = split_pixel(i >> 2, g.Wo, g.Ho);
+    const int ow = pp.ow, oh = pp.oh;
+    const size_t plane = pp.plane;
+    const int cbk = (int)((uint32_t)plane % (uint32_t)cblocks);   // planes < 2^31 (checked by the launcher)
     const uint32_t *src = in + plane * (size_t)g.H * g.W * 4 + q;
     const uint32_t *f = filt + (size_t)cbk * g.kh * g.kw * 4 + q;
     const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
@@ -326,6 +321,7 @@ int dw_check(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     if (!in || !filt || !out || !aligned16(in) || !aligned16(filt) || !aligned16(out))
     { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
     if (in == out) { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    if ((long)batch * (C / CB) > 0x7fffffffL) { set_error("%s: batch * C / 16 too large", op); return SMALL_HIP_EINVAL; }
     g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
     g->Ho = out_dim(H, pt, pb, kh, stride);
     g->Wo = out_dim(W, pl, pr, kw, stride);

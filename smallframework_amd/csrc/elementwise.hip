@@ -103,11 +103,9 @@ __global__ __launch_bounds__(TPB) void upsample2_f32_kernel(const float4 *__rest
         if (i < n4out)
         {
             const int q = (int)(i & 3);
-            size_t pix = i >> 2;
-            const int ow = (int)(pix % (size_t)Wo);
-            pix /= (size_t)Wo;
-            const int oh = (int)(pix % (size_t)Ho);
-            const size_t plane = pix / (size_t)Ho;            // n * cblocks + cb
+            const PixelPos pp = split_pixel(i >> 2, Wo, Ho);
+            const int ow = pp.ow, oh = pp.oh;
+            const size_t plane = pp.plane;                    // n * cblocks + cb
             out[i] = in[((plane * H + (oh >> 1)) * W + (ow >> 1)) * 4 + q];
         }
     }

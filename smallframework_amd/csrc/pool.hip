@@ -25,11 +25,9 @@ __global__ __launch_bounds__(TPB) void pool_f32_kernel(const float4 *__restrict_
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= total4) return;
     const int q = (int)(i & 3);
-    size_t pix = i >> 2;
-    const int ow = (int)(pix % (size_t)g.Wo);
-    pix /= (size_t)g.Wo;
-    const int oh = (int)(pix % (size_t)g.Ho);
-    const size_t plane = pix / (size_t)g.Ho;              // n * cblocks + cb
+    const PixelPos pp = split_pixel(i >> 2, g.Wo, g.Ho);
+    const int ow = pp.ow, oh = pp.oh;
+    const size_t plane = pp.plane;                        // n * cblocks + cb
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
     const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
     const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
@@ -71,11 +69,9 @@ __global__ __launch_bounds__(TPB) void pool_win_f32_kernel(const float4 *__restr
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= total4) return;
     const int q = (int)(i & 3);
-    size_t pix = i >> 2;
-    const int ow = (int)(pix % (size_t)g.Wo);
-    pix /= (size_t)g.Wo;
-    const int oh = (int)(pix % (size_t)g.Ho);
-    const size_t plane = pix / (size_t)g.Ho;
+    const PixelPos pp = split_pixel(i >> 2, g.Wo, g.Ho);
+    const int ow = pp.ow, oh = pp.oh;
+    const size_t plane = pp.plane;
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
     const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
     float4 v[KH * KW];
@@ -123,11 +119,9 @@ __global__ __launch_bounds__(TPB) void pool_u8_kernel(const uint32_t *__restrict
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= total) return;
     const int q = (int)(i & 3);
-    size_t pix = i >> 2;
-    const int ow = (int)(pix % (size_t)g.Wo);
-    pix /= (size_t)g.Wo;
-    const int oh = (int)(pix % (size_t)g.Ho);
-    const size_t plane = pix / (size_t)g.Ho;
+    const PixelPos pp = split_pixel(i >> 2, g.Wo, g.Ho);
+    const int ow = pp.ow, oh = pp.oh;
+    const size_t plane = pp.plane;
     const uint32_t *src = in + plane * (size_t)g.H * g.W * 4 + q;
     const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
     const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
