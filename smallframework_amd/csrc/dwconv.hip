@@ -32,6 +32,19 @@ __device__ __forceinline__ float act1(float v, int act, float slope)
     return v;
 }
 
+// The same without a branch on the activation kind (a branch per output row splits the unrolled
+// compute loop into blocks the compiler cannot schedule across): negative inputs are multiplied by
+// 1 (none), 0 (ReLU) or the slope (LeakyReLU); "+ 0.f" turns the -0 of x * 0 into the +0 ReLU gives.
+__device__ __forceinline__ float act_scale(int act, float slope)
+{
+    return act == SMALL_HIP_ACT_RELU ? 0.f : act == SMALL_HIP_ACT_LEAKY ? slope : 1.f;
+}
+__device__ __forceinline__ float act_bf(float v, float neg_scale)
+{
+    const float n = fmaf(v, neg_scale, 0.f);
+    return v > 0.f ? v : n;
+}
+
 // KH/KW == 0: run-time window size
 template <int KH, int KW>
 __global__ __launch_bounds__(TPB) void dw_f32_kernel(const float4 *__restrict__ in,
@@ -80,7 +93,7 @@ __global__ __launch_bounds__(TPB) void dw_f32_kernel(const float4 *__restrict__ 
 // are loaded once per lane, and the memory latency is paid once per lane instead of once per tap.
 // Neighbouring lanes are neighbouring columns, so each row access of a wave is one contiguous
 // kilobyte (stride 1).
-template <int STRIDE, int ROWS>
+template <int STRIDE, int ROWS, bool ACC>
 __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__restrict__ in,
                                                               const float4 *__restrict__ filt, float4 *out,
                                                               size_t ncols4, int cblocks, int nstrips,
@@ -129,13 +142,16 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
     for (int t = 0; t < 9; ++t) w[t] = f[t * 4];
     float4 bias = zero;
     if (e.bias) bias = e.bias[cbk * 4 + q];
+    const float nscale = act_scale(e.act, e.slope);
 
+    // no branch inside the unrolled rows: rows past the end are computed and not stored
 #pragma unroll
     for (int o = 0; o < ROWS; ++o)
     {
         const int oh = oh_lo + o;
-        if (oh >= g.Ho) break;
-        float4 acc = e.accumulate ? dst[(size_t)oh * g.Wo * 4] : bias;
+        const bool ok = oh < g.Ho;
+        float4 acc = bias;
+        if (ACC) { acc = zero; if (ok) acc = dst[(size_t)oh * g.Wo * 4]; }
 #pragma unroll
         for (int a = 0; a < 3; ++a)
 #pragma unroll
@@ -146,10 +162,10 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
                 acc.x = fmaf(v.x, k.x, acc.x); acc.y = fmaf(v.y, k.y, acc.y);
                 acc.z = fmaf(v.z, k.z, acc.z); acc.w = fmaf(v.w, k.w, acc.w);
             }
-        if (e.accumulate && e.bias) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }
-        acc.x = act1(acc.x, e.act, e.slope); acc.y = act1(acc.y, e.act, e.slope);
-        acc.z = act1(acc.z, e.act, e.slope); acc.w = act1(acc.w, e.act, e.slope);
-        dst[(size_t)oh * g.Wo * 4] = acc;
+        if (ACC) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }   // bias is zero without one
+        acc.x = act_bf(acc.x, nscale); acc.y = act_bf(acc.y, nscale);
+        acc.z = act_bf(acc.z, nscale); acc.w = act_bf(acc.w, nscale);
+        if (ok) dst[(size_t)oh * g.Wo * 4] = acc;
     }
 }
 
@@ -161,7 +177,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
 // three-row register window down the staged tile (three 16-byte LDS reads per output); at stride 2
 // it reads its nine taps per output.  The strip kernel issued 4.5 (stride 1) to 7 (stride 2)
 // vector-cache loads per output plus nine tap loads per lane, and that cache, not HBM, was its limit.
-template <int S, int TW, int R>
+template <int S, int TW, int R, bool ACC>
 __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__restrict__ in,
                                                              const float4 *__restrict__ filt, float4 *out,
                                                              int cblocks, int tiles_x, int tiles_y,
@@ -217,6 +233,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     for (int t = 0; t < 9; ++t) w[t] = sW[t * 4 + q];
     float4 bias = zero;
     if (e.bias) bias = e.bias[cbk * 4 + q];
+    const float nscale = act_scale(e.act, e.slope);
     const float4 *xs = sX + ((sy * R * S) * IW + tx * S) * 4 + q;
     float4 *dst = out + (size_t)plane * g.Ho * g.Wo * 4 + (size_t)ow * 4 + q;
     const bool col_ok = ow < g.Wo;
@@ -248,7 +265,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
         const int oh = oh0 + sy * R + o;
         const bool ok = col_ok && oh < g.Ho;
         float4 acc = bias;
-        if (e.accumulate) { acc = zero; if (ok) acc = dst[(size_t)oh * g.Wo * 4]; }
+        if (ACC) { acc = zero; if (ok) acc = dst[(size_t)oh * g.Wo * 4]; }
 #pragma unroll
         for (int a = 0; a < 3; ++a)
 #pragma unroll
@@ -259,9 +276,9 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
                 acc.x = fmaf(x.x, k.x, acc.x); acc.y = fmaf(x.y, k.y, acc.y);
                 acc.z = fmaf(x.z, k.z, acc.z); acc.w = fmaf(x.w, k.w, acc.w);
             }
-        if (e.accumulate && e.bias) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }
-        acc.x = act1(acc.x, e.act, e.slope); acc.y = act1(acc.y, e.act, e.slope);
-        acc.z = act1(acc.z, e.act, e.slope); acc.w = act1(acc.w, e.act, e.slope);
+        if (ACC) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }   // bias is zero without one
+        acc.x = act_bf(acc.x, nscale); acc.y = act_bf(acc.y, nscale);
+        acc.z = act_bf(acc.z, nscale); acc.w = act_bf(acc.w, nscale);
         if (ok) dst[(size_t)oh * g.Wo * 4] = acc;
     }
 }
@@ -367,14 +384,14 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 const size_t nb = (size_t)batch * (C / CB) * tiles_x * tiles_y;
                 if (nb > 0x7fffffff / 2) { set_error("%s: too many blocks for one launch", op); return SMALL_HIP_EINVAL; }
                 const int nblocks = (int)nb, per_xcd = (nblocks + NUM_XCD - 1) / NUM_XCD;
-                decltype(&dw3x3_f32_tile_kernel<1, 16, 4>) tk;
+                decltype(&dw3x3_f32_tile_kernel<1, 16, 4, false>) tk;
+#define SHP_DW_TILE(S_, TW_, R_) (accumulate ? dw3x3_f32_tile_kernel<S_, TW_, R_, true> : dw3x3_f32_tile_kernel<S_, TW_, R_, false>)
                 if (stride == 1)
-                    tk = best == 0 ? dw3x3_f32_tile_kernel<1, 16, 4> : best == 1 ? dw3x3_f32_tile_kernel<1, 8, 7>
-                       : best == 2 ? dw3x3_f32_tile_kernel<1, 16, 7> : best == 3 ? dw3x3_f32_tile_kernel<1, 32, 4>
-                                                                     : dw3x3_f32_tile_kernel<1, 8, 1>;
+                    tk = best == 0 ? SHP_DW_TILE(1, 16, 4) : best == 1 ? SHP_DW_TILE(1, 8, 7)
+                       : best == 2 ? SHP_DW_TILE(1, 16, 7) : best == 3 ? SHP_DW_TILE(1, 32, 4) : SHP_DW_TILE(1, 8, 1);
                 else
-                    tk = best == 0 ? dw3x3_f32_tile_kernel<2, 8, 1> : best == 1 ? dw3x3_f32_tile_kernel<2, 4, 1>
-                                                                   : dw3x3_f32_tile_kernel<2, 16, 1>;
+                    tk = best == 0 ? SHP_DW_TILE(2, 8, 1) : best == 1 ? SHP_DW_TILE(2, 4, 1) : SHP_DW_TILE(2, 16, 1);
+#undef SHP_DW_TILE
                 hipLaunchKernelGGL(tk, dim3(per_xcd * NUM_XCD), dim3(TPB), 0, as_stream(stream),
                                    reinterpret_cast<const float4 *>(in), reinterpret_cast<const float4 *>(filt),
                                    reinterpret_cast<float4 *>(out), C / CB, tiles_x, tiles_y, nblocks, per_xcd, g, e);
@@ -388,7 +405,8 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
         const size_t nb = ((ncols4 + TPB - 1) / TPB) * (size_t)nstrips;
         if (nb > 0x7fffffff / 2) { set_error("%s: too many blocks for one launch", op); return SMALL_HIP_EINVAL; }
         const int nblocks = (int)nb, per_xcd = (nblocks + NUM_XCD - 1) / NUM_XCD;
-        auto sk = stride == 1 ? dw3x3_f32_strip_kernel<1, R1> : dw3x3_f32_strip_kernel<2, R2>;
+        auto sk = stride == 1 ? (accumulate ? dw3x3_f32_strip_kernel<1, R1, true> : dw3x3_f32_strip_kernel<1, R1, false>)
+                              : (accumulate ? dw3x3_f32_strip_kernel<2, R2, true> : dw3x3_f32_strip_kernel<2, R2, false>);
         hipLaunchKernelGGL(sk, dim3(per_xcd * NUM_XCD), dim3(TPB), 0, as_stream(stream),
                            reinterpret_cast<const float4 *>(in), reinterpret_cast<const float4 *>(filt),
                            reinterpret_cast<float4 *>(out), ncols4, C / CB, nstrips, nblocks, per_xcd, g, e);
