@@ -72,12 +72,44 @@ __device__ __forceinline__ float act1(float v, int act, float slope)
     return v;
 }
 
-// accumulate / bias / activation in registers, then 16-byte stores: a lane holds channels
-// 8q + 4*half + {0..3} of its pixel in accumulator registers 4q .. 4q+3
-template <int COT, int PXT>
-__device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
-                                              int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+// negative inputs are multiplied by 1 (no activation), 0 (ReLU) or the slope (LeakyReLU): the
+// activation without a branch on its kind; "+ 0.f" turns the -0 of x * 0 into the +0 ReLU gives
+__device__ __forceinline__ float act_scale(int act, float slope)
 {
+    return act == SMALL_HIP_ACT_RELU ? 0.f : act == SMALL_HIP_ACT_LEAKY ? slope : 1.f;
+}
+__device__ __forceinline__ float act_bf(float v, float neg_scale)
+{
+    const float n = fmaf(v, neg_scale, 0.f);
+    return v > 0.f ? v : n;
+}
+
+// accumulate / bias / activation in registers, then 16-byte stores: a lane holds channels
+// 8q + 4*half + {0..3} of its pixel in accumulator registers 4q .. 4q+3.  Straight-line code:
+// pixels past the end and channels past Co are computed and not stored, the bias is loaded once
+// per channel quad, PartialConv2D (ACC) is a compile-time variant.
+template <int COT, int PXT, bool ACC>
+__device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
+                                                   int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+{
+    const float nscale = act_scale(a.act, a.slope);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 bb[COT][4];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bb[c][q] = zero;
+    if (a.bias)
+    {
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int co4 = (cg * COT + c) * 32 + 8 * q + 4 * half;
+                if (co4 < a.Co) bb[c][q] = *reinterpret_cast<const float4 *>(a.bias + co4);
+            }
+    }
 #pragma unroll
     for (int c = 0; c < COT; ++c)
     {
@@ -85,32 +117,36 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
-            if (!pvalid[t]) continue;
 #pragma unroll
             for (int q = 0; q < 4; ++q)
             {
                 const int co4 = co_tile + 8 * q + 4 * half;
-                if (co4 >= a.Co) continue;
+                const bool ok = pvalid[t] && co4 < a.Co;
                 float4 v = make_float4(acc[c][t][4 * q + 0], acc[c][t][4 * q + 1],
                                        acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
                 float4 *o = reinterpret_cast<float4 *>(a.out + out_pix[t] +
                                                        (size_t)(co4 / CB) * HoWo * CB + (co4 % CB));
-                if (a.accumulate)
+                if (ACC)
                 {
-                    const float4 old = *o;
+                    float4 old = zero;
+                    if (ok) old = *o;
                     v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
                 }
-                if (a.bias)
-                {
-                    const float4 bb = *reinterpret_cast<const float4 *>(a.bias + co4);
-                    v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
-                }
-                v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
-                v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
-                *o = v;
+                v.x += bb[c][q].x; v.y += bb[c][q].y; v.z += bb[c][q].z; v.w += bb[c][q].w;
+                v.x = act_bf(v.x, nscale); v.y = act_bf(v.y, nscale);
+                v.z = act_bf(v.z, nscale); v.w = act_bf(v.w, nscale);
+                if (ok) *o = v;
             }
         }
     }
+}
+
+template <int COT, int PXT>
+__device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
+                                              int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+{
+    if (a.accumulate) conv_epilogue_impl<COT, PXT, true>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
 template <int COT, int PXT>
