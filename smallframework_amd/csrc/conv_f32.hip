@@ -366,31 +366,40 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     bool live = true;
 
     // issues the global loads of the step at (ta, tb, cib) and advances the position
+    // Straight-line on purpose (selects, no branches; 32-bit element offsets inside an image, which the
+    // launcher guarantees fit): a K-step is then one basic block and the compiler can slot this
+    // address arithmetic between the MFMAs instead of running it after them.
+    const int in_blk32 = a.H * a.W * CB;
     auto fetch = [&](float4 (&Areg)[A_PER_THREAD], float4 (&B)[PXT][2]) {
         const int tap = ta * a.kw + tb;
         // filter first: its staging store is the first consumer, so it can wait for these loads
         // alone and leave the activation loads of the same step in flight
-        const size_t woff = ((size_t)cib * taps + tap) * (CB * CB);
+        const int woff = (cib * taps + tap) * (CB * CB);
 #pragma unroll
         for (int j = 0; j < A_PER_THREAD; ++j) Areg[j] = *reinterpret_cast<const float4 *>(a_src[j] + woff);
+        const int cib_off = cib * in_blk32;
 #pragma unroll
         for (int t = 0; t < PXT; ++t)
         {
             const int ih = ih0[t] + ta, iw = iw0[t] + tb;
-            const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
-            const float4 *p = reinterpret_cast<const float4 *>(ok ? in_img[t] + off : zero_half);
+            const bool ok = live && pvalid[t] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+            const int off = cib_off + (ih * a.W + iw) * CB;
+            const float *pp = in_img[t] + off;
+            const float4 *p = reinterpret_cast<const float4 *>(ok ? pp : zero_half);
             B[t][0] = p[0];
             B[t][1] = p[1];
         }
-        int ncib = cib + 1, ntb = tb, nta = ta;
-        if (ncib == CiB)
-        {
-            ncib = 0;
-            if (++ntb == a.kw) { ntb = 0; ++nta; }
-        }
-        if (nta < a.kh) { cib = ncib; tb = ntb; ta = nta; }
-        else live = false;
+        // next (tap, channel block): channel block fastest, then the window column, then the row
+        const bool w1 = cib + 1 == CiB;
+        const int ncib = w1 ? 0 : cib + 1;
+        const bool w2 = w1 && tb + 1 == a.kw;
+        const int ntb = w2 ? 0 : tb + (w1 ? 1 : 0);
+        const int nta = ta + (w2 ? 1 : 0);
+        const bool more = nta < a.kh;
+        cib = more ? ncib : cib;
+        tb = more ? ntb : tb;
+        ta = more ? nta : ta;
+        live = live && more;
     };
     auto stage = [&](int buf, const float4 (&Areg)[A_PER_THREAD]) {
 #pragma unroll
@@ -880,6 +889,8 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     const long P = (long)batch * a.Ho * a.Wo;
     if (P == 0) return SMALL_HIP_OK;
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
+    if ((long)Ci * H * W > 0x7fffffffL / 2 || (long)Ci * kh * kw * CB > 0x7fffffffL / 2)
+    { set_error("%s: one image or one filter block too large for 32-bit offsets", op); return SMALL_HIP_EINVAL; }
     a.P = (int)P;
     hipStream_t s = as_stream(stream);
 
