@@ -1,35 +1,28 @@
 // Conv2D / PartialConv2D / Dense (float32) for gfx950.
 //
-// Two kernels:
-//
-//  conv_mfma_f32_kernel   input_channels % 16 == 0.  Implicit GEMM on v_mfma_f32_32x32x2_f32:
+// input_channels % 16 == 0: implicit GEMM on v_mfma_f32_32x32x2_f32,
 //      D[co][px] += sum_k  F[co][k] * I[k][px],   k = (tap, ci)
-//    MFMA rows are output channels, MFMA columns are output pixels flattened over
-//    (image, oh, ow).  With the packed layouts a K-step of 16 (one input-channel block at one
-//    filter tap) needs no shuffling at all:
-//      - B operand: lane (px = lane%32, half = lane/32) reads 8 consecutive floats of its
-//        pixel's 64-byte channel block: two 16-byte loads straight from global memory into the
-//        register the MFMA consumes.  The two wave halves take channels 0-7 and 8-15, so MFMA
-//        number kk of the step contracts channels {kk, 8+kk}; the pairing of k inside an MFMA
-//        is free as long as A and B agree.
-//      - A operand: lane (co = lane%32, half) reads F[ci = 8*half+kk][co%16] of its channel
-//        block's [16 ci][16 co] tile: 8 dword loads, each coalesced over 16 lanes.
-//      - D: lane holds 4 consecutive output channels of one pixel per register quad, i.e.
-//        16-byte stores into the packed [px][16] output.
-//    Padded taps are contributed as zeros by predicating the B operand.  The loads of step
-//    s+1 are issued before the MFMAs of step s (register double buffer).
-//    A wave owns COT x PXT tiles of 32 x 32; the four waves of a workgroup share the output
-//    channel group (their filter reads hit in the vector cache) and take consecutive pixel
-//    tiles.  Workgroup ids are re-mapped so that all channel groups of a pixel range run on
-//    one XCD and share its L2.
+// MFMA rows are output channels, MFMA columns are output pixels flattened over (image, oh, ow).
+// With the packed layouts a K-step of 16 (one input-channel block at one filter tap) needs no
+// shuffling at all:
+//   - B operand: lane (px = lane%32, half = lane/32) reads 8 consecutive floats of its pixel's
+//     64-byte channel block: two 16-byte loads straight from global memory into the register the
+//     MFMA consumes.  The two wave halves take channels 0-7 and 8-15, so MFMA number kk of the
+//     step contracts channels {kk, 8+kk}; the pairing of k inside an MFMA is free as long as A
+//     and B agree.  Padded taps load a block of zeros.
+//   - A operand: F[ci = 8*half+kk][co%16] of the channel block's [16 ci][16 co] tile, staged
+//     through LDS once per workgroup (conv_lds_tile) or read directly (conv_splitk_tile).
+//   - D: a lane holds 4 consecutive output channels of one pixel per register quad, i.e. 16-byte
+//     stores into the packed [px][16] output, after accumulate / bias / activation in registers.
+// A wave owns COT x PXT tiles of 32 x 32; the four waves of a workgroup share the output channel
+// group and take consecutive pixel tiles.  Workgroup ids are re-mapped so that all channel groups
+// of a pixel range run on one XCD and share its L2.  Kernels:
+//   conv_mfma_f32_lds_kernel      every workgroup runs conv_lds_tile
+//   conv_mfma_f32_hybrid_kernel   whole rounds of conv_lds_tile + the remainder as split-K tiles
+//   conv_mfma_f32_splitk_kernel   small outputs: one 32x32 tile per workgroup, K split over its waves
 //
-//  conv_smallci_f32_kernel   input_channels in {1,2,3} (first layers).  K is only
-//    Ci*kh*kw (27 for a 3x3 RGB stem), so these layers are bound by HBM traffic of their
-//    large outputs; a lane computes the 16 output channels of one pixel with scalar-loaded
-//    weights on the vector ALU.
-//
-// Epilogue (both kernels, in registers): optional accumulate onto the existing output
-// (PartialConv2D), optional bias, optional ReLU / LeakyReLU.
+// input_channels in {1,2,3} (first layers): conv_smallci_mfma_f32_kernel (3x3 and 10x4 windows,
+// at least 32 output channels) and conv_smallci_f32_kernel (vector ALU, everything else).
 #include "common.h"
 
 #include <cstdlib>
@@ -149,145 +142,13 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
     else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
-template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_kernel(const ConvArgs a)
-{
-    // XCD-aware id: hardware deals consecutive workgroup ids round-robin over the 8 XCDs
-    const int bid = blockIdx.x;
-    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
-    if (lid >= a.n_blocks) return;
-    const int cg = lid % a.n_co_groups;
-    const int pxb = lid / a.n_co_groups;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int col = lane & 31;
-    const int half = lane >> 5;
-
-    const int HoWo = a.Ho * a.Wo;
-    const int CiB = a.Ci / CB;
-    const int CoB = a.Co / CB;
-    const int taps = a.kh * a.kw;
-    const size_t in_blk = (size_t)a.H * a.W * CB;     // floats per input channel block
-    const float *zero_half = g_zero_block + half * 8;
-
-    // ---- per-lane pixel columns --------------------------------------------------------
-    const float *in_img[PXT];   // image base + half offset
-    int ih0[PXT], iw0[PXT];
-    bool pvalid[PXT];
-    size_t out_pix[PXT];        // float index of (n, co block 0, pixel), co block stride = HoWo*16
-#pragma unroll
-    for (int t = 0; t < PXT; ++t)
-    {
-        const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
-        pvalid[t] = p < a.P;
-        const int pc = pvalid[t] ? p : 0;
-        const int n = pc / HoWo;
-        const int rem = pc - n * HoWo;
-        const int oh = rem / a.Wo;
-        const int ow = rem - oh * a.Wo;
-        ih0[t] = oh * a.stride - a.pt;
-        iw0[t] = ow * a.stride - a.pl;
-        in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
-        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
-    }
-    // ---- per-lane filter rows ------------------------------------------------------------
-    const float *w_row[COT];
-    int co_of[COT];
-#pragma unroll
-    for (int c = 0; c < COT; ++c)
-    {
-        const int co = (cg * COT + c) * 32 + col;
-        co_of[c] = co;
-        const int cc = co < a.Co ? co : a.Co - 1;   // rows past Co compute garbage, never stored
-        w_row[c] = a.filt + (size_t)(cc / CB) * CiB * taps * (CB * CB) + (cc % CB) + half * 8 * CB;
-    }
-
-    floatx16 acc[COT][PXT];
-#pragma unroll
-    for (int c = 0; c < COT; ++c)
-#pragma unroll
-        for (int t = 0; t < PXT; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
-
-    // ---- K loop state: tap (ta, tb) outer, input channel block inner ---------------------
-    // The loop below is branch-free: it always runs an even number of steps and a step past the
-    // end (`live` false) loads from valid addresses and contributes zeros through the B operand.
-    int ta = 0, tb = 0, cib = 0;
-    const int nsteps = taps * CiB;
-    bool live = true;
-
-    auto load_step = [&](float (&A)[COT][8], float4 (&B)[PXT][2]) {
-        const int tap = ta * a.kw + tb;
-#pragma unroll
-        for (int t = 0; t < PXT; ++t)
-        {
-            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
-            const bool ok = live && pvalid[t] && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-            const size_t off = (size_t)cib * in_blk + ((size_t)ih * a.W + iw) * CB;
-            const float4 *p = reinterpret_cast<const float4 *>(ok ? in_img[t] + off : zero_half);
-            B[t][0] = p[0];
-            B[t][1] = p[1];
-        }
-#pragma unroll
-        for (int c = 0; c < COT; ++c)
-        {
-            const float *w = w_row[c] + ((size_t)cib * taps + tap) * (CB * CB);
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) A[c][kk] = w[kk * CB];
-        }
-        // advance; the state parks on the last step once the end is reached
-        int ncib = cib + 1, ntb = tb, nta = ta;
-        if (ncib == CiB)
-        {
-            ncib = 0;
-            if (++ntb == a.kw) { ntb = 0; ++nta; }
-        }
-        if (nta < a.kh) { cib = ncib; tb = ntb; ta = nta; }
-        else live = false;
-    };
-
-    auto compute_step = [&](const float (&A)[COT][8], const float4 (&B)[PXT][2]) {
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk)
-        {
-#pragma unroll
-            for (int t = 0; t < PXT; ++t)
-            {
-                const float4 bv = B[t][kk >> 2];
-                const float b = (kk & 3) == 0 ? bv.x : (kk & 3) == 1 ? bv.y : (kk & 3) == 2 ? bv.z : bv.w;
-#pragma unroll
-                for (int c = 0; c < COT; ++c)
-                    acc[c][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[c][kk], b, acc[c][t], 0, 0, 0);
-            }
-        }
-    };
-
-    // register double buffer: the loads of step s+1 are in flight while step s is multiplied
-    float A0[COT][8], A1[COT][8];
-    float4 B0[PXT][2], B1[PXT][2];
-    load_step(A0, B0);
-    const int npairs = (nsteps + 1) >> 1;
-    for (int it = 0; it < npairs; ++it)
-    {
-        load_step(A1, B1);
-        compute_step(A0, B0);
-        load_step(A0, B0);
-        compute_step(A1, B1);
-    }
-
-    conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
-    (void)co_of;
-}
-
 // ---------------------------------------------------------------------------------------------
-// Same contraction with the filter operand staged through LDS.  The four waves of a workgroup
+// The main kernel body: filter operand staged through LDS.  The four waves of a workgroup
 // multiply the same output-channel group, so the step's [16 ci][16 co] filter tiles (COT*2 KiB)
 // are fetched once per workgroup with fully coalesced 16-byte loads, written to LDS (double
-// buffered, one barrier per K-step) and read back by every wave in MFMA operand order.  This cuts
-// the vector-cache accesses of the filter by 4x and replaces 8 strided dword loads per tile by
-// one 16-byte load per lane.  The activation operand still goes straight from global memory to
+// buffered, one barrier per K-step) and read back by every wave in MFMA operand order: a quarter
+// of the vector-cache accesses of per-wave filter reads, and one 16-byte load per lane instead
+// of 8 strided dword loads per tile.  The activation operand goes straight from global memory to
 // the MFMA register, two 16-byte loads per lane and tile.
 constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks start 16 banks apart
 
@@ -845,20 +706,16 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    // SMALL_HIP_CONV_LDS=0 selects the variant that reads the filter operand straight from global memory
-    static const bool use_lds = [] { const char *e = std::getenv("SMALL_HIP_CONV_LDS"); return !(e && e[0] == '0'); }();
     static const bool use_tail = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return !(e && e[0] == '0'); }();
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
-    if (use_lds && use_tail && rest > 0 && a.kh * a.kw * (a.Ci / CB) >= 8)
+    if (use_tail && rest > 0 && a.kh * a.kw * (a.Ci / CB) >= 8)
     {
         a.n_main = n_main;
         hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT), dim3(256),
                            0, s, a);
     }
-    else if (use_lds)
-        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL((conv_mfma_f32_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
 }
 
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
@@ -943,7 +800,7 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }
-    // tuning knob: SMALL_HIP_CONV_TILE="<cot>,<pxt>" forces a wave tile (32-channel x 32-pixel units)
+    // tuning knob: SMALL_HIP_CONV_TILE="<cot>,<pxt>" forces a wave tile (32-channel x 32-pixel units; 1,1 1,2 2,1 2,2)
     if (const char *e = std::getenv("SMALL_HIP_CONV_TILE"))
     {
         int c2 = 0, p2 = 0;
@@ -952,10 +809,6 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     if (cot == 2 && pxt == 2) launch_mfma<2, 2>(a, s);
     else if (cot == 1 && pxt == 2) launch_mfma<1, 2>(a, s);
     else if (cot == 2 && pxt == 1) launch_mfma<2, 1>(a, s);
-    else if (cot == 4 && pxt == 1) launch_mfma<4, 1>(a, s);
-    else if (cot == 4 && pxt == 2) launch_mfma<4, 2>(a, s);
-    else if (cot == 2 && pxt == 4) launch_mfma<2, 4>(a, s);
-    else if (cot == 1 && pxt == 4) launch_mfma<1, 4>(a, s);
     else launch_mfma<1, 1>(a, s);
     SHP_LAUNCH_CHECK(op);
     return SMALL_HIP_OK;
