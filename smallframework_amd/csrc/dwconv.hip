@@ -177,13 +177,13 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
 // three-row register window down the staged tile (three 16-byte LDS reads per output); at stride 2
 // it reads its nine taps per output.  The strip kernel issued 4.5 (stride 1) to 7 (stride 2)
 // vector-cache loads per output plus nine tap loads per lane, and that cache, not HBM, was its limit.
-template <int S, int TW, int R, bool ACC>
+template <int S, int TW, int R, bool ACC, int SRU = 0>
 __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__restrict__ in,
                                                              const float4 *__restrict__ filt, float4 *out,
                                                              int cblocks, int tiles_x, int tiles_y,
                                                              int nblocks, int per_xcd, Geom g, Epi e)
 {
-    constexpr int SR = 64 / TW;                              // rows of lane slots
+    constexpr int SR = SRU ? SRU : 64 / TW;                  // rows of lane slots in use (SRU < 64/TW leaves slots idle for a smaller tile)
     constexpr int TH = SR * R;                               // output rows per tile
     constexpr int IW = (TW - 1) * S + 3, IH = (TH - 1) * S + 3;  // staged input tile, in pixels
     constexpr int ROW4 = IW * 4;                             // float4 per staged row
@@ -226,7 +226,9 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     __syncthreads();
 
     const int q = tid & 3, slot = tid >> 2;
-    const int tx = slot % TW, sy = slot / TW;
+    const int tx = slot % TW, sy_raw = slot / TW;
+    const bool slot_on = sy_raw < SR;
+    const int sy = slot_on ? sy_raw : 0;      // idle slots read in bounds and store nothing
     const int ow = ow0 + tx;
     float4 w[9];
 #pragma unroll
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     const float nscale = act_scale(e.act, e.slope);
     const float4 *xs = sX + ((sy * R * S) * IW + tx * S) * 4 + q;
     float4 *dst = out + (size_t)plane * g.Ho * g.Wo * 4 + (size_t)ow * 4 + q;
-    const bool col_ok = ow < g.Wo;
+    const bool col_ok = slot_on && ow < g.Wo;
 
     float4 win[3][3];
     if (S == 1)
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
 
 // tile shapes of the LDS kernel: (TW, R) -> a TW x (64/TW)*R tile of output pixels
 struct TileShape { int tw, th; };
-constexpr TileShape TILE_SHAPES_S1[] = {{16, 16}, {8, 56}, {16, 28}, {32, 8}, {8, 8}};
+constexpr TileShape TILE_SHAPES_S1[] = {{16, 16}, {8, 28}, {16, 28}, {32, 8}, {8, 8}};
 constexpr TileShape TILE_SHAPES_S2[] = {{8, 8}, {4, 16}, {16, 4}};
 
 
@@ -373,10 +375,16 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
             {
                 const int tx = (g.Wo + shapes[t].tw - 1) / shapes[t].tw;
                 const int ty = (g.Ho + shapes[t].th - 1) / shapes[t].th;
-                const double util = (double)g.Wo * g.Ho / ((double)tx * shapes[t].tw * ty * shapes[t].th);
+                double util = (double)g.Wo * g.Ho / ((double)tx * shapes[t].tw * ty * shapes[t].th);
+                if (stride == 1 && t == 1) util *= 0.875;      // the 8x28 tile leaves one slot row of eight idle
                 if (util > best_util + 1e-9) { best_util = util; best = t; }
             }
-            if (const char *v = std::getenv("SMALL_HIP_DW_SHAPE")) best = std::atoi(v);
+            // tuning knob: force a shape of the table
+            if (const char *v = std::getenv("SMALL_HIP_DW_SHAPE"))
+            {
+                const int f = std::atoi(v);
+                if (f >= 0 && f < nshapes) best = f;
+            }
             if (best >= 0)
             {
                 const int tiles_x = (g.Wo + shapes[best].tw - 1) / shapes[best].tw;
@@ -387,7 +395,8 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 decltype(&dw3x3_f32_tile_kernel<1, 16, 4, false>) tk;
 #define SHP_DW_TILE(S_, TW_, R_) (accumulate ? dw3x3_f32_tile_kernel<S_, TW_, R_, true> : dw3x3_f32_tile_kernel<S_, TW_, R_, false>)
                 if (stride == 1)
-                    tk = best == 0 ? SHP_DW_TILE(1, 16, 4) : best == 1 ? SHP_DW_TILE(1, 8, 7)
+                    tk = best == 0 ? SHP_DW_TILE(1, 16, 4)
+                       : best == 1 ? (accumulate ? dw3x3_f32_tile_kernel<1, 8, 4, true, 7> : dw3x3_f32_tile_kernel<1, 8, 4, false, 7>)
                        : best == 2 ? SHP_DW_TILE(1, 16, 7) : best == 3 ? SHP_DW_TILE(1, 32, 4) : SHP_DW_TILE(1, 8, 1);
                 else
                     tk = best == 0 ? SHP_DW_TILE(2, 8, 1) : best == 1 ? SHP_DW_TILE(2, 4, 1) : SHP_DW_TILE(2, 16, 1);

@@ -174,7 +174,7 @@ WIN_CASES = [
     (2, 7, 7, 1, (0, 0, 0, 0), 64, 7, 7),
     (1, 25, 5, 1, (0, 0, 0, 0), 64, 25, 5),
     (1, 3, 3, 2, (0, 0, 0, 0), 256, 56, 56),
-    # stride-1 3x3 at sizes that select each tile shape of the LDS depthwise kernel, whole and ragged
+    # stride-1 3x3 at sizes that select each tile shape of the LDS depthwise kernel (16x16, 8x28, 16x28, 32x8, 8x8), whole and ragged
     (2, 3, 3, 1, (1, 1, 1, 1), 32, 16, 16),
     (1, 3, 3, 1, (1, 1, 1, 1), 16, 56, 56),
     (2, 3, 3, 1, (1, 1, 1, 1), 32, 28, 28),
