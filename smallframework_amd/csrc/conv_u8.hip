@@ -536,7 +536,7 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     a.r_howo = 1.0 / ((double)a.Ho * a.Wo); a.r_wo = 1.0 / a.Wo;
     a.ZI = (int32_t)((uint32_t)iq->zero + 128u);
     a.ZF = (int32_t)((uint32_t)fq->zero + 128u);
-    a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
+    a.q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
     const long P = (long)batch * a.Ho * a.Wo;
     if (P == 0) return SMALL_HIP_OK;
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
@@ -572,7 +572,7 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         a.Wo = out_dim(W, pl, pr, kw, stride);
         a.zi = iq->zero; a.zf = fq->zero;
         a.accum_src = fz.accum_src; a.zS = fz.zS; a.zO = oq->zero; a.relu = fz.relu;
-        a.q = QOut{oq->multiplier, oq->lshift, oq->rshift};
+        a.q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
         const long P = (long)batch * a.Ho * a.Wo;
         if (P == 0) return SMALL_HIP_OK;
         if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }

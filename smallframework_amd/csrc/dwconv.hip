@@ -481,7 +481,7 @@ int small_hip_depthwise_conv2d_u8(int batch, int kh, int kw, int stride, int pt,
     if (int rc = dw_check(op, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, filt, out, &g)) return rc;
     const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total == 0) return SMALL_HIP_OK;
-    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    const QOut q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
     hipLaunchKernelGGL(dw_u8_kernel, dim3((unsigned)((total + TPB - 1) / TPB)), dim3(TPB), 0, as_stream(stream),
                        reinterpret_cast<const uint32_t *>(in), reinterpret_cast<const uint32_t *>(filt),
                        reinterpret_cast<uint32_t *>(out), total, C / CB, g, iq->zero, fq->zero, q);

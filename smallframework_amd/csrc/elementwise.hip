@@ -291,7 +291,7 @@ int small_hip_relu_u8(int batch, int C, int H, int W, const uint8_t *in, const s
     if (!iq || !oq) return einval("small_hip_relu_u8: null quantisation parameters");
     if (int rc = check_act_args("small_hip_relu_u8", batch, C, H, W, in, out)) return rc;
     const size_t n16 = (size_t)batch * C * H * W / 16;
-    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    const QOut q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
     hipLaunchKernelGGL(ew_u8_kernel<false>, dim3(blocks_for(n16)), dim3(TPB), 0, as_stream(stream),
                        reinterpret_cast<const uint4 *>(in), reinterpret_cast<uint4 *>(out), n16,
                        iq->zero, 0, q);
@@ -305,7 +305,7 @@ int small_hip_accum_u8(int batch, int C, int H, int W, const uint8_t *in, const 
     if (!iq || !oq) return einval("small_hip_accum_u8: null quantisation parameters");
     if (int rc = check_act_args("small_hip_accum_u8", batch, C, H, W, in, out)) return rc;
     const size_t n16 = (size_t)batch * C * H * W / 16;
-    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    const QOut q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
     hipLaunchKernelGGL(ew_u8_kernel<true>, dim3(blocks_for(n16)), dim3(TPB), 0, as_stream(stream),
                        reinterpret_cast<const uint4 *>(in), reinterpret_cast<uint4 *>(out), n16,
                        iq->zero, oq->zero, q);

@@ -302,7 +302,7 @@ int pool_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
     if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
     const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total == 0) return SMALL_HIP_OK;
-    const QOut q{oq->multiplier, oq->lshift, oq->rshift};
+    const QOut q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
     if (is_global(g, pt, pb, pl, pr))
     {
         const int planes = batch * (C / CB);

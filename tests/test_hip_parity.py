@@ -351,6 +351,8 @@ QPARAMS = [
     (-120, -131, 2000000000, 0, 0),
     # zero points beyond 24 bits: int32 wrap-around arithmetic, the 32-bit multiply path of the stem kernel
     (-(1 << 24) - 77, (1 << 23) + 5, 1518500250, 0, 3),
+    # a negative multiplier: the general form of the requantisation (the short form needs multiplier > 0)
+    (-128, -128, -1518500250, 0, 5),
 ]
 
 
