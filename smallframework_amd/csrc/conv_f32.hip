@@ -311,8 +311,11 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
+// The second launch bound (minimum waves per SIMD: 6 / 5 / 2 for one / two / four MFMA tiles per
+// wave) makes the compiler keep the accumulators in the unified register file and pack tighter
+// (2x1: 108 -> 76 registers, 2x2: 184 -> 131, no spills); measured 1-3% faster, tighter bounds spill.
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_lds_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a)
 {
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
     const int bid = blockIdx.x;
@@ -490,7 +493,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
 // 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
 // The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_hybrid_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a)
 {
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
     __shared__ float red[3][1][16][64];
