@@ -157,6 +157,40 @@ def cpu_port_u8(model, batch=8):
             "sample": "%d images x %d passes of %s on the scalar C restatement" % (batch, reps, model.name)}
 
 
+def layout_rows(lib, torch, steps, warmup):
+    """On-device pack_buffer / unpack_buffer (NCHW <-> packed), HIP-event timed; pure data movement,
+    bound = HBM with one read and one write per element."""
+    import ctypes as C
+    cases = [("pack_input_3x224x224_b64", "pack", 64, 3, 224, 224),
+             ("pack_256x56x56_b64", "pack", 64, 256, 56, 56),
+             ("unpack_256x56x56_b64", "unpack", 64, 256, 56, 56),
+             ("unpack_logits_1008_b64", "unpack", 64, 1008, 1, 1)]
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rows = []
+    for name, way, b, c, h, w in cases:
+        n = b * c * h * w
+        src = torch.randn(n, device="cuda")
+        dst = torch.empty_like(src)
+        fn = lib.small_hip_pack if way == "pack" else lib.small_hip_unpack
+        call = lambda: fn(0, b, 1, c, h, w, 16, 16, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), 4, st)
+        for _ in range(warmup):
+            assert call() == 0
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        nbytes = 2 * n * 4
+        rows.append({"layer": name, "ms": round(ms, 5), "bound": "hbm", "GB/s": round(nbytes / ms / 1e6, 1),
+                     "roofline_frac": round(nbytes / PEAK_HBM / (ms * 1e-3), 4)})
+        log("%-26s %.4f ms  %.0f GB/s  %.1f%% of HBM peak" % (name, ms, nbytes / ms / 1e6, 100 * rows[-1]["roofline_frac"]))
+        del src, dst
+    torch.cuda.empty_cache()
+    return rows
+
+
 def sweep_only(args, torch, models):
     """--model layer_sweep: the four single layers at C = 256, 56x56 (Conv2D 3x3, DepthwiseConv2D 3x3,
     MaxPool2D 3x3 stride 2, ReLU), each run `steps` times at --batch (default 64).  The JSON line is
@@ -177,6 +211,8 @@ def sweep_only(args, torch, models):
             head = (m, sec, r)
         del ex
         torch.cuda.empty_cache()
+    from smallframework_amd import capi
+    rows += layout_rows(capi.load(), torch, args.steps, args.warmup)
     m, sec, r = head
     op = m.ops[0]
     out = {"metric": "images/s @batch%d %s fp32" % (batch, m.name), "value": round(batch / sec, 2),
@@ -320,6 +356,8 @@ def main():
                                                            100 * (r["roofline_frac"] or 0)))
             del e2
             torch.cuda.empty_cache()
+
+        extras["layout"] = {"layers": layout_rows(capi.load(), torch, args.steps, args.warmup)}
 
     cpu = None
     if not args.no_cpu:

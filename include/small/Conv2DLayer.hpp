@@ -1,0 +1,291 @@
+// Conv2DLayer: convolution with constant weights, optional bias, folded batch normalisation and
+// activation (same constructors, accessors, checks and messages as the reference's
+// include/small/Conv2DLayer.hpp:27-916).
+//
+// What differs underneath:
+//   - compute_output() is ONE launch: bias + convolution + activation fused
+//     (small_hip_conv2d_bias_act_f32), where the reference issues Bias, PartialConv2D and the
+//     activation as three passes over the output (Conv2DLayer.hpp:827-879);
+//   - the batch extent of the input shape is honoured (N packed images per call);
+//   - unpacked filters are packed on the device; on the quantised path the filter is also brought
+//     into the kernel's operand order once, at construction.
+#pragma once
+
+#include <algorithm>
+#include <cmath>
+
+#include "Layer.hpp"
+
+namespace small
+{
+
+namespace detail
+{
+
+// the quantisation fields travel with a QUInt8Buffer's data; a float buffer has none
+inline void copy_quant(QUInt8Buffer const &from, QUInt8Buffer &to)
+{
+    to.scale = from.scale;
+    to.offset = from.offset;
+    to.multiplier = from.multiplier;
+    to.lshift = from.lshift;
+    to.rshift = from.rshift;
+    to.m_zero = from.m_zero;
+    to.min_val = from.min_val;
+    to.max_val = from.max_val;
+    to.b = from.b;
+}
+inline void copy_quant(FloatBuffer const &, FloatBuffer &) {}
+
+// batch-normalisation statistics handed to a constructor; all four empty = none
+template <class BufferT>
+struct BatchNormRefs
+{
+    BufferT const &weight, &bias, &mean, &variance;
+    float eps;
+    bool any() const { return weight.size() || bias.size() || mean.size() || variance.size(); }
+    bool all_sized(size_t n) const
+    {
+        return weight.size() == n && bias.size() == n && mean.size() == n && variance.size() == n;
+    }
+};
+
+// Fills packed_filters ([Co/16][Ci/cib][kh][kw][cib][16], Co = num_output_channels, rows past
+// num_effective_output_channels zero) and packed_bias (empty, or Co long) from the caller's buffers and
+// folds the batch normalisation into both:
+//     scale = gamma / sqrt(var + eps);  filter[co] *= scale;
+//     bias[co] = beta - mean * scale               (no bias given)
+//              = beta + scale * (bias[co] - mean)  (bias given)
+// the reference's initialize_conv2d_buffers (Conv2DLayer.hpp:135-341) with the same float expressions.
+// `who` is the message prefix ("*Conv2DLayer" there).  Depthwise filters: num_input_channels = 1 and
+// depthwise = true (tensor type FILTER_DW).
+template <class BufferT>
+void build_conv_weights(std::string const &who, bool depthwise, uint32_t num_output_channels,
+                        uint32_t num_effective_output_channels, uint32_t num_input_channels, uint32_t kernel_height,
+                        uint32_t kernel_width, BufferT const &filters, BufferT const &bias,
+                        BatchNormRefs<BufferT> const &bn, bool buffers_are_packed, BufferT &packed_filters,
+                        BufferT &packed_bias)
+{
+    typedef typename BufferT::value_type T;
+    const size_t taps = (size_t)num_input_channels * kernel_height * kernel_width;
+    if (filters.size() != num_effective_output_channels * taps)
+        throw std::invalid_argument(who + "::ctor ERROR: filters buffer is incorrect size.");
+    const size_t packed_size = (size_t)num_output_channels * taps;
+    const BufferTypeEnum ftype = depthwise ? FILTER_DW : FILTER_CONV;
+    const uint32_t cib = depthwise ? 1U : BufferT::C_ib;
+
+    if (buffers_are_packed)
+    {
+        if (num_output_channels != num_effective_output_channels)
+            throw std::invalid_argument("Conv2DLayer::ctor error: invalid number of output channels.");
+        packed_filters = filters;
+    }
+    else
+    {
+        // zero rows up to the padded channel count, then one pack on the device
+        BufferT flat(packed_size);
+        T *f = flat.data();
+        std::copy(filters.data(), filters.data() + filters.size(), f);
+        std::fill(f + filters.size(), f + packed_size, T(0));
+        BufferT packed(packed_size);
+        pack_buffer(flat, ftype, num_output_channels, num_input_channels, kernel_height, kernel_width, BufferT::C_ib,
+                    BufferT::C_ob, packed);
+        packed_filters = std::move(packed);
+        copy_quant(filters, packed_filters);   // the packed copy keeps the filter's zero point
+    }
+
+    if (bias.size() > 0)
+    {
+        if (bias.size() != num_effective_output_channels)
+            throw std::invalid_argument(who + "::ctor ERROR: bias buffer incorrect size.");
+        BufferT local(num_output_channels);
+        std::fill(local.data(), local.data() + num_output_channels, T(0));
+        std::copy(bias.data(), bias.data() + num_effective_output_channels, local.data());
+        packed_bias = std::move(local);
+    }
+
+    if (!bn.any()) return;
+    if (!bn.all_sized(num_effective_output_channels))
+        throw std::invalid_argument(who + "::ctor ERROR: BN buffers incorrect size.");
+    const bool no_bias = packed_bias.size() == 0;
+    if (no_bias)
+    {
+        BufferT zeros(num_output_channels);
+        std::fill(zeros.data(), zeros.data() + num_output_channels, T(0));
+        packed_bias = std::move(zeros);
+    }
+    T *pf = packed_filters.data();
+    T *pb = packed_bias.data();
+    for (size_t co = 0; co < num_effective_output_channels; ++co)
+    {
+        const float rsq = 1.0f / std::sqrt(bn.variance[co] + bn.eps);
+        const float filter_scale = bn.weight[co] * rsq;
+        if (no_bias) pb[co] = bn.bias[co] - bn.mean[co] * filter_scale;
+        else pb[co] = bn.bias[co] + filter_scale * (pb[co] - bn.mean[co]);
+        for (size_t ci = 0; ci < num_input_channels; ++ci)
+            for (size_t fh = 0; fh < kernel_height; ++fh)
+                for (size_t fw = 0; fw < kernel_width; ++fw)
+                    pf[packed_weight_index(num_output_channels, num_input_channels, kernel_height, kernel_width,
+                                           BufferT::C_ob, cib, co, ci, fh, fw)] *= filter_scale;
+    }
+}
+
+// quantised filters in the convolution kernel's operand order (device memory owned by the layer)
+class PreparedFilter
+{
+public:
+    PreparedFilter() = default;
+    PreparedFilter(PreparedFilter const &) = delete;
+    PreparedFilter &operator=(PreparedFilter const &) = delete;
+    ~PreparedFilter() { if (m_dev) small_hip_free(m_dev); }
+
+    // no-op unless the element type is uint8 and the kernel supports the shape (Ci % 16 == 0)
+    template <class BufferT>
+    void build(uint32_t kh, uint32_t kw, uint32_t Co, uint32_t Ci, BufferT const &packed_filters)
+    {
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            if (Ci % QUInt8Buffer::C_ib != 0) return;
+            const size_t bytes = small_hip_conv2d_u8_prepared_filter_bytes(kh, kw, Co, Ci);
+            if (bytes == 0) return;
+            hip_check(small_hip_malloc(&m_dev, bytes), "prepared filter allocation");
+            hip_check(small_hip_conv2d_u8_prepare_filter(kh, kw, Co, Ci, packed_filters.device_in(), m_dev,
+                                                         current_stream()),
+                      "small_hip_conv2d_u8_prepare_filter");
+        }
+    }
+    void const *get() const { return m_dev; }
+
+private:
+    void *m_dev = nullptr;
+};
+
+inline void reject_softmax(ActivationType a, char const *who)
+{
+    if (a == SOFTMAX)
+        throw std::invalid_argument(std::string(who) + "::ctor ERROR: SOFTMAX activation is not part of this build.");
+}
+
+// padded output channel count, or the reference's error when packed buffers do not allow padding
+template <class BufferT>
+uint32_t padded_output_channels(uint32_t num_output_channels, bool buffers_are_packed)
+{
+    const uint32_t rem = num_output_channels % BufferT::C_ob;
+    if (rem == 0) return num_output_channels;
+    if (buffers_are_packed)
+        throw std::invalid_argument("Conv2DLayer::ctor ERROR: invalid number of output channels.");
+    return num_output_channels + (BufferT::C_ob - rem);
+}
+
+} // namespace detail
+
+//****************************************************************************
+template <typename BufferT>
+class Conv2DLayer : public Layer<BufferT>
+{
+public:
+    typedef typename BufferT::value_type value_type;
+
+    Conv2DLayer(shape_type const &input_shape, uint32_t kernel_height, uint32_t kernel_width, uint32_t stride,
+                PaddingEnum padding_type, uint32_t num_output_channels, BufferT const &filters,
+                bool buffers_are_packed = true, ActivationType activation_type = NONE, float leaky_slope = 1.e-2)
+        : Conv2DLayer(input_shape, kernel_height, kernel_width, stride, padding_type, num_output_channels, filters,
+                      BufferT(), BufferT(), BufferT(), BufferT(), BufferT(), 0.f, buffers_are_packed,
+                      activation_type, leaky_slope)
+    {
+    }
+
+    Conv2DLayer(shape_type const &input_shape, uint32_t kernel_height, uint32_t kernel_width, uint32_t stride,
+                PaddingEnum padding_type, uint32_t num_output_channels, BufferT const &filters, BufferT const &bias,
+                bool buffers_are_packed = true, ActivationType activation_type = NONE, float leaky_slope = 1.e-2)
+        : Conv2DLayer(input_shape, kernel_height, kernel_width, stride, padding_type, num_output_channels, filters,
+                      bias, BufferT(), BufferT(), BufferT(), BufferT(), 0.f, buffers_are_packed, activation_type,
+                      leaky_slope)
+    {
+    }
+
+    Conv2DLayer(shape_type const &input_shape, uint32_t kernel_height, uint32_t kernel_width, uint32_t stride,
+                PaddingEnum padding_type, uint32_t num_output_channels, BufferT const &filters,
+                BufferT const &bn_weight, BufferT const &bn_bias, BufferT const &bn_running_mean,
+                BufferT const &bn_running_variance, float const &bn_eps = 1.e-3, bool buffers_are_packed = true,
+                ActivationType activation_type = NONE, float leaky_slope = 1.e-2)
+        : Conv2DLayer(input_shape, kernel_height, kernel_width, stride, padding_type, num_output_channels, filters,
+                      BufferT(), bn_weight, bn_bias, bn_running_mean, bn_running_variance, bn_eps,
+                      buffers_are_packed, activation_type, leaky_slope)
+    {
+    }
+
+    Conv2DLayer(shape_type const &input_shape, uint32_t kernel_height, uint32_t kernel_width, uint32_t stride,
+                PaddingEnum padding_type, uint32_t num_output_channels, BufferT const &filters, BufferT const &bias,
+                BufferT const &bn_weight, BufferT const &bn_bias, BufferT const &bn_running_mean,
+                BufferT const &bn_running_variance, float const &bn_eps = 1.e-3, bool buffers_are_packed = true,
+                ActivationType activation_type = NONE, float leaky_slope = 1.e-2)
+        : Layer<BufferT>(),
+          m_input_shape(input_shape),
+          m_window(input_shape, kernel_height, kernel_width, stride, padding_type),
+          m_effective_output_channels(num_output_channels),
+          m_activation_type(activation_type),
+          m_slope(leaky_slope)
+    {
+        detail::reject_softmax(activation_type, "Conv2DLayer");
+        // 1 and 2 input channels are accepted like 3: small::Conv2D takes all three (the reference's layer
+        // class only lets 3 through)
+        if ((input_shape[CHANNEL] % BufferT::C_ib) != 0 && (input_shape[CHANNEL] == 0 || input_shape[CHANNEL] > 3))
+            throw std::invalid_argument("Conv2DLayer::ctor ERROR: invalid number of input channels.");
+        const uint32_t Co = detail::padded_output_channels<BufferT>(num_output_channels, buffers_are_packed);
+        this->set_output_shape({input_shape[BATCH], Co, m_window.Ho, m_window.Wo});
+        detail::build_conv_weights("*Conv2DLayer", false, Co, m_effective_output_channels,
+                                   (uint32_t)input_shape[CHANNEL], kernel_height, kernel_width, filters, bias,
+                                   detail::BatchNormRefs<BufferT>{bn_weight, bn_bias, bn_running_mean,
+                                                                  bn_running_variance, bn_eps},
+                                   buffers_are_packed, m_packed_filters, m_packed_bias);
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            if (m_packed_bias.size() > 0 || activation_type == LEAKY)
+                throw std::invalid_argument(
+                    "Conv2DLayer::ctor ERROR: bias / LeakyReLU have no quantised implementation.");
+        }
+        m_prepared.build(kernel_height, kernel_width, Co, (uint32_t)input_shape[CHANNEL], m_packed_filters);
+    }
+
+    virtual ~Conv2DLayer() {}
+
+    uint32_t get_effective_output_channels() const { return m_effective_output_channels; }
+    BufferT const &get_packed_filters() const { return m_packed_filters; }
+    BufferT const &get_packed_bias() const { return m_packed_bias; }
+
+    virtual void compute_output(std::vector<Tensor<BufferT> const *> input, Tensor<BufferT> *output) const
+    {
+        this->check_single_input("Conv2DLayer", input, m_input_shape, output);
+        auto const &os = this->output_shape();
+        const int batch = (int)m_input_shape[BATCH];
+        if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        {
+            batched::Conv2D_Bias_Act(batch, m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b,
+                                     m_window.l, m_window.r, (int)os[CHANNEL], (int)m_input_shape[CHANNEL],
+                                     (int)m_input_shape[HEIGHT], (int)m_input_shape[WIDTH], input[0]->buffer(),
+                                     m_packed_filters, m_packed_bias, m_activation_type, m_slope, output->buffer());
+        }
+        else
+        {
+            batched::Conv2D_Accum_ReLU(batch, m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b,
+                                       m_window.l, m_window.r, (int)os[CHANNEL], (int)m_input_shape[CHANNEL],
+                                       (int)m_input_shape[HEIGHT], (int)m_input_shape[WIDTH], input[0]->buffer(),
+                                       m_packed_filters, m_prepared.get(), (BufferT const *)nullptr,
+                                       m_activation_type == RELU, output->buffer());
+        }
+        output->set_shape(os);
+    }
+
+private:
+    shape_type const m_input_shape;
+    detail::Window const m_window;
+    uint32_t const m_effective_output_channels;
+    ActivationType const m_activation_type;
+    float const m_slope;
+    BufferT m_packed_filters;
+    BufferT m_packed_bias;
+    detail::PreparedFilter m_prepared;
+};
+
+} // namespace small

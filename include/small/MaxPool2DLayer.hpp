@@ -1,0 +1,42 @@
+// MaxPool2DLayer: window maximum (padding counts as zero-valued pixels) over the window geometry of the padding type (same constructor, checks
+// and messages as the reference's include/small/MaxPool2DLayer.hpp:24-116); the batch extent of the
+// input shape is honoured.
+#pragma once
+
+#include "Layer.hpp"
+
+namespace small
+{
+
+template <typename BufferT>
+class MaxPool2DLayer : public Layer<BufferT>
+{
+public:
+    typedef typename BufferT::value_type value_type;
+
+    MaxPool2DLayer(shape_type const &input_shape, uint32_t kernel_height, uint32_t kernel_width, uint32_t stride,
+                  PaddingEnum padding_type)
+        : Layer<BufferT>(),
+          m_input_shape(input_shape),
+          m_window(input_shape, kernel_height, kernel_width, stride, padding_type)
+    {
+        this->set_output_shape({input_shape[BATCH], input_shape[CHANNEL], m_window.Ho, m_window.Wo});
+    }
+
+    virtual ~MaxPool2DLayer() {}
+
+    virtual void compute_output(std::vector<Tensor<BufferT> const *> input, Tensor<BufferT> *output) const
+    {
+        this->check_single_input("MaxPool2DLayer", input, m_input_shape, output);
+        batched::MaxPool2D((int)m_input_shape[BATCH], m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b,
+                      m_window.l, m_window.r, (int)m_input_shape[CHANNEL], (int)m_input_shape[HEIGHT],
+                      (int)m_input_shape[WIDTH], input[0]->buffer(), output->buffer());
+        output->set_shape(this->output_shape());
+    }
+
+private:
+    shape_type const m_input_shape;
+    detail::Window const m_window;
+};
+
+} // namespace small

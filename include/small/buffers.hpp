@@ -9,7 +9,10 @@
 #include <cstdlib>
 #include <iostream>
 #include <stdexcept>
+#include <string>
 #include <type_traits>
+
+#include "Buffer.hpp"
 
 namespace small
 {
@@ -113,20 +116,46 @@ uint32_t convert_dc2tensor(ScalarT const *dc_array, BufferTypeEnum type, uint32_
                                [&](size_t p, size_t f) { flat_t[f] = dc_array[p]; });
 }
 
+namespace detail
+{
+// pack_buffer / unpack_buffer run on the device (small_hip_pack / small_hip_unpack): the source is
+// uploaded if its newest copy is on the host, the result stays on the device for the layer call that
+// follows.  An unknown tensor type prints the reference's message and returns 0 as the reference does;
+// extents that do not fill their channel blocks (the reference then indexes past the tensor) throw.
+template <class BufferT, class Fn>
+uint32_t repack_on_device(Fn fn, BufferT const &src, BufferTypeEnum type, uint32_t dim0, uint32_t dim1,
+                          uint32_t dim2, uint32_t dim3, uint32_t c_ib, uint32_t c_ob, BufferT &dst, char const *who)
+{
+    if (type < INPUT || type > FILTER_FC)
+    {
+        std::printf("ERROR: unsupported tensor buffer type\n");
+        return 0;
+    }
+    const size_t n = (size_t)dim0 * dim1 * (type == FILTER_FC ? 1 : (size_t)dim2 * dim3);
+    if (n == 0) return 0;
+    if (src.size() < n || dst.size() < n) throw std::invalid_argument(std::string(who) + " ERROR: buffer too small.");
+    const int rc = fn((int)type, 1, dim0, dim1, dim2, dim3, c_ib, c_ob, src.device_in(), dst.device_out(),
+                      sizeof(typename BufferT::value_type), current_stream());
+    if (rc == SMALL_HIP_EINVAL) throw std::invalid_argument(std::string(who) + " ERROR: " + small_hip_last_error());
+    hip_check(rc, who);
+    return (uint32_t)((size_t)dim0 * dim1 * dim2 * dim3);
+}
+} // namespace detail
+
 template <class BufferT>
 uint32_t pack_buffer(BufferT const &flat_t, BufferTypeEnum type, uint32_t dim0, uint32_t dim1, uint32_t dim2,
                      uint32_t dim3, uint32_t _C_ib, uint32_t _C_ob, BufferT &dc_array)
 {
-    return convert_tensor2dc<typename BufferT::value_type>(flat_t.data(), type, dim0, dim1, dim2, dim3, _C_ib,
-                                                           _C_ob, dc_array.data());
+    return detail::repack_on_device(small_hip_pack, flat_t, type, dim0, dim1, dim2, dim3, _C_ib, _C_ob, dc_array,
+                                    "pack_buffer");
 }
 
 template <class BufferT>
 uint32_t unpack_buffer(BufferT const &dc_array, BufferTypeEnum type, uint32_t dim0, uint32_t dim1,
                        uint32_t dim2, uint32_t dim3, uint32_t _C_ib, uint32_t _C_ob, BufferT &flat_t)
 {
-    return convert_dc2tensor<typename BufferT::value_type>(dc_array.data(), type, dim0, dim1, dim2, dim3, _C_ib,
-                                                           _C_ob, flat_t.data());
+    return detail::repack_on_device(small_hip_unpack, dc_array, type, dim0, dim1, dim2, dim3, _C_ib, _C_ob, flat_t,
+                                    "unpack_buffer");
 }
 
 //****************************************************************************

@@ -31,7 +31,8 @@ enum ActivationType
 {
     NONE = SMALL_HIP_ACT_NONE,
     RELU = SMALL_HIP_ACT_RELU,
-    LEAKY = SMALL_HIP_ACT_LEAKY
+    LEAKY = SMALL_HIP_ACT_LEAKY,
+    SOFTMAX = 3   // named by the reference's Layer classes; SoftMax itself is not part of this build
 };
 
 namespace detail
@@ -124,6 +125,53 @@ void Conv2D_Bias_Act(int batch, int kernel_height, int kernel_width, int stride,
                                       bias_buf.size() ? bias_buf.device_in() : nullptr, (int)act, negative_slope,
                                       output_buf.device_out(), detail::st()),
         "Conv2D_Bias_Act");
+}
+
+// out = act((out + conv(in, filter)) + bias): PartialConv2D + PartialBias + activation in one pass
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialConv2D_Bias_Act(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad,
+                            uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels,
+                            int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                            BufferT const &bias_buf, ActivationType act, float negative_slope, BufferT &output_buf)
+{
+    detail::raise<BufferT>(
+        small_hip_partial_conv2d_bias_act_f32(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                              r_pad, output_channels, input_channels, input_height, input_width,
+                                              input_buf.device_in(), filter_buf.device_in(),
+                                              bias_buf.size() ? bias_buf.device_in() : nullptr, (int)act,
+                                              negative_slope, output_buf.device_out(), detail::st()),
+        "PartialConv2D_Bias_Act");
+}
+
+// Conv2D [+ Accum(accum_buf, out)] [+ ReLU] on the quantised path in one launch, bit-identical to the
+// separate calls; accum_buf may be null.  `prepared` (may be null) is the filter in the form
+// small_hip_conv2d_u8_prepare_filter writes; with it the per-call filter pre-pass is skipped.
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void Conv2D_Accum_ReLU(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                       uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels, int input_height,
+                       int input_width, BufferT const &input_buf, BufferT const &filter_buf, void const *prepared,
+                       BufferT const *accum_buf, bool relu, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), fq = filter_buf.quant(), oq = output_buf.quant();
+    small_hip_quant aq = oq;
+    uint8_t const *acc = nullptr;
+    if (accum_buf)
+    {
+        aq = accum_buf->quant();
+        acc = accum_buf->device_in();
+    }
+    int rc;
+    if (prepared)
+        rc = small_hip_conv2d_accum_relu_u8_prepared(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad,
+                                                     r_pad, output_channels, input_channels, input_height,
+                                                     input_width, input_buf.device_in(), &iq, prepared, &fq, acc,
+                                                     &aq, relu ? 1 : 0, output_buf.device_out(), &oq, detail::st());
+    else
+        rc = small_hip_conv2d_accum_relu_u8(batch, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad,
+                                            output_channels, input_channels, input_height, input_width,
+                                            input_buf.device_in(), &iq, filter_buf.device_in(), &fq, acc, &aq,
+                                            relu ? 1 : 0, output_buf.device_out(), &oq, detail::st());
+    detail::raise<BufferT>(rc, "Conv2D");
 }
 
 // ---- DepthwiseConv2D / PartialDepthwiseConv2D ------------------------------------------------------

@@ -106,6 +106,14 @@ int small_hip_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width
                                   int input_channels, int input_height, int input_width,
                                   const float *input, const float *filter, const float *bias,
                                   int act, float slope, float *output, small_hip_stream_t stream);
+/* PartialConv2DLayer::compute_output (include/small/PartialConv2DLayer.hpp:407-463) in one pass:
+ * out = act((out + conv(in, filter)) + bias), i.e. PartialConv2D + PartialBias + activation. */
+int small_hip_partial_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                          int t_pad, int b_pad, int l_pad, int r_pad,
+                                          int output_channels, int input_channels, int input_height,
+                                          int input_width, const float *input, const float *filter,
+                                          const float *bias, int act, float negative_slope,
+                                          float *output, small_hip_stream_t stream);
 /* small::DepthwiseConv2D<FloatBuffer>         interface.hpp:138-145, interface_abstract.hpp:994-1051 */
 int small_hip_depthwise_conv2d_f32(int batch, int kernel_height, int kernel_width, int stride,
                                    int t_pad, int b_pad, int l_pad, int r_pad, int input_channels,
@@ -255,6 +263,27 @@ int small_hip_avgpool2d_u8(int batch, int kernel_height, int kernel_width, int s
                            int input_width, const uint8_t *input, const small_hip_quant *input_q,
                            uint8_t *output, const small_hip_quant *output_q,
                            small_hip_stream_t stream);
+
+/* small::pack_buffer / unpack_buffer (convert_tensor2dc / convert_dc2tensor)
+ * include/small/buffers.hpp:138-283, on the device: a flat [dim0][dim1][dim2][dim3] tensor (NCHW
+ * activations with dim0 = 1, OIHW filters) to / from the packed layout.  type is one of
+ * SMALL_HIP_INPUT .. SMALL_HIP_FILTER_FC with the reference's BufferTypeEnum meaning and the same
+ * adjustments (FILTER_DW: c_ib = 1; FILTER_FC: dim2 = dim3 = 1; INPUT / FILTER_CONV with
+ * dim1 < c_ib: c_ib = dim1).  element_size is 4 (float) or 1 (uint8).  batch consecutive tensors are
+ * converted in one launch (no counterpart in the reference: its buffers hold one image).
+ * SMALL_HIP_EINVAL where the reference prints an error and returns 0 (unknown type) or would index
+ * past the tensor (extents that are not multiples of their block). */
+#define SMALL_HIP_INPUT 0
+#define SMALL_HIP_OUTPUT 1
+#define SMALL_HIP_FILTER_DW 2
+#define SMALL_HIP_FILTER_CONV 3
+#define SMALL_HIP_FILTER_FC 4
+int small_hip_pack(int type, int batch, uint32_t dim0, uint32_t dim1, uint32_t dim2, uint32_t dim3,
+                   uint32_t c_ib, uint32_t c_ob, const void *flat, void *packed, size_t element_size,
+                   small_hip_stream_t stream);
+int small_hip_unpack(int type, int batch, uint32_t dim0, uint32_t dim1, uint32_t dim2, uint32_t dim3,
+                     uint32_t c_ib, uint32_t c_ob, const void *packed, void *flat, size_t element_size,
+                     small_hip_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -25,6 +25,23 @@
 #include <omp.h>
 
 #include <small.h>
+#include <small/Conv2DLayer.hpp>
+#include <small/PartialConv2DLayer.hpp>
+#include <small/DepthwiseConv2DLayer.hpp>
+#include <small/MaxPool2DLayer.hpp>
+#include <small/AveragePool2DLayer.hpp>
+#include <small/ReLULayer.hpp>
+#include <small/LeakyReLULayer.hpp>
+#include <small/UpSample2DLayer.hpp>
+#include <small/AddLayer.hpp>
+#include <small/RouteLayer.hpp>
+#include <small/models/MobileNetTiny.hpp>
+#include <small/models/Resnet8Tiny.hpp>
+#include <small/models/DSCNNTiny.hpp>
+#include <small/models/TinyYoloV2.hpp>
+
+#include <memory>
+#include <vector>
 
 namespace {
 thread_local std::string g_err;
@@ -232,5 +249,145 @@ int sref_dense_u8(int No, int Ni, void *in, void *filt, void *out)
     return guarded([&] { small::Dense(No, Ni, Q(in), Q(filt), Q(out)); });
 }
 #endif // quint8
+
+// ---- Layer and Model classes (float) -----------------------------------------
+// The reference's own Layer / Model objects on flat (NCHW / OIHW, unpacked) data: the shim packs the
+// input for this platform's blocking, runs compute_output() / inference() and unpacks the result, so
+// the REF and ZEN2 builds can be compared with each other and with other implementations.
+#if defined(SMALL_HAS_FLOAT_SUPPORT)
+} // extern "C"
+namespace {
+FB fb_from(const float *p, size_t n)
+{
+    FB b(n);
+    if (n) std::memcpy(b.data(), p, n * sizeof(float));
+    return b;
+}
+small::Tensor<FB> packed_tensor(const float *flat, small::shape_type const &shape)
+{
+    const size_t n = small::compute_size(shape);
+    FB f = fb_from(flat, n), p(n);
+    small::pack_buffer(f, small::INPUT, 1U, shape[1], shape[2], shape[3], FB::C_ib, FB::C_ob, p);
+    return small::Tensor<FB>(shape, std::move(p));
+}
+void unpack_tensor(small::Tensor<FB> const &t, float *flat, int *out_shape)
+{
+    auto const &s = t.shape();
+    for (int i = 0; i < 4; ++i) out_shape[i] = (int)s[i];
+    const size_t n = small::compute_size(s);
+    FB p(n), f(n);
+    std::memcpy(p.data(), t.buffer().data(), n * sizeof(float));
+    small::unpack_buffer(p, small::OUTPUT, 1U, s[1], s[2], s[3], FB::C_ib, FB::C_ob, f);
+    std::memcpy(flat, f.data(), n * sizeof(float));
+}
+} // namespace
+extern "C" {
+
+// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer; batch 1 (the reference computes one
+// image).  filters [Co][Ci][kh][kw] (depthwise [C][kh][kw]); bias Co or NULL; bn 4 x Co (gamma, beta, mean,
+// variance) or NULL; out is in/out, flat [Co_padded][Ho][Wo].
+int sref_conv_layer_f32(int kind, int C, int H, int W, int kh, int kw, int stride, int padding, int Co,
+                        const float *filters, const float *bias, const float *bn, float eps, int act, float slope,
+                        const float *in, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{1UL, (size_t)C, (size_t)H, (size_t)W};
+        const size_t nf = (kind == 2 ? (size_t)C : (size_t)Co * C) * kh * kw;
+        const size_t nb = kind == 2 ? C : Co;
+        FB f = fb_from(filters, nf), b = bias ? fb_from(bias, nb) : FB();
+        FB g, be, mu, var;
+        if (bn) { g = fb_from(bn, nb); be = fb_from(bn + nb, nb); mu = fb_from(bn + 2 * nb, nb); var = fb_from(bn + 3 * nb, nb); }
+        const auto pad = padding ? small::PADDING_F : small::PADDING_V;
+        const auto a = (small::ActivationType)act;
+        std::unique_ptr<small::Layer<FB>> layer;
+        if (kind == 2)
+        {
+            if (bn) layer.reset(new small::DepthwiseConv2DLayer<FB>(is, kh, kw, stride, pad, f, b, g, be, mu, var, eps, false, a, slope));
+            else if (bias) layer.reset(new small::DepthwiseConv2DLayer<FB>(is, kh, kw, stride, pad, f, b, false, a, slope));
+            else layer.reset(new small::DepthwiseConv2DLayer<FB>(is, kh, kw, stride, pad, f, false, a, slope));
+        }
+        else if (kind == 1)
+        {
+            if (bn) layer.reset(new small::PartialConv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, b, g, be, mu, var, eps, false, a, slope));
+            else if (bias) layer.reset(new small::PartialConv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, b, false, a, slope));
+            else layer.reset(new small::PartialConv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, false, a, slope));
+        }
+        else
+        {
+            if (bn) layer.reset(new small::Conv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, b, g, be, mu, var, eps, false, a, slope));
+            else if (bias) layer.reset(new small::Conv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, b, false, a, slope));
+            else layer.reset(new small::Conv2DLayer<FB>(is, kh, kw, stride, pad, Co, f, false, a, slope));
+        }
+        auto x = packed_tensor(in, is);
+        auto y = packed_tensor(out, layer->output_shape());
+        layer->compute_output({&x}, &y);
+        unpack_tensor(y, out, out_shape);
+    });
+}
+
+// kind: 0 MaxPool2DLayer, 1 AveragePool2DLayer, 2 ReLULayer, 3 LeakyReLULayer(slope), 4 UpSample2DLayer(k = scale),
+// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels)
+int sref_simple_layer_f32(int kind, int C, int H, int W, int k, int kw, int stride, int padding, float slope,
+                          const float *in, const float *in2, int C2, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{1UL, (size_t)C, (size_t)H, (size_t)W};
+        const small::shape_type is2{1UL, (size_t)C2, (size_t)H, (size_t)W};
+        const auto pad = padding ? small::PADDING_F : small::PADDING_V;
+        std::unique_ptr<small::Layer<FB>> layer;
+        switch (kind)
+        {
+        case 0: layer.reset(new small::MaxPool2DLayer<FB>(is, k, kw, stride, pad)); break;
+        case 1: layer.reset(new small::AveragePool2DLayer<FB>(is, k, kw, stride, pad)); break;
+        case 2: layer.reset(new small::ReLULayer<FB>(is)); break;
+        case 3: layer.reset(new small::LeakyReLULayer<FB>(is, slope)); break;
+        case 4: layer.reset(new small::UpSample2DLayer<FB>(is, k)); break;
+        case 5: layer.reset(new small::AddLayer<FB>(is, is)); break;
+        case 6: layer.reset(new small::RouteLayer<FB>(is)); break;
+        case 7: layer.reset(new small::RouteLayer<FB>(is, is2)); break;
+        default: throw std::invalid_argument("sref_simple_layer_f32: unknown kind");
+        }
+        auto x = packed_tensor(in, is);
+        auto y = packed_tensor(out, layer->output_shape());
+        if (kind == 7)
+        {
+            auto x2 = packed_tensor(in2, is2);
+            layer->compute_output({&x, &x2}, &y);
+        }
+        else
+            layer->compute_output({&x}, &y);
+        unpack_tensor(y, out, out_shape);
+    });
+}
+
+// which: 0 MobileNetTiny, 1 Resnet8Tiny, 2 DSCNNTiny, 3 TinyYoloV2 as the reference defines them;
+// filters unpacked, in the model's own filter order.
+int sref_model_f32(int which, int C, int H, int W, const float *const *filters, const size_t *sizes, int nfilters,
+                   const float *in, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{1UL, (size_t)C, (size_t)H, (size_t)W};
+        std::vector<std::unique_ptr<FB>> own;
+        std::vector<FB *> fl;
+        for (int i = 0; i < nfilters; ++i)
+        {
+            own.emplace_back(new FB(fb_from(filters[i], sizes[i])));
+            fl.push_back(own.back().get());
+        }
+        std::unique_ptr<small::Model<FB>> m;
+        switch (which)
+        {
+        case 0: m.reset(new small::MobileNetTiny<FB>(is, fl, false)); break;
+        case 1: m.reset(new small::Resnet8Tiny<FB>(is, fl, false)); break;
+        case 2: m.reset(new small::DSCNNTiny<FB>(is, fl, false)); break;
+        case 3: m.reset(new small::TinyYoloV2<FB>(is, fl, false)); break;
+        default: throw std::invalid_argument("sref_model_f32: unknown model");
+        }
+        auto x = packed_tensor(in, is);
+        auto outs = m->inference(&x);
+        unpack_tensor(*outs[0], out, out_shape);
+    });
+}
+#endif // float layers
 
 } // extern "C"

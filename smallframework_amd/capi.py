@@ -55,6 +55,7 @@ SIGNATURES = {
     "small_hip_conv2d_f32": (_i, _conv + [_p, _p, _p, _p]),
     "small_hip_partial_conv2d_f32": (_i, _conv + [_p, _p, _p, _p]),
     "small_hip_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
+    "small_hip_partial_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_partial_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_depthwise_conv2d_bias_act_f32": (_i, _win + [_p, _p, _p, _i, _f, _p, _p]),
@@ -81,6 +82,8 @@ SIGNATURES = {
     "small_hip_dense_u8": (_i, [_i] * 3 + [_p, _q, _p, _q, _p, _q, _p]),
     "small_hip_accum_u8": (_i, [_i] * 4 + [_p, _q, _p, _q, _p]),
     "small_hip_avgpool2d_u8": (_i, _win + [_p, _q, _p, _q, _p]),
+    "small_hip_pack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
+    "small_hip_unpack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
 }
 
 _lib = None

@@ -846,6 +846,15 @@ int small_hip_conv2d_bias_act_f32(int batch, int kh, int kw, int stride, int pt,
                     filt, bias, act, slope, 0, out, stream);
 }
 
+int small_hip_partial_conv2d_bias_act_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                          int Co, int Ci, int H, int W, const float *in, const float *filt,
+                                          const float *bias, int act, float slope, float *out,
+                                          small_hip_stream_t stream)
+{
+    return conv_f32("small_hip_partial_conv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W,
+                    in, filt, bias, act, slope, 1, out, stream);
+}
+
 int small_hip_dense_f32(int batch, int No, int Ni, const float *in, const float *filt, float *out,
                         small_hip_stream_t stream)
 {

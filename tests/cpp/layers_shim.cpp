@@ -1,0 +1,270 @@
+// Test-only C entry points around the C++ Layer / Model classes of include/small/ so that the
+// Python parity tests can drive them with numpy data (built by tests/test_cpp_layers.py with g++,
+// linked against libsmall_hip.so).  oracle/ref_shim.cpp exports the same functions (prefix sref_)
+// around the reference's own classes; the two are compared through the oracle.
+//
+// Tensors cross this boundary flat (NCHW / OIHW, unpacked): the shim packs inputs and unpacks
+// outputs with pack_buffer / unpack_buffer, as a user of the Layer API would.
+// Return value: 0 ok, 1 std::invalid_argument, 2 any other exception; stest_last_error() has the text.
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include <small.h>
+#include <small/AddLayer.hpp>
+#include <small/AveragePool2DLayer.hpp>
+#include <small/Conv2DLayer.hpp>
+#include <small/DepthwiseConv2DLayer.hpp>
+#include <small/DummyLayer.hpp>
+#include <small/LeakyReLULayer.hpp>
+#include <small/MaxPool2DLayer.hpp>
+#include <small/PartialConv2DLayer.hpp>
+#include <small/ReLULayer.hpp>
+#include <small/RouteLayer.hpp>
+#include <small/UpSample2DLayer.hpp>
+#include <small/models/DSCNNTiny.hpp>
+#include <small/models/MobileNetTiny.hpp>
+#include <small/models/Resnet8Tiny.hpp>
+#include <small/models/TinyYoloV2.hpp>
+
+namespace
+{
+thread_local std::string g_err;
+
+template <class Fn>
+int guarded(Fn &&fn)
+{
+    try { fn(); return 0; }
+    catch (std::invalid_argument const &e) { g_err = e.what(); return 1; }
+    catch (std::exception const &e) { g_err = e.what(); return 2; }
+    catch (...) { g_err = "unknown exception"; return 2; }
+}
+
+template <class BufferT>
+BufferT from_host(typename BufferT::value_type const *p, size_t n)
+{
+    BufferT b(n);
+    if (n) std::memcpy(b.data(), p, n * sizeof(typename BufferT::value_type));
+    return b;
+}
+
+// flat [batch][C][H][W] -> packed tensor of that shape
+template <class BufferT>
+small::Tensor<BufferT> packed_tensor(typename BufferT::value_type const *flat, small::shape_type const &shape,
+                                     size_t capacity = 0)
+{
+    const size_t per = shape[1] * shape[2] * shape[3], n = shape[0] * per;
+    BufferT f = from_host<BufferT>(flat, n);
+    BufferT p(std::max(n, capacity));
+    // one call per image keeps this independent of the library's batched pack
+    for (size_t i = 0; i < shape[0]; ++i)
+    {
+        BufferT fi = from_host<BufferT>(flat + i * per, per), pi(per);
+        small::pack_buffer(fi, small::INPUT, 1U, (uint32_t)shape[1], (uint32_t)shape[2], (uint32_t)shape[3],
+                           BufferT::C_ib, BufferT::C_ob, pi);
+        std::memcpy(p.data() + i * per, pi.data(), per * sizeof(typename BufferT::value_type));
+    }
+    return small::Tensor<BufferT>(shape, std::move(p));
+}
+
+template <class BufferT>
+void unpack_tensor(small::Tensor<BufferT> const &t, typename BufferT::value_type *flat, int *out_shape)
+{
+    auto const &s = t.shape();
+    for (int i = 0; i < 4; ++i) out_shape[i] = (int)s[i];
+    const size_t per = s[1] * s[2] * s[3];
+    for (size_t i = 0; i < s[0]; ++i)
+    {
+        BufferT pi(per), fi(per);
+        std::memcpy(pi.data(), t.buffer().data() + i * per, per * sizeof(typename BufferT::value_type));
+        small::unpack_buffer(pi, small::OUTPUT, 1U, (uint32_t)s[1], (uint32_t)s[2], (uint32_t)s[3], BufferT::C_ib,
+                             BufferT::C_ob, fi);
+        std::memcpy(flat + i * per, fi.data(), per * sizeof(typename BufferT::value_type));
+    }
+}
+
+void set_quant(small::QUInt8Buffer &b, int32_t const *q)
+{
+    b.m_zero = q[0];
+    b.multiplier = q[1];
+    b.lshift = q[2];
+    b.rshift = q[3];
+}
+
+// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer
+template <class BufferT>
+std::unique_ptr<small::Layer<BufferT>> make_conv_layer(int kind, small::shape_type const &in_shape, int kh, int kw,
+                                                       int stride, int padding, int Co, BufferT const &filt,
+                                                       BufferT const &bias, BufferT const *bn, float eps, int act,
+                                                       float slope)
+{
+    const auto pad = padding ? small::PADDING_F : small::PADDING_V;
+    const auto a = (small::ActivationType)act;
+    small::Layer<BufferT> *l = nullptr;
+    if (kind == 2)
+    {
+        if (bn) l = new small::DepthwiseConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, filt, bias, bn[0], bn[1], bn[2], bn[3], eps, false, a, slope);
+        else if (bias.size()) l = new small::DepthwiseConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, filt, bias, false, a, slope);
+        else l = new small::DepthwiseConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, filt, false, a, slope);
+    }
+    else if (kind == 1)
+    {
+        if (bn) l = new small::PartialConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, bias, bn[0], bn[1], bn[2], bn[3], eps, false, a, slope);
+        else if (bias.size()) l = new small::PartialConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, bias, false, a, slope);
+        else l = new small::PartialConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, false, a, slope);
+    }
+    else
+    {
+        if (bn) l = new small::Conv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, bias, bn[0], bn[1], bn[2], bn[3], eps, false, a, slope);
+        else if (bias.size()) l = new small::Conv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, bias, false, a, slope);
+        else l = new small::Conv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, Co, filt, false, a, slope);
+    }
+    return std::unique_ptr<small::Layer<BufferT>>(l);
+}
+} // namespace
+
+using FB = small::FloatBuffer;
+using QB = small::QUInt8Buffer;
+
+extern "C"
+{
+
+const char *stest_last_error(void) { return g_err.c_str(); }
+
+// Convolution-type layer on flat data.  filters: [Co][Ci][kh][kw] (depthwise: [C][kh][kw]); bias: Co or
+// NULL; bn: 4 x Co (gamma, beta, mean, variance) or NULL.  out: in/out, flat [batch][Co_padded][Ho][Wo]
+// (read first by the partial layer); out_shape receives the layer's output shape.
+int stest_conv_layer_f32(int kind, int batch, int C, int H, int W, int kh, int kw, int stride, int padding, int Co,
+                         const float *filters, const float *bias, const float *bn, float eps, int act, float slope,
+                         const float *in, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, (size_t)C, (size_t)H, (size_t)W};
+        const size_t nf = (kind == 2 ? (size_t)C : (size_t)Co * C) * kh * kw;
+        const size_t nb = kind == 2 ? C : Co;
+        FB f = from_host<FB>(filters, nf), b = bias ? from_host<FB>(bias, nb) : FB();
+        FB bnb[4];
+        if (bn)
+            for (int i = 0; i < 4; ++i) bnb[i] = from_host<FB>(bn + i * nb, nb);
+        auto layer = make_conv_layer<FB>(kind, is, kh, kw, stride, padding, Co, f, b, bn ? bnb : nullptr, eps, act, slope);
+        auto x = packed_tensor<FB>(in, is);
+        auto y = packed_tensor<FB>(out, layer->output_shape());
+        layer->compute_output({&x}, &y);
+        unpack_tensor<FB>(y, out, out_shape);
+    });
+}
+
+// quantised: q = {zero, multiplier, lshift, rshift} for input, filter, output
+int stest_conv_layer_u8(int kind, int batch, int C, int H, int W, int kh, int kw, int stride, int padding, int Co,
+                        const uint8_t *filters, int act, const uint8_t *in, const int32_t *in_q,
+                        const int32_t *filter_q, const int32_t *out_q, uint8_t *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, (size_t)C, (size_t)H, (size_t)W};
+        const size_t nf = (kind == 2 ? (size_t)C : (size_t)Co * C) * kh * kw;
+        QB f = from_host<QB>(filters, nf);
+        set_quant(f, filter_q);
+        auto layer = make_conv_layer<QB>(kind, is, kh, kw, stride, padding, Co, f, QB(), nullptr, 0.f, act, 0.f);
+        auto x = packed_tensor<QB>(in, is);
+        set_quant(x.buffer(), in_q);
+        auto y = packed_tensor<QB>(out, layer->output_shape());
+        set_quant(y.buffer(), out_q);
+        layer->compute_output({&x}, &y);
+        unpack_tensor<QB>(y, out, out_shape);
+    });
+}
+
+// kind: 0 MaxPool2DLayer, 1 AveragePool2DLayer, 2 ReLULayer, 3 LeakyReLULayer(slope), 4 UpSample2DLayer(k = scale),
+// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels)
+int stest_simple_layer_f32(int kind, int batch, int C, int H, int W, int k, int kw, int stride, int padding,
+                           float slope, const float *in, const float *in2, int C2, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, (size_t)C, (size_t)H, (size_t)W};
+        const small::shape_type is2{(size_t)batch, (size_t)C2, (size_t)H, (size_t)W};
+        const auto pad = padding ? small::PADDING_F : small::PADDING_V;
+        std::unique_ptr<small::Layer<FB>> layer;
+        switch (kind)
+        {
+        case 0: layer.reset(new small::MaxPool2DLayer<FB>(is, k, kw, stride, pad)); break;
+        case 1: layer.reset(new small::AveragePool2DLayer<FB>(is, k, kw, stride, pad)); break;
+        case 2: layer.reset(new small::ReLULayer<FB>(is)); break;
+        case 3: layer.reset(new small::LeakyReLULayer<FB>(is, slope)); break;
+        case 4: layer.reset(new small::UpSample2DLayer<FB>(is, k)); break;
+        case 5: layer.reset(new small::AddLayer<FB>(is, is)); break;
+        case 6: layer.reset(new small::RouteLayer<FB>(is)); break;
+        case 7: layer.reset(new small::RouteLayer<FB>(is, is2)); break;
+        default: throw std::invalid_argument("stest_simple_layer_f32: unknown kind");
+        }
+        auto x = packed_tensor<FB>(in, is);
+        auto y = packed_tensor<FB>(out, layer->output_shape());
+        if (kind == 7)
+        {
+            auto x2 = packed_tensor<FB>(in2, is2);
+            layer->compute_output({&x, &x2}, &y);
+        }
+        else
+            layer->compute_output({&x}, &y);
+        unpack_tensor<FB>(y, out, out_shape);
+    });
+}
+
+// which: 0 MobileNetTiny, 1 Resnet8Tiny, 2 DSCNNTiny, 3 TinyYoloV2, built with the reference's defaults
+// (variant 0) or as the benchmark topology (variant 1: MobileNet 1000 classes + average pooling; ResNet-8
+// 10 classes; DS-CNN 10x4 stem, 12 classes, average pooling; Tiny-YOLOv2 LeakyReLU 0.1 with 125 linear outputs).
+// filters: unpacked, in the model's filter order; sizes[i] elements each.
+int stest_model_f32(int which, int variant, int batch, int C, int H, int W, const float *const *filters,
+                    const size_t *sizes, int nfilters, const float *in, float *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, (size_t)C, (size_t)H, (size_t)W};
+        std::vector<std::unique_ptr<FB>> own;
+        std::vector<FB *> fl;
+        for (int i = 0; i < nfilters; ++i)
+        {
+            own.emplace_back(new FB(from_host<FB>(filters[i], sizes[i])));
+            fl.push_back(own.back().get());
+        }
+        std::unique_ptr<small::Model<FB>> m;
+        switch (which)
+        {
+        case 0: m.reset(variant ? new small::MobileNetTiny<FB>(is, fl, false, 32, 1000, true)
+                                : new small::MobileNetTiny<FB>(is, fl, false)); break;
+        case 1: m.reset(variant ? new small::Resnet8Tiny<FB>(is, fl, false, 10) : new small::Resnet8Tiny<FB>(is, fl, false)); break;
+        case 2: m.reset(variant ? new small::DSCNNTiny<FB>(is, fl, false, 10, 4, 12, true)
+                                : new small::DSCNNTiny<FB>(is, fl, false)); break;
+        case 3: m.reset(variant ? new small::TinyYoloV2<FB>(is, fl, false, small::LEAKY, 0.1f, 125, false)
+                                : new small::TinyYoloV2<FB>(is, fl, false)); break;
+        default: throw std::invalid_argument("stest_model_f32: unknown model");
+        }
+        auto x = packed_tensor<FB>(in, is);
+        auto outs = m->inference(&x);
+        unpack_tensor<FB>(*outs[0], out, out_shape);
+    });
+}
+
+// Resnet8Tiny<QUInt8Buffer>: every tensor of the model shares one set of quantisation fields per role
+// (input, filters, activations), enough to exercise the quantised layer classes end to end.
+int stest_resnet8_u8(int batch, const uint8_t *const *filters, const size_t *sizes, int nfilters, const uint8_t *in,
+                     const int32_t *in_q, const int32_t *filter_q, uint8_t *out, int *out_shape)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, 3, 32, 32};
+        std::vector<std::unique_ptr<QB>> own;
+        std::vector<QB *> fl;
+        for (int i = 0; i < nfilters; ++i)
+        {
+            own.emplace_back(new QB(from_host<QB>(filters[i], sizes[i])));
+            set_quant(*own.back(), filter_q);
+            fl.push_back(own.back().get());
+        }
+        small::Resnet8Tiny<QB> m(is, fl, false, 10);
+        auto x = packed_tensor<QB>(in, is);
+        set_quant(x.buffer(), in_q);
+        auto outs = m.inference(&x);
+        unpack_tensor<QB>(*outs[0], out, out_shape);
+    });
+}
+
+} // extern "C"

@@ -106,6 +106,27 @@ static void test_shapes_and_packing()
     CHECK(packed[small::packed_buffer_index(32, 3, 5, 16, 20, 1, 4)] == flat[(20 * 3 + 1) * 5 + 4]);
     small::unpack_buffer(packed, small::INPUT, 1, 32, 3, 5, 16, 16, back);
     CHECK(small::equals(480, flat, back));
+    // the device pack agrees with the host index walk for every tensor type
+    struct { small::BufferTypeEnum t; uint32_t d0, d1, d2, d3; } shapes[] = {
+        {small::INPUT, 1, 3, 8, 6}, {small::OUTPUT, 1, 48, 4, 5}, {small::FILTER_DW, 32, 1, 3, 3},
+        {small::FILTER_CONV, 32, 48, 3, 3}, {small::FILTER_CONV, 16, 3, 3, 3}, {small::FILTER_FC, 32, 64, 1, 1}};
+    for (auto const &sh : shapes)
+    {
+        const size_t n = (size_t)sh.d0 * sh.d1 * sh.d2 * sh.d3;
+        FloatBuffer fl(n), dev(n), host(n);
+        for (size_t i = 0; i < n; ++i) fl[i] = float(i) * 0.5f - 7.f;
+        CHECK(small::pack_buffer(fl, sh.t, sh.d0, sh.d1, sh.d2, sh.d3, 16, 16, dev) == n);
+        CHECK(small::convert_tensor2dc<float>(fl.data(), sh.t, sh.d0, sh.d1, sh.d2, sh.d3, 16, 16, host.data()) == n);
+        CHECK(small::equals(n, dev, host, 0.f));
+    }
+    QUInt8Buffer qf(3 * 16 * 16), qp(3 * 16 * 16), qh(3 * 16 * 16);
+    for (size_t i = 0; i < qf.size(); ++i) qf[i] = uint8_t(i * 7);
+    CHECK(small::pack_buffer(qf, small::INPUT, 1, 3, 16, 16, 16, 16, qp) == 768);
+    small::convert_tensor2dc<uint8_t>(qf.data(), small::INPUT, 1, 3, 16, 16, 16, 16, qh.data());
+    CHECK(small::equals(768, qp, qh));
+    threw = false;
+    try { small::pack_buffer(flat, small::INPUT, 1, 20, 3, 8, 16, 16, packed); } catch (std::invalid_argument const &) { threw = true; }
+    CHECK(threw);
 }
 
 static void test_relu_leaky_accum_upsample_concat()

@@ -1,0 +1,161 @@
+"""The C++ Layer / Model classes (include/small/*Layer.hpp, include/small/models/) on the GPU against the
+CPU restatement of the reference's classes (oracle/layers.py, pinned against the reference's own
+classes by test_oracle_layers_vs_ref.py).  The classes are driven through tests/cpp/layers_shim.cpp.
+
+CPU: the shim compiles and links with plain g++.  GPU: float32 within the parity tolerance, uint8 bit-exact;
+batched layers must equal the batch-1 results image by image.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import layers as ol
+from oracle.binding import quant
+from smallframework_amd import synth
+from util import assert_close_f32, assert_equal_exact
+import layer_shims
+from test_oracle_layers_vs_ref import CONV_LAYER_CASES, SIMPLE_CASES, conv_layer_inputs, simple_inputs
+
+
+@pytest.mark.skipif(not os.path.exists(os.path.join(layer_shims.LIBDIR, "libsmall_hip.so")), reason="library not built")
+def test_layer_shim_compiles_and_links():
+    assert os.path.exists(layer_shims.build_hip_shim())
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return layer_shims.HipLayers()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch", [1, 3])
+@pytest.mark.parametrize("case", CONV_LAYER_CASES, ids=str)
+def test_conv_layers(hip, oracle, case, batch):
+    kind, C, H, W, kh, kw, stride, padding, Co, has_bias, has_bn, act = case
+    x, f, bias, bn, init = conv_layer_inputs(case, batch)
+    got = hip.conv_layer_f32(kind, x, f, bias, bn, 1e-3, act, 0.1, kh, kw, stride, padding, out_init=init)
+    want = ol.conv_layer_f32(oracle, kind, x, f, bias, bn, 1e-3, act, 0.1, kh, kw, stride, padding, out_init=init)
+    assert got.shape == want.shape
+    assert_close_f32(got, want, what="%s batch %d" % (case, batch))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", SIMPLE_CASES, ids=str)
+def test_simple_layers(hip, oracle, case):
+    kind, C, H, W, k, kw, stride, padding, slope, C2 = case
+    x, x2, init = simple_inputs(case, batch=2)
+    got = hip.simple_layer_f32(kind, x, k, kw, stride, padding, slope, x2, init)
+    want = ol.simple_layer_f32(oracle, kind, x, k, kw, stride, padding, slope, x2, init)
+    assert got.shape == want.shape
+    if kind == 1:
+        assert_close_f32(got, want, what=str(case))
+    else:
+        assert_equal_exact(got, want, str(case))
+
+
+@pytest.mark.gpu
+def test_layer_errors(hip):
+    x = np.zeros((1, 16, 8, 8), np.float32)
+    f = np.zeros((16, 16, 3, 3), np.float32)
+    with pytest.raises(ValueError, match="SOFTMAX"):
+        hip.conv_layer_f32(0, x, f, None, None, 0, 3, 0, 3, 3, 1, 1)
+    with pytest.raises(ValueError, match="invalid number of input channels"):
+        hip.conv_layer_f32(0, np.zeros((1, 5, 8, 8), np.float32), np.zeros((16, 5, 3, 3), np.float32), None, None, 0, 0,
+                           0, 3, 3, 1, 1)
+    with pytest.raises(ValueError, match="invalid number of output channels"):       # partial layers cannot pad
+        hip.conv_layer_f32(1, x, np.zeros((10, 16, 3, 3), np.float32), None, None, 0, 0, 0, 3, 3, 1, 1)
+    with pytest.raises(ValueError, match="kernel too large"):
+        hip.simple_layer_f32(0, np.zeros((1, 16, 2, 2), np.float32), 3, 3, 1, 0)
+    with pytest.raises(ValueError, match="unsupported scale factor"):
+        hip.simple_layer_f32(4, x, 3)
+    with pytest.raises(ValueError, match="stride unsupported"):
+        hip.conv_layer_f32(0, x, f, None, None, 0, 0, 0, 3, 3, 3, 1)
+
+
+def _model_case(name):
+    """-> (which, variant, oracle fn(oracle, x, filters), filters, input [N, C, H, W])"""
+    if name == "MobileNetTiny":
+        fl = ol.make_filters(synth, ol.mobilenet_specs(), 16)
+        return 0, 0, ol.mobilenet_tiny, fl, (2, 3, 96, 96)
+    if name == "MobileNetV1_224_1000":
+        fl = ol.make_filters(synth, ol.mobilenet_specs(), 1000)
+        return 0, 1, lambda o, x, f: ol.mobilenet_tiny(o, x, f, average_pool=True), fl, (2, 3, 224, 224)
+    if name == "Resnet8Tiny":
+        return 1, 0, ol.resnet8_tiny, ol.make_filters(synth, ol.resnet8_specs(), 16), (5, 3, 32, 32)
+    if name == "Resnet8_10":
+        return 1, 1, ol.resnet8_tiny, ol.make_filters(synth, ol.resnet8_specs(), 10), (2, 3, 32, 32)
+    if name == "DSCNNTiny":
+        return 2, 0, ol.dscnn_tiny, ol.make_filters(synth, ol.dscnn_specs(), 16), (3, 3, 49, 10)
+    if name == "DSCNN_10x4_12":
+        fl = ol.make_filters(synth, ol.dscnn_specs((10, 4), 1), 12)
+        return 2, 1, lambda o, x, f: ol.dscnn_tiny(o, x, f, stem=(10, 4), average_pool=True), fl, (3, 1, 49, 10)
+    if name == "TinyYoloV2":
+        return 3, 0, ol.tiny_yolo_v2, ol.make_filters(synth, ol.yolo_specs(), 16), (2, 3, 96, 96)
+    if name == "TinyYoloV2_leaky_125":
+        fl = ol.make_filters(synth, ol.yolo_specs(), 125)
+        return 3, 1, lambda o, x, f: ol.tiny_yolo_v2(o, x, f, ol.LEAKY, 0.1, False), fl, (2, 3, 160, 160)
+    raise KeyError(name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["MobileNetTiny", "MobileNetV1_224_1000", "Resnet8Tiny", "Resnet8_10", "DSCNNTiny",
+                                  "DSCNN_10x4_12", "TinyYoloV2", "TinyYoloV2_leaky_125"])
+def test_models(hip, oracle, name):
+    which, variant, fn, filters, shape = _model_case(name)
+    x = synth.normal(55, int(np.prod(shape))).reshape(shape)
+    got = hip.model_f32(which, x, filters, variant)
+    want = fn(oracle, x, filters)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    scale = max(1.0, float(np.abs(want).max()))
+    assert_close_f32(got, want, atol=1e-5 * scale, what=name)
+    # the batched model equals the batch-1 model image by image (same kernels or within tolerance)
+    one = hip.model_f32(which, x[1:2], filters, variant)
+    assert_close_f32(one[0], got[1], atol=1e-5 * scale, what=name + " batch-1 vs batched")
+
+
+# ---- quantised layers -------------------------------------------------------------------------------------
+DEFAULT_Q = (128, 1077952576, 0, 6)       # the fields of a fresh QUInt8Buffer
+QMAX = (1 << 31) - 1                      # multiplier ~ 1.0: ReLU and Accum requantise with the output's scale again
+
+# (kind, C, H, W, k, stride, padding, Co, act, iq, fq, oq)
+U8_CASES = [
+    (0, 3, 16, 16, 3, 1, 1, 16, ol.RELU, (-128, 1 << 30, 0, 0), (-120, 1 << 30, 0, 0), (0, QMAX, 0, 4)),
+    (0, 16, 12, 12, 3, 2, 1, 32, ol.NONE, (-100, 1 << 30, 0, 0), (-131, 1 << 30, 0, 0), (0, 1500000000, 0, 11)),
+    (0, 32, 8, 8, 1, 2, 0, 64, ol.RELU, DEFAULT_Q, (-128, 1 << 30, 0, 0), (5, QMAX, 0, 5)),
+    (0, 64, 1, 1, 1, 1, 0, 10, ol.NONE, (-90, 1 << 30, 0, 0), (-128, 1 << 30, 0, 0), (0, 1 << 30, 0, 8)),
+    (1, 16, 10, 10, 3, 1, 1, 16, ol.RELU, (-128, 1 << 30, 0, 0), (-128, 1 << 30, 0, 0), (0, QMAX, 0, 1)),
+    (1, 32, 6, 6, 3, 1, 1, 32, ol.NONE, DEFAULT_Q, (-125, 1 << 30, 0, 0), (-20, QMAX, 0, 1)),
+    (2, 32, 9, 9, 3, 1, 1, 32, ol.RELU, (-128, 1 << 30, 0, 0), (-128, 1 << 30, 0, 0), (0, QMAX, 0, 3)),
+    (2, 16, 10, 10, 3, 2, 1, 16, ol.NONE, (-110, 1 << 30, 0, 0), (-140, 1 << 30, 0, 0), (0, 1 << 30, 0, 4)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch", [1, 4])
+@pytest.mark.parametrize("case", U8_CASES, ids=str)
+def test_quantised_layers(hip, oracle, case, batch):
+    kind, C, H, W, k, stride, padding, Co, act, iq, fq, oq = case
+    x = synth.uniform_u8(31, batch * C * H * W).reshape(batch, C, H, W)
+    f = synth.uniform_u8(32, Co * (1 if kind == 2 else C) * k * k).reshape((Co, k, k) if kind == 2 else (Co, C, k, k))
+    t, b, l, r, Ho, Wo = ol.window(H, W, k, k, stride, padding)
+    init = synth.uniform_u8(33, batch * Co * Ho * Wo).reshape(batch, Co, Ho, Wo) if kind == 1 else None
+    got = hip.conv_layer_u8(kind, x, iq, f, fq, oq, act, k, k, stride, padding, out_init=init)
+    want = ol.conv_layer_u8(oracle, quant, kind, x, iq, f, fq, oq, act, k, k, stride, padding, out_init=init)
+    assert got.shape == want.shape
+    assert_equal_exact(got, want, "%s batch %d" % (case, batch))
+    assert len(np.unique(want)) >= 7, "case does not discriminate (saturated output)"
+
+
+@pytest.mark.gpu
+def test_resnet8_quantised_model(hip, oracle):
+    batch = 4
+    iq, fq = (-128, 1 << 30, 0, 0), (-128, 1 << 30, 0, 0)
+    x = synth.uniform_u8(41, batch * 3 * 32 * 32).reshape(batch, 3, 32, 32)
+    filters = ol.make_filters(synth, ol.resnet8_specs(), 10, dtype=np.uint8)
+    got = hip.resnet8_u8(x, iq, filters, fq)
+    want = ol.resnet8_tiny_u8(oracle, quant, x, iq, filters, fq, DEFAULT_Q)
+    assert got.shape == want.shape == (batch, 16, 1, 1)
+    assert_equal_exact(got, want, "Resnet8Tiny<QUInt8Buffer>")
