@@ -160,10 +160,17 @@ private:
     void *m_dev = nullptr;
 };
 
-inline void reject_softmax(ActivationType a, char const *who)
+// the activation the fused convolution call applies itself; SOFTMAX runs as a second call on the output
+inline ActivationType fused_act(ActivationType a) { return a == SOFTMAX ? NONE : a; }
+
+template <class BufferT>
+void softmax_in_place(ActivationType a, shape_type const &os, BufferT &buf)
 {
-    if (a == SOFTMAX)
-        throw std::invalid_argument(std::string(who) + "::ctor ERROR: SOFTMAX activation is not part of this build.");
+    if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+    {
+        if (a == SOFTMAX)
+            batched::SoftMax((int)os[BATCH], (int)os[CHANNEL], (int)os[HEIGHT], (int)os[WIDTH], buf, buf);
+    }
 }
 
 // padded output channel count, or the reference's error when packed buffers do not allow padding
@@ -227,7 +234,6 @@ public:
           m_activation_type(activation_type),
           m_slope(leaky_slope)
     {
-        detail::reject_softmax(activation_type, "Conv2DLayer");
         // 1 and 2 input channels are accepted like 3: small::Conv2D takes all three (the reference's layer
         // class only lets 3 through)
         if ((input_shape[CHANNEL] % BufferT::C_ib) != 0 && (input_shape[CHANNEL] == 0 || input_shape[CHANNEL] > 3))
@@ -241,9 +247,9 @@ public:
                                    buffers_are_packed, m_packed_filters, m_packed_bias);
         if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
         {
-            if (m_packed_bias.size() > 0 || activation_type == LEAKY)
+            if (m_packed_bias.size() > 0 || activation_type == LEAKY || activation_type == SOFTMAX)
                 throw std::invalid_argument(
-                    "Conv2DLayer::ctor ERROR: bias / LeakyReLU have no quantised implementation.");
+                    "Conv2DLayer::ctor ERROR: bias / LeakyReLU / SoftMax have no quantised implementation.");
         }
         m_prepared.build(kernel_height, kernel_width, Co, (uint32_t)input_shape[CHANNEL], m_packed_filters);
     }
@@ -264,7 +270,7 @@ public:
             batched::Conv2D_Bias_Act(batch, m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b,
                                      m_window.l, m_window.r, (int)os[CHANNEL], (int)m_input_shape[CHANNEL],
                                      (int)m_input_shape[HEIGHT], (int)m_input_shape[WIDTH], input[0]->buffer(),
-                                     m_packed_filters, m_packed_bias, m_activation_type, m_slope, output->buffer());
+                                     m_packed_filters, m_packed_bias, detail::fused_act(m_activation_type), m_slope, output->buffer());
         }
         else
         {
@@ -274,6 +280,7 @@ public:
                                        m_packed_filters, m_prepared.get(), (BufferT const *)nullptr,
                                        m_activation_type == RELU, output->buffer());
         }
+        detail::softmax_in_place(m_activation_type, os, output->buffer());
         output->set_shape(os);
     }
 

@@ -61,7 +61,6 @@ public:
           m_activation_type(activation_type),
           m_slope(leaky_slope)
     {
-        detail::reject_softmax(activation_type, "DepthwiseConv2DLayer");
         if ((input_shape[CHANNEL] % BufferT::C_ib) != 0)
             throw std::invalid_argument("DepthwiseConv2DLayer::ctor ERROR: invalid number of input channels.");
         const uint32_t C = (uint32_t)input_shape[CHANNEL];
@@ -73,9 +72,9 @@ public:
                                    buffers_are_packed, m_packed_filters, m_packed_bias);
         if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
         {
-            if (m_packed_bias.size() > 0 || activation_type == LEAKY)
+            if (m_packed_bias.size() > 0 || activation_type == LEAKY || activation_type == SOFTMAX)
                 throw std::invalid_argument(
-                    "DepthwiseConv2DLayer::ctor ERROR: bias / LeakyReLU have no quantised implementation.");
+                    "DepthwiseConv2DLayer::ctor ERROR: bias / LeakyReLU / SoftMax have no quantised implementation.");
         }
     }
 
@@ -94,7 +93,7 @@ public:
         {
             batched::DepthwiseConv2D_Bias_Act(batch, m_window.kh, m_window.kw, m_window.stride, m_window.t,
                                               m_window.b, m_window.l, m_window.r, C, H, W, input[0]->buffer(),
-                                              m_packed_filters, m_packed_bias, m_activation_type, m_slope,
+                                              m_packed_filters, m_packed_bias, detail::fused_act(m_activation_type), m_slope,
                                               output->buffer());
         }
         else
@@ -106,6 +105,7 @@ public:
                 batched::ReLUActivation(batch, C, (int)os[HEIGHT], (int)os[WIDTH], output->buffer(),
                                         output->buffer());
         }
+        detail::softmax_in_place(m_activation_type, os, output->buffer());
         output->set_shape(os);
     }
 

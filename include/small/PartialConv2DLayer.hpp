@@ -66,7 +66,6 @@ public:
           m_activation_type(activation_type),
           m_slope(leaky_slope)
     {
-        detail::reject_softmax(activation_type, "PartialConv2DLayer");
         // 1 and 2 input channels are accepted like 3: small::Conv2D takes all three (the reference's layer
         // class only lets 3 through)
         if ((input_shape[CHANNEL] % BufferT::C_ib) != 0 && (input_shape[CHANNEL] == 0 || input_shape[CHANNEL] > 3))
@@ -81,9 +80,9 @@ public:
                                    buffers_are_packed, m_packed_filters, m_packed_bias);
         if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
         {
-            if (m_packed_bias.size() > 0 || activation_type == LEAKY)
+            if (m_packed_bias.size() > 0 || activation_type == LEAKY || activation_type == SOFTMAX)
                 throw std::invalid_argument(
-                    "PartialConv2DLayer::ctor ERROR: bias / LeakyReLU have no quantised implementation.");
+                    "PartialConv2DLayer::ctor ERROR: bias / LeakyReLU / SoftMax have no quantised implementation.");
             m_scratch = BufferT(this->output_size());
         }
         m_prepared.build(kernel_height, kernel_width, num_output_channels, (uint32_t)input_shape[CHANNEL],
@@ -106,7 +105,7 @@ public:
         {
             batched::PartialConv2D_Bias_Act(batch, m_window.kh, m_window.kw, m_window.stride, m_window.t,
                                             m_window.b, m_window.l, m_window.r, Co, Ci, H, W, input[0]->buffer(),
-                                            m_packed_filters, m_packed_bias, m_activation_type, m_slope,
+                                            m_packed_filters, m_packed_bias, detail::fused_act(m_activation_type), m_slope,
                                             output->buffer());
         }
         else
@@ -122,6 +121,7 @@ public:
                 batched::ReLUActivation(batch, Co, (int)os[HEIGHT], (int)os[WIDTH], output->buffer(),
                                         output->buffer());
         }
+        detail::softmax_in_place(m_activation_type, os, output->buffer());
         output->set_shape(os);
     }
 

@@ -32,7 +32,7 @@ enum ActivationType
     NONE = SMALL_HIP_ACT_NONE,
     RELU = SMALL_HIP_ACT_RELU,
     LEAKY = SMALL_HIP_ACT_LEAKY,
-    SOFTMAX = 3   // named by the reference's Layer classes; SoftMax itself is not part of this build
+    SOFTMAX = 3   // Layer classes only: small::SoftMax applied after the layer (float)
 };
 
 namespace detail
@@ -314,6 +314,29 @@ void LeakyReLUActivation(int batch, int input_channels, int input_height, int in
                            "LeakyReLUActivation");
 }
 
+// Dropout at inference: a multiplication by filter_buf[0] (interface_abstract.hpp:1697-1726); float only
+template <class BufferT, detail::if_float<BufferT> = true>
+void Dropout(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+             BufferT const &filter_buf, BufferT &output_buf)
+{
+    const float scale = filter_buf.data()[0];
+    float const *in = input_buf.device_in();
+    detail::raise<BufferT>(small_hip_dropout_f32(batch, input_channels, input_height, input_width, in, scale,
+                                                 output_buf.device_out(), detail::st()),
+                           "Dropout");
+}
+
+// SoftMax over the whole tensor of each image (interface_abstract.hpp:1778-1832); float only
+template <class BufferT, detail::if_float<BufferT> = true>
+void SoftMax(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
+             BufferT &output_buf)
+{
+    float const *in = input_buf.device_in();
+    detail::raise<BufferT>(small_hip_softmax_f32(batch, input_channels, input_height, input_width, in,
+                                                 output_buf.device_out(), detail::st()),
+                           "SoftMax");
+}
+
 template <class BufferT, detail::if_float<BufferT> = true>
 void Accum(int batch, int input_channels, int input_height, int input_width, BufferT const &input_buf,
            BufferT &output_buf)
@@ -478,6 +501,19 @@ void LeakyReLUActivation(int input_channels, int input_height, int input_width, 
                          BufferT const &filter_buf, BufferT &output_buf)
 {
     batched::LeakyReLUActivation(1, input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void Dropout(int input_channels, int input_height, int input_width, BufferT const &input_buf,
+             BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::Dropout(1, input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void SoftMax(int input_channels, int input_height, int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::SoftMax(1, input_channels, input_height, input_width, input_buf, output_buf);
 }
 
 template <class BufferT>

@@ -152,6 +152,15 @@ int small_hip_relu_f32(int batch, int input_channels, int input_height, int inpu
 int small_hip_leaky_relu_f32(int batch, int input_channels, int input_height, int input_width,
                              const float *input, float negative_slope, float *output,
                              small_hip_stream_t stream);
+/* small::Dropout<FloatBuffer>  interface_abstract.hpp:1697-1726: at inference a multiplication by
+ * filter_buf[0] (passed here by value): out = in * scale.  In place allowed. */
+int small_hip_dropout_f32(int batch, int input_channels, int input_height, int input_width,
+                          const float *input, float scale, float *output, small_hip_stream_t stream);
+/* small::SoftMax<FloatBuffer>  interface_abstract.hpp:1778-1832: over the WHOLE tensor of an image,
+ * out = exp(in) * float(1 / sum of exp(in) over all channels and pixels); no maximum is subtracted.
+ * In place allowed.  No quantised version in the reference. */
+int small_hip_softmax_f32(int batch, int input_channels, int input_height, int input_width,
+                          const float *input, float *output, small_hip_stream_t stream);
 /* small::Accum<FloatBuffer>           interface.hpp:451-455, interface_abstract.hpp:1950-1978 */
 int small_hip_accum_f32(int batch, int input_channels, int input_height, int input_width,
                         const float *input, float *output, small_hip_stream_t stream);

@@ -63,6 +63,8 @@ class Oracle:
         L.so_maxpool2d_f32.argtypes = win + [c_vp, c_vp]
         L.so_avgpool2d_f32.argtypes = win + [c_vp, c_vp]
         L.so_relu_f32.argtypes = [c_int] * 5 + [c_vp, c_vp]
+        L.so_softmax_f32.argtypes = [c_int] * 5 + [c_vp, c_vp]
+        L.so_dropout_f32.argtypes = [c_int] * 5 + [c_vp, c_f, c_vp]
         L.so_leaky_relu_f32.argtypes = [c_int] * 5 + [c_vp, c_f, c_vp]
         L.so_accum_f32.argtypes = [c_int] * 5 + [c_vp, c_vp]
         L.so_bias_f32.argtypes = [c_int] * 5 + [c_vp, c_vp, c_int]
@@ -155,6 +157,14 @@ class Oracle:
     def leaky_relu_f32(self, batch, cb, Cn, H, W, x, slope):
         out = np.empty_like(x)
         return self.lib.so_leaky_relu_f32(batch, cb, Cn, H, W, _p(x), slope, _p(out)), out
+
+    def dropout_f32(self, batch, cb, Cn, H, W, x, scale):
+        out = np.empty_like(x)
+        return self.lib.so_dropout_f32(batch, cb, Cn, H, W, _p(x), scale, _p(out)), out
+
+    def softmax_f32(self, batch, cb, Cn, H, W, x):
+        out = np.empty_like(x)
+        return self.lib.so_softmax_f32(batch, cb, Cn, H, W, _p(x), _p(out)), out
 
     def accum_f32(self, batch, cb, Cn, H, W, x, out):
         out = out.copy()
@@ -307,6 +317,8 @@ class RefLib:
             for f in (L.sref_relu_f32, L.sref_accum_f32, L.sref_bias_f32, L.sref_partial_bias_f32):
                 f.argtypes = [c_int] * 3 + [c_vp] * 2
             L.sref_leaky_relu_f32.argtypes = [c_int] * 3 + [c_vp] * 3
+            L.sref_dropout_f32.argtypes = [c_int] * 3 + [c_vp] * 3
+            L.sref_softmax_f32.argtypes = [c_int] * 3 + [c_vp] * 2
             L.sref_upsample2d_f32.argtypes = [c_int] * 4 + [c_vp] * 2
             L.sref_concat_f32.argtypes = [C.c_uint32] * 4 + [c_vp] * 3
             L.sref_dense_f32.argtypes = [c_int] * 2 + [c_vp] * 3

@@ -17,7 +17,7 @@ one, and PartialConv2DLayer / AddLayer follow this build's own definition: parit
 import numpy as np
 
 CB = 16      # channel block; a test that compares with the reference's scalar build sets it to 1
-NONE, RELU, LEAKY = 0, 1, 2
+NONE, RELU, LEAKY, SOFTMAX = 0, 1, 2, 3
 INPUT, OUTPUT, FILTER_DW, FILTER_CONV, FILTER_FC = range(5)
 
 
@@ -110,12 +110,14 @@ def conv_layer_f32(oracle, kind, x, filters, bias, bn, eps, act, slope, kh, kw, 
         rc, y = oracle.relu_f32(n, CB, cop, ho, wo, y)
     elif act == LEAKY:
         rc, y = oracle.leaky_relu_f32(n, CB, cop, ho, wo, y, slope)
+    elif act == SOFTMAX:
+        rc, y = oracle.softmax_f32(n, CB, cop, ho, wo, y)
     return _unpack_images(oracle, y, n, cop, ho, wo)
 
 
 def simple_layer_f32(oracle, kind, x, k=1, kw=1, stride=1, padding=0, slope=0.0, x2=None, out_init=None):
     """kind as in the shims: 0 max pool, 1 average pool, 2 ReLU, 3 LeakyReLU, 4 upsample (k = scale),
-    5 add (out_init += x), 6 route (copy), 7 route (concatenate x, x2)."""
+    5 add (out_init += x), 6 route (copy), 7 route (concatenate x, x2), 8 softmax."""
     n, c, h, w = x.shape
     xp = _pack_images(oracle, x, INPUT)
     if kind in (0, 1):
@@ -137,6 +139,9 @@ def simple_layer_f32(oracle, kind, x, k=1, kw=1, stride=1, padding=0, slope=0.0,
         shape = (c, h, w)
     elif kind == 6:
         rc, y = 0, xp
+        shape = (c, h, w)
+    elif kind == 8:
+        rc, y = oracle.softmax_f32(n, CB, c, h, w, xp)
         shape = (c, h, w)
     elif kind == 7:
         c2 = x2.shape[1]

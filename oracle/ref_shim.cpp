@@ -35,6 +35,7 @@
 #include <small/UpSample2DLayer.hpp>
 #include <small/AddLayer.hpp>
 #include <small/RouteLayer.hpp>
+#include <small/SoftMaxLayer.hpp>
 #include <small/models/MobileNetTiny.hpp>
 #include <small/models/Resnet8Tiny.hpp>
 #include <small/models/DSCNNTiny.hpp>
@@ -173,6 +174,14 @@ int sref_relu_f32(int C, int H, int W, void *in, void *out)
 int sref_leaky_relu_f32(int C, int H, int W, void *in, void *slope, void *out)
 {
     return guarded([&] { small::LeakyReLUActivation(C, H, W, F(in), F(slope), F(out)); });
+}
+int sref_dropout_f32(int C, int H, int W, void *in, void *scale, void *out)
+{
+    return guarded([&] { small::Dropout(C, H, W, F(in), F(scale), F(out)); });
+}
+int sref_softmax_f32(int C, int H, int W, void *in, void *out)
+{
+    return guarded([&] { small::SoftMax(C, H, W, F(in), F(out)); });
 }
 int sref_accum_f32(int C, int H, int W, void *in, void *out)
 {
@@ -326,7 +335,7 @@ int sref_conv_layer_f32(int kind, int C, int H, int W, int kh, int kw, int strid
 }
 
 // kind: 0 MaxPool2DLayer, 1 AveragePool2DLayer, 2 ReLULayer, 3 LeakyReLULayer(slope), 4 UpSample2DLayer(k = scale),
-// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels)
+// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels), 8 SoftMaxLayer
 int sref_simple_layer_f32(int kind, int C, int H, int W, int k, int kw, int stride, int padding, float slope,
                           const float *in, const float *in2, int C2, float *out, int *out_shape)
 {
@@ -345,6 +354,7 @@ int sref_simple_layer_f32(int kind, int C, int H, int W, int k, int kw, int stri
         case 5: layer.reset(new small::AddLayer<FB>(is, is)); break;
         case 6: layer.reset(new small::RouteLayer<FB>(is)); break;
         case 7: layer.reset(new small::RouteLayer<FB>(is, is2)); break;
+        case 8: layer.reset(new small::SoftMaxLayer<FB>(is)); break;
         default: throw std::invalid_argument("sref_simple_layer_f32: unknown kind");
         }
         auto x = packed_tensor(in, is);

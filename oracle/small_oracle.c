@@ -24,6 +24,8 @@
  *        reference fixtures, REF/ZEN2 builds with negative inputs on padded borders
  *   so_relu_f32, so_leaky_relu_f32, so_accum_f32, so_bias_f32, so_upsample2d_f32, so_concat
  *        closed forms (exact), reference fixtures (relu), REF/ZEN2 builds
+ *   so_dropout_f32, so_softmax_f32   REF/ZEN2 builds (dropout exact; softmax within 1e-6 relative:
+ *        the reduction order of the global sum differs), closed form sum(out) == 1
  *   so_dense_f32   REF build's Conv2D on a 1x1 image, plain matmul
  *   so_dense_literal_f32   REF build's small::Dense
  *   so_requant, so_conv2d_u8, so_dwconv2d_u8, so_maxpool2d_u8, so_relu_u8, so_dense_u8
@@ -376,6 +378,39 @@ int so_leaky_relu_f32(int batch, int cb, int C, int H, int W, const float *in, f
     if (C <= 0 || C % cb != 0) return SO_ECHANNELS;
     size_t n = (size_t)batch * C * H * W;
     for (size_t i = 0; i < n; i++) { float v = in[i]; out[i] = (v > 0.0f) ? v : v * slope; }
+    return SO_OK;
+}
+
+/* Dropout at inference: c = a * filter[0] (abstract_layer.hpp:82-86 "drop_out_rate = b_cur[0]",
+ * intrinsics_float.h:534-545 FLOAT_DIV_TILE_C multiplies), interface_abstract.hpp:1697-1726 */
+int so_dropout_f32(int batch, int cb, int C, int H, int W, const float *in, float scale, float *out)
+{
+    if (C <= 0 || C % cb != 0) return SO_ECHANNELS;
+    size_t n = (size_t)batch * C * H * W;
+    for (size_t i = 0; i < n; i++) out[i] = in[i] * scale;
+    return SO_OK;
+}
+
+/* SoftMax over the WHOLE tensor of an image (interface_abstract.hpp:1778-1832): element-wise exp
+ * (intrinsics_float.h:671-686, std::exp on float, no maximum subtracted), one global sum of all
+ * C*H*W values, then a multiplication by float(1.0 / sum) (the reciprocal is taken in double and
+ * stored in a float buffer).  The sum here is accumulated in double and rounded to float once: the
+ * reference adds floats in its tile order, which differs from this by float rounding only (about 1e-7
+ * relative at class-score sizes, checked; it grows with the element count, so a float restatement in
+ * any other order would be no closer to it). */
+int so_softmax_f32(int batch, int cb, int C, int H, int W, const float *in, float *out)
+{
+    if (C <= 0 || C % cb != 0) return SO_ECHANNELS;
+    size_t per = (size_t)C * H * W;
+    for (int n = 0; n < batch; n++)
+    {
+        const float *a = in + (size_t)n * per;
+        float *c = out + (size_t)n * per;
+        double sum = 0.0;
+        for (size_t i = 0; i < per; i++) { c[i] = expf(a[i]); sum += (double)c[i]; }
+        const float inv = (float)(1.0 / (double)(float)sum);
+        for (size_t i = 0; i < per; i++) c[i] *= inv;
+    }
     return SO_OK;
 }
 

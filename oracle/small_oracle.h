@@ -78,6 +78,8 @@ int so_maxpool2d_f32(int batch, int cb, int kh, int kw, int stride, int pt, int 
 int so_avgpool2d_f32(int batch, int cb, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
                      int C, int H, int W, const float *in, float *out);
 int so_relu_f32(int batch, int cb, int C, int H, int W, const float *in, float *out);
+int so_dropout_f32(int batch, int cb, int C, int H, int W, const float *in, float scale, float *out);
+int so_softmax_f32(int batch, int cb, int C, int H, int W, const float *in, float *out);
 int so_leaky_relu_f32(int batch, int cb, int C, int H, int W, const float *in, float slope,
                       float *out);
 int so_accum_f32(int batch, int cb, int C, int H, int W, const float *in, float *out);

@@ -63,6 +63,8 @@ SIGNATURES = {
     "small_hip_avgpool2d_f32": (_i, _win + [_p, _p, _p]),
     "small_hip_relu_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_leaky_relu_f32": (_i, [_i] * 4 + [_p, _f, _p, _p]),
+    "small_hip_dropout_f32": (_i, [_i] * 4 + [_p, _f, _p, _p]),
+    "small_hip_softmax_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_accum_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_partial_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),

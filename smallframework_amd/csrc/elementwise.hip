@@ -12,7 +12,7 @@ namespace
 constexpr int TPB = 256;
 constexpr int UNROLL = 4;
 
-enum EwOp { EW_RELU, EW_LEAKY, EW_ACCUM };
+enum EwOp { EW_RELU, EW_LEAKY, EW_ACCUM, EW_SCALE };
 
 template <int OP>
 __device__ __forceinline__ float4 ew_apply(float4 x, float4 o, float slope)
@@ -27,6 +27,10 @@ __device__ __forceinline__ float4 ew_apply(float4 x, float4 o, float slope)
     {
         r.x = x.x > 0.f ? x.x : x.x * slope; r.y = x.y > 0.f ? x.y : x.y * slope;
         r.z = x.z > 0.f ? x.z : x.z * slope; r.w = x.w > 0.f ? x.w : x.w * slope;
+    }
+    else if (OP == EW_SCALE)
+    {
+        r.x = x.x * slope; r.y = x.y * slope; r.z = x.z * slope; r.w = x.w * slope;
     }
     else
     {
@@ -167,6 +171,45 @@ __global__ __launch_bounds__(TPB) void ew_u8_kernel(const uint4 *in, uint4 *out,
     }
 }
 
+// SoftMax over the whole tensor of an image: out = exp(in) * float(1 / sum(exp(in))), no maximum
+// subtracted (interface_abstract.hpp:1778-1832).  One workgroup per image: pass 1 writes exp(in) and
+// reduces the sum (per lane, then wave shuffles, then LDS), pass 2 scales what pass 1 wrote (it is
+// still in cache for the class-score sized tensors this layer sees).  In place is allowed.
+__global__ __launch_bounds__(TPB) void softmax_f32_kernel(const float4 *in, float4 *out, size_t per4)
+{
+    __shared__ float part[TPB / WAVE];
+    __shared__ float inv_s;
+    const float4 *a = in + (size_t)blockIdx.x * per4;
+    float4 *c = out + (size_t)blockIdx.x * per4;
+    float sum = 0.f;
+    for (size_t i = threadIdx.x; i < per4; i += TPB)
+    {
+        const float4 x = a[i];
+        const float4 e = make_float4(expf(x.x), expf(x.y), expf(x.z), expf(x.w));
+        c[i] = e;
+        sum += (e.x + e.y) + (e.z + e.w);
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, WAVE);
+    if ((threadIdx.x & (WAVE - 1)) == 0) part[threadIdx.x / WAVE] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < TPB / WAVE; ++w) t += part[w];
+        inv_s = (float)(1.0 / (double)t);
+    }
+    __syncthreads();
+    const float inv = inv_s;
+    for (size_t i = threadIdx.x; i < per4; i += TPB)
+    {
+        float4 e = c[i];
+        e.x *= inv; e.y *= inv; e.z *= inv; e.w *= inv;
+        c[i] = e;
+    }
+}
+
 inline unsigned blocks_for(size_t nvec) { return (unsigned)((nvec + TPB * UNROLL - 1) / (TPB * UNROLL)); }
 
 int check_act_args(const char *op, int batch, int C, int H, int W, const void *in, const void *out)
@@ -203,6 +246,22 @@ int small_hip_leaky_relu_f32(int batch, int C, int H, int W, const float *in, fl
                              small_hip_stream_t stream)
 {
     return launch_ew<EW_LEAKY>("small_hip_leaky_relu_f32", batch, C, H, W, in, out, slope, stream);
+}
+
+int small_hip_dropout_f32(int batch, int C, int H, int W, const float *in, float scale, float *out,
+                          small_hip_stream_t stream)
+{
+    return launch_ew<EW_SCALE>("small_hip_dropout_f32", batch, C, H, W, in, out, scale, stream);
+}
+
+int small_hip_softmax_f32(int batch, int C, int H, int W, const float *in, float *out, small_hip_stream_t stream)
+{
+    if (int rc = check_act_args("small_hip_softmax_f32", batch, C, H, W, in, out)) return rc;
+    const size_t per4 = (size_t)C * H * W / 4;
+    hipLaunchKernelGGL(softmax_f32_kernel, dim3((unsigned)batch), dim3(TPB), 0, as_stream(stream),
+                       reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out), per4);
+    SHP_LAUNCH_CHECK("small_hip_softmax_f32");
+    return SMALL_HIP_OK;
 }
 
 int small_hip_accum_f32(int batch, int C, int H, int W, const float *in, float *out,

@@ -22,6 +22,7 @@
 #include <small/PartialConv2DLayer.hpp>
 #include <small/ReLULayer.hpp>
 #include <small/RouteLayer.hpp>
+#include <small/SoftMaxLayer.hpp>
 #include <small/UpSample2DLayer.hpp>
 #include <small/models/DSCNNTiny.hpp>
 #include <small/models/MobileNetTiny.hpp>
@@ -176,7 +177,7 @@ int stest_conv_layer_u8(int kind, int batch, int C, int H, int W, int kh, int kw
 }
 
 // kind: 0 MaxPool2DLayer, 1 AveragePool2DLayer, 2 ReLULayer, 3 LeakyReLULayer(slope), 4 UpSample2DLayer(k = scale),
-// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels)
+// 5 AddLayer (out += in), 6 RouteLayer(one input), 7 RouteLayer(in, in2 with C2 channels), 8 SoftMaxLayer
 int stest_simple_layer_f32(int kind, int batch, int C, int H, int W, int k, int kw, int stride, int padding,
                            float slope, const float *in, const float *in2, int C2, float *out, int *out_shape)
 {
@@ -195,6 +196,7 @@ int stest_simple_layer_f32(int kind, int batch, int C, int H, int W, int k, int 
         case 5: layer.reset(new small::AddLayer<FB>(is, is)); break;
         case 6: layer.reset(new small::RouteLayer<FB>(is)); break;
         case 7: layer.reset(new small::RouteLayer<FB>(is, is2)); break;
+        case 8: layer.reset(new small::SoftMaxLayer<FB>(is)); break;
         default: throw std::invalid_argument("stest_simple_layer_f32: unknown kind");
         }
         auto x = packed_tensor<FB>(in, is);

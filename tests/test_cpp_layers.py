@@ -50,7 +50,7 @@ def test_simple_layers(hip, oracle, case):
     got = hip.simple_layer_f32(kind, x, k, kw, stride, padding, slope, x2, init)
     want = ol.simple_layer_f32(oracle, kind, x, k, kw, stride, padding, slope, x2, init)
     assert got.shape == want.shape
-    if kind == 1:
+    if kind in (1, 8):
         assert_close_f32(got, want, what=str(case))
     else:
         assert_equal_exact(got, want, str(case))
@@ -60,8 +60,6 @@ def test_simple_layers(hip, oracle, case):
 def test_layer_errors(hip):
     x = np.zeros((1, 16, 8, 8), np.float32)
     f = np.zeros((16, 16, 3, 3), np.float32)
-    with pytest.raises(ValueError, match="SOFTMAX"):
-        hip.conv_layer_f32(0, x, f, None, None, 0, 3, 0, 3, 3, 1, 1)
     with pytest.raises(ValueError, match="invalid number of input channels"):
         hip.conv_layer_f32(0, np.zeros((1, 5, 8, 8), np.float32), np.zeros((16, 5, 3, 3), np.float32), None, None, 0, 0,
                            0, 3, 3, 1, 1)

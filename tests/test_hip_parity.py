@@ -264,6 +264,19 @@ def test_elementwise_f32(lib, oracle, shape):
     dx = hu.dev(x)
     assert lib.small_hip_leaky_relu_f32(batch, Cn, H, W, hu.ptr(dx), 0.1, hu.ptr(do), st()) == 0
     assert_equal_exact(hu.host(do), oracle.leaky_relu_f32(batch, CB, Cn, H, W, x, 0.1)[1], "leaky")
+    # dropout (inference): a multiplication, exact
+    assert lib.small_hip_dropout_f32(batch, Cn, H, W, hu.ptr(dx), 0.8, hu.ptr(do), st()) == 0
+    assert_equal_exact(hu.host(do), oracle.dropout_f32(batch, CB, Cn, H, W, x, 0.8)[1], "dropout")
+    # softmax over the whole tensor of each image, out of place and in place
+    xs = (2.0 * x).astype(np.float32)
+    ds = hu.dev(xs)
+    assert lib.small_hip_softmax_f32(batch, Cn, H, W, hu.ptr(ds), hu.ptr(do), st()) == 0
+    want_s = oracle.softmax_f32(batch, CB, Cn, H, W, xs)[1]
+    assert_close_f32(hu.host(do), want_s, rtol=1e-5, atol=1e-12, what="softmax")
+    assert lib.small_hip_softmax_f32(batch, Cn, H, W, hu.ptr(ds), hu.ptr(ds), st()) == 0
+    assert_close_f32(hu.host(ds), want_s, rtol=1e-5, atol=1e-12, what="softmax in place")
+    per = Cn * H * W
+    assert np.allclose(hu.host(ds).astype(np.float64).reshape(batch, per).sum(1), 1.0, atol=1e-5)
     # accum
     do = hu.dev(y0)
     assert lib.small_hip_accum_f32(batch, Cn, H, W, hu.ptr(dx), hu.ptr(do), st()) == 0

@@ -16,9 +16,9 @@ from util import assert_close_f32, assert_equal_exact
 from layer_shims import RefLayers
 
 
-def _cmp(name, got, want, what):
+def _cmp(name, got, want, what, exact_on_ref=True):
     assert got.shape == want.shape, (what, got.shape, want.shape)
-    if name == "REF":
+    if name == "REF" and exact_on_ref:
         assert_equal_exact(got, want, what)
     else:
         assert_close_f32(got, want, what=what)
@@ -48,6 +48,8 @@ CONV_LAYER_CASES = [
     (2, 16, 10, 10, 3, 3, 2, 1, 16, True, False, ol.NONE),
     (2, 48, 7, 7, 3, 3, 1, 1, 48, True, True, ol.RELU),
     (2, 16, 8, 8, 3, 3, 2, 0, 16, False, True, ol.LEAKY),
+    (0, 64, 1, 1, 1, 1, 1, 0, 16, True, False, ol.SOFTMAX),     # classifier head with the softmax attached
+    (0, 16, 4, 4, 3, 3, 1, 1, 16, False, False, ol.SOFTMAX),
 ]
 
 
@@ -75,8 +77,8 @@ def test_conv_layers(oracle, plat, case):
     eps, slope = 1e-3, 0.1
     want = ref.conv_layer_f32(kind, x, f, bias, bn, eps, act, slope, kh, kw, stride, padding, out_init=init)
     got = ol.conv_layer_f32(oracle, kind, x, f, bias, bn, eps, act, slope, kh, kw, stride, padding, out_init=init)
-    _cmp(name, got, want, str(case))
-    if got.shape[1] != Co and act != ol.LEAKY:
+    _cmp(name, got, want, str(case), exact_on_ref=act != ol.SOFTMAX)     # softmax: the global sum's order differs
+    if got.shape[1] != Co and act not in (ol.LEAKY, ol.SOFTMAX):
         assert not got[:, Co:].any()      # padded channels: zero filter rows and zero bias
 
 
@@ -99,6 +101,7 @@ SIMPLE_CASES = [
     (2, 32, 6, 7, 1, 1, 1, 0, 0.0, 0), (3, 16, 6, 7, 1, 1, 1, 0, 0.1, 0),
     (4, 16, 5, 6, 2, 1, 1, 0, 0.0, 0), (5, 32, 6, 6, 1, 1, 1, 0, 0.0, 0),
     (6, 16, 4, 5, 1, 1, 1, 0, 0.0, 0), (7, 16, 4, 5, 1, 1, 1, 0, 0.0, 32),
+    (8, 16, 1, 1, 1, 1, 1, 0, 0.0, 0), (8, 32, 3, 5, 1, 1, 1, 0, 0.0, 0),
 ]
 
 
@@ -117,7 +120,7 @@ def test_simple_layers(oracle, plat, case):
     x, x2, init = simple_inputs(case)
     want = ref.simple_layer_f32(kind, x, k, kw, stride, padding, slope, x2, init)
     got = ol.simple_layer_f32(oracle, kind, x, k, kw, stride, padding, slope, x2, init)
-    _cmp(name, got, want, str(case))
+    _cmp(name, got, want, str(case), exact_on_ref=kind != 8)
 
 
 # (which, name, specs, oracle fn, input shape); the reference builds 16-class heads and, for DS-CNN and

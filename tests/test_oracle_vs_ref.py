@@ -208,6 +208,21 @@ def test_elementwise_f32(request, oracle, name):
         b, bs, bo = ref.fbuf(n, x), ref.fbuf(1, np.float32([slope])), ref.fbuf(n)
         assert ref.lib.sref_leaky_relu_f32(Cn, H, W, b.h, bs.h, bo.h) == 0
         _cmp(name, oracle.leaky_relu_f32(1, cb, Cn, H, W, x, slope)[1], bo.a, "leaky")
+    # dropout (inference): a multiplication by filter[0]
+    b, bs, bo = ref.fbuf(n, x), ref.fbuf(1, np.float32([0.8])), ref.fbuf(n)
+    assert ref.lib.sref_dropout_f32(Cn, H, W, b.h, bs.h, bo.h) == 0
+    assert_equal_exact(oracle.dropout_f32(1, cb, Cn, H, W, x, 0.8)[1], bo.a, "dropout")
+    # softmax over the whole tensor: exp, one global sum, scale; the reduction order differs -> 2e-6
+    for shape in ((Cn, H, W), (1008 if cb == 16 else 1000, 1, 1), (16, 1, 1)):
+        c2, h2, w2 = shape
+        xs = synth.normal(24, c2 * h2 * w2, std=2.0)
+        b, bo = ref.fbuf(xs.size, xs), ref.fbuf(xs.size)
+        assert ref.lib.sref_softmax_f32(c2, h2, w2, b.h, bo.h) == 0
+        mine = oracle.softmax_f32(1, cb, c2, h2, w2, xs)[1]
+        assert_close_f32(mine, bo.a, rtol=2e-6, atol=0.0, what="softmax %s" % (shape,))
+        assert abs(float(mine.astype(np.float64).sum()) - 1.0) < 1e-5
+        e = np.exp(xs.astype(np.float64))
+        assert_close_f32(mine, e / e.sum(), rtol=1e-5, atol=0.0, what="softmax closed form")
     # accum
     b, bo = ref.fbuf(n, x), ref.fbuf(n, y0)
     assert ref.lib.sref_accum_f32(Cn, H, W, b.h, bo.h) == 0
