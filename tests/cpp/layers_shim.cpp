@@ -6,6 +6,7 @@
 // Tensors cross this boundary flat (NCHW / OIHW, unpacked): the shim packs inputs and unpacks
 // outputs with pack_buffer / unpack_buffer, as a user of the Layer API would.
 // Return value: 0 ok, 1 std::invalid_argument, 2 any other exception; stest_last_error() has the text.
+#include <chrono>
 #include <cstring>
 #include <memory>
 #include <string>
@@ -243,6 +244,47 @@ int stest_model_f32(int which, int variant, int batch, int C, int H, int W, cons
         auto x = packed_tensor<FB>(in, is);
         auto outs = m->inference(&x);
         unpack_tensor<FB>(*outs[0], out, out_shape);
+    });
+}
+
+// Milliseconds per inference() call of a model class on a resident input (synthetic filters and input made
+// here; `steps` timed calls after `warmup`, bracketed by stream synchronisation).  Same which / variant as above.
+int stest_model_time_f32(int which, int variant, int batch, int C, int H, int W, const size_t *sizes, int nfilters,
+                         int steps, int warmup, double *ms_per_call)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, (size_t)C, (size_t)H, (size_t)W};
+        std::vector<std::unique_ptr<FB>> own;
+        std::vector<FB *> fl;
+        for (int i = 0; i < nfilters; ++i)
+        {
+            own.emplace_back(new FB(sizes[i]));
+            float *p = own.back()->data();
+            for (size_t k = 0; k < sizes[i]; ++k) p[k] = 0.01f * float((int)((k * 2654435761u) >> 24) - 128) / 128.f;
+            fl.push_back(own.back().get());
+        }
+        std::unique_ptr<small::Model<FB>> m;
+        switch (which)
+        {
+        case 0: m.reset(variant ? new small::MobileNetTiny<FB>(is, fl, false, 32, 1000, true)
+                                : new small::MobileNetTiny<FB>(is, fl, false)); break;
+        case 1: m.reset(variant ? new small::Resnet8Tiny<FB>(is, fl, false, 10) : new small::Resnet8Tiny<FB>(is, fl, false)); break;
+        case 2: m.reset(variant ? new small::DSCNNTiny<FB>(is, fl, false, 10, 4, 12, true)
+                                : new small::DSCNNTiny<FB>(is, fl, false)); break;
+        case 3: m.reset(variant ? new small::TinyYoloV2<FB>(is, fl, false, small::LEAKY, 0.1f, 125, false)
+                                : new small::TinyYoloV2<FB>(is, fl, false)); break;
+        default: throw std::invalid_argument("stest_model_time_f32: unknown model");
+        }
+        small::Tensor<FB> x(is);
+        float *px = x.buffer().data();
+        for (size_t k = 0; k < x.size(); ++k) px[k] = float((int)((k * 40503u) & 255) - 128) / 128.f;
+        for (int i = 0; i < warmup; ++i) m->inference(&x);
+        small::synchronize();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < steps; ++i) m->inference(&x);
+        small::synchronize();
+        const auto t1 = std::chrono::steady_clock::now();
+        *ms_per_call = std::chrono::duration<double, std::milli>(t1 - t0).count() / steps;
     });
 }
 

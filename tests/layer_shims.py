@@ -113,6 +113,17 @@ class HipLayers(_Shim):
             build_hip_shim()
         super().__init__(C.CDLL(SHIM_SO), "stest_", True)
 
+    def model_time_f32(self, which, variant, shape, filter_sizes, steps=20, warmup=3):
+        """-> milliseconds per Model::inference() call at input shape (N, C, H, W)."""
+        n, c, h, w = shape
+        sizes = (C.c_size_t * len(filter_sizes))(*filter_sizes)
+        ms = C.c_double()
+        rc = self.lib.stest_model_time_f32(C.c_int(which), C.c_int(variant), C.c_int(n), C.c_int(c), C.c_int(h),
+                                           C.c_int(w), sizes, C.c_int(len(filter_sizes)), C.c_int(steps),
+                                           C.c_int(warmup), C.byref(ms))
+        self._check(rc)
+        return ms.value
+
     def conv_layer_u8(self, kind, x, iq, filters, fq, oq, act, kh, kw, stride, padding, out_init=None):
         n, c, h, w = x.shape
         co = filters.shape[0]

@@ -157,3 +157,15 @@ def test_resnet8_quantised_model(hip, oracle):
     want = ol.resnet8_tiny_u8(oracle, quant, x, iq, filters, fq, DEFAULT_Q)
     assert got.shape == want.shape == (batch, 16, 1, 1)
     assert_equal_exact(got, want, "Resnet8Tiny<QUInt8Buffer>")
+
+
+@pytest.mark.gpu
+def test_model_class_throughput(hip):
+    """MobileNetTiny<FloatBuffer> built as MobileNetV1 (224x224, 1000 classes) at batch 64: one
+    Model::inference() call is the same 29 launches bench.py times through the C ABI, so it must land in the
+    same range (the bound below is loose: 2x the bench figure recorded for this build, ~1.05 ms)."""
+    sizes = [int(np.prod(f.shape)) for f in ol.make_filters(synth, ol.mobilenet_specs(), 1000)]
+    ms = hip.model_time_f32(0, 1, (64, 3, 224, 224), sizes)
+    print("MobileNetTiny<FloatBuffer> (MobileNetV1 224x224, 1000 classes) batch 64: %.3f ms per inference, %.0f images/s"
+          % (ms, 64 / ms * 1e3))
+    assert ms < 2.2
