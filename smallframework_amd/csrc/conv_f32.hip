@@ -522,8 +522,15 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
 template <int CI>
 __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
 {
-    const int p = blockIdx.x * 256 + threadIdx.x;
-    if (p >= a.P) return;
+    // a lane computes all 16 channels of one output pixel; the wave's 64 x 16 results are turned round in a
+    // wave-private LDS tile so that every store instruction writes 1 KiB of consecutive bytes (a lane
+    // storing its own 64 bytes in four pieces touches a quarter of each line per instruction)
+    constexpr int ROW = CB + 4;                              // padded pixel row in floats
+    __shared__ __align__(16) float tile[4][WAVE * ROW];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int p0 = blockIdx.x * 256 + threadIdx.x;
+    const bool live = p0 < a.P;
+    const int p = live ? p0 : 0;
     const int cob = blockIdx.y;
     const int HoWo = a.Ho * a.Wo;
     const int n = p / HoWo;
@@ -533,54 +540,65 @@ __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
     const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
     const float *img = a.in + (size_t)n * a.H * a.W * CI;
     const float *w = a.filt + (size_t)cob * a.kh * a.kw * CI * CB;
-    float *o = a.out + (((size_t)n * (a.Co / CB) + cob) * HoWo + rem) * CB;
 
     float acc[CB];
-    if (a.accumulate)
+#pragma unroll
+    for (int j = 0; j < CB; ++j) acc[j] = 0.f;
+    // One window tap per iteration, straight-line inside (a padded tap reads the zero block): the tap's
+    // CI x 16 weights are uniform, i.e. scalar loads feeding the FMAs directly.  The loop is kept rolled on
+    // purpose: unrolled, the compiler hoists all kh*kw*CI*16 scalar weights and spills them.
+    const int taps = a.kh * a.kw;
+    int ta = 0, tb = 0;
+#pragma unroll 1
+    for (int tap = 0; tap < taps; ++tap)
     {
+        const int ih = ih0 + ta, iw = iw0 + tb;
+        const bool ok = live && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+        const float *ip = ok ? img + (ih * a.W + iw) * CI : g_zero_block;
+        const float *wp = w + tap * (CI * CB);
+        float x[CI];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-        {
-            const float4 v = reinterpret_cast<const float4 *>(o)[q];
-            acc[4 * q] = v.x; acc[4 * q + 1] = v.y; acc[4 * q + 2] = v.z; acc[4 * q + 3] = v.w;
-        }
+        for (int ci = 0; ci < CI; ++ci) x[ci] = ip[ci];
+#pragma unroll
+        for (int ci = 0; ci < CI; ++ci)
+#pragma unroll
+            for (int j = 0; j < CB; ++j) acc[j] = fmaf(x[ci], wp[ci * CB + j], acc[j]);
+        if (++tb == a.kw) { tb = 0; ++ta; }
     }
-    else
-    {
-#pragma unroll
-        for (int j = 0; j < CB; ++j) acc[j] = a.bias ? a.bias[cob * CB + j] : 0.f;
-    }
-    for (int ta = 0; ta < a.kh; ++ta)
-    {
-        const int ih = ih0 + ta;
-        if (ih < 0 || ih >= a.H) continue;
-        for (int tb = 0; tb < a.kw; ++tb)
-        {
-            const int iw = iw0 + tb;
-            if (iw < 0 || iw >= a.W) continue;
-            const float *ip = img + ((size_t)ih * a.W + iw) * CI;
-            const float *wp = w + (size_t)(ta * a.kw + tb) * CI * CB;
-#pragma unroll
-            for (int ci = 0; ci < CI; ++ci)
-            {
-                const float x = ip[ci];
-#pragma unroll
-                for (int j = 0; j < CB; ++j) acc[j] = fmaf(x, wp[ci * CB + j], acc[j]);
-            }
-        }
-    }
+    float *mine = &tile[wave][lane * ROW];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
+        reinterpret_cast<float4 *>(mine)[q] = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+    // the pixel's position in the output travels with its row (in the padding): consecutive pixels of the
+    // wave's run are consecutive in the output except where the run crosses into the next image
+    const unsigned long long opos = (((unsigned long long)n * (a.Co / CB) + cob) * HoWo + rem) * CB;
+    *reinterpret_cast<uint2 *>(mine + CB) = make_uint2((unsigned)opos, (unsigned)(opos >> 32));
+    __syncthreads();
+    // vector v of the wave's 64-pixel run: pixel v / 4, channel quad v % 4
+    const float nscale = act_scale(a.act, a.slope);
+    const int wave_p0 = blockIdx.x * 256 + wave * WAVE;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
     {
-        float4 v = make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
-        if (a.accumulate && a.bias)
+        const int v = j * WAVE + lane, px = v >> 2, q = v & 3;
+        if (wave_p0 + px < a.P)
         {
-            v.x += a.bias[cob * CB + 4 * q]; v.y += a.bias[cob * CB + 4 * q + 1];
-            v.z += a.bias[cob * CB + 4 * q + 2]; v.w += a.bias[cob * CB + 4 * q + 3];
+            const uint2 op = *reinterpret_cast<const uint2 *>(&tile[wave][px * ROW + CB]);
+            float4 *o = reinterpret_cast<float4 *>(a.out + (((unsigned long long)op.y << 32) | op.x)) + q;
+            float4 r = *reinterpret_cast<const float4 *>(&tile[wave][px * ROW + q * 4]);
+            if (a.accumulate)
+            {
+                const float4 old = *o;
+                r.x += old.x; r.y += old.y; r.z += old.z; r.w += old.w;
+            }
+            if (a.bias)
+            {
+                const float4 b = *reinterpret_cast<const float4 *>(a.bias + cob * CB + q * 4);
+                r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w;
+            }
+            r.x = act_bf(r.x, nscale); r.y = act_bf(r.y, nscale); r.z = act_bf(r.z, nscale); r.w = act_bf(r.w, nscale);
+            *o = r;
         }
-        v.x = act1(v.x, a.act, a.slope); v.y = act1(v.y, a.act, a.slope);
-        v.z = act1(v.z, a.act, a.slope); v.w = act1(v.w, a.act, a.slope);
-        reinterpret_cast<float4 *>(o)[q] = v;
     }
 }
 
