@@ -710,6 +710,130 @@ __global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvAr
     conv_epilogue<1, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
+// First layers with a 3x3 window (Ci in {1,2,3}), any multiple of 16 output channels: the input patch
+// under a 16 x 16 tile of output pixels is staged ONCE per workgroup in LDS (coalesced row segments of the
+// [H][W][Ci] image, zero where the window leaves the image), and the product runs on
+// v_mfma_f32_16x16x4_f32: rows = the 16 channels of the block, columns = the 16 pixels of one tile row,
+// K-step = four consecutive reduction elements k = tap * Ci + ci, one per 16-lane group.  In LDS the patch
+// has a compile-time pitch, so the position of (tap, ci) relative to a lane's pixel is a compile-time
+// constant: a B operand costs one LDS read with an immediate offset, where a gather from global memory
+// costs about eight address instructions per element (what bounds the kernels above on these layers).
+// A lane ends up with four consecutive channels of one pixel; a store instruction covers 16 pixels x 64
+// bytes of consecutive memory.  Wave w owns tile rows 4w .. 4w+3; a workgroup runs NCOB channel blocks on
+// the patch it staged.
+template <int CI, int S, int NCOB>
+__global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArgs a, int tiles_x, int tiles_y)
+{
+    typedef float floatx4v __attribute__((ext_vector_type(4)));
+    constexpr int T = 16;                                    // tile side in output pixels
+    constexpr int PH = (T - 1) * S + 3, PW = PH;             // input patch in pixels
+    constexpr int PITCH = PW * CI;                           // floats per patch row
+    constexpr int NEL = PH * PITCH;
+    constexpr int K = 9 * CI, NS = (K + 3) / 4;
+    __shared__ float patch[NEL];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, kq = lane >> 4;
+    const int CoB = a.Co / CB;
+    const int HoWo = a.Ho * a.Wo;
+    int tile = blockIdx.x;
+    const int n = tile / (tiles_x * tiles_y);
+    tile -= n * (tiles_x * tiles_y);
+    const int ty = tile / tiles_x, tx = tile - ty * tiles_x;
+    const int oh0 = ty * T, ow0 = tx * T;
+    const int ih_base = oh0 * S - a.pt, iw_base = ow0 * S - a.pl;
+
+    // ---- stage the patch: element e = (patch row, position inside the row segment) ------------------
+    const float *img = a.in + (size_t)n * a.H * a.W * CI;
+    const int row_el = a.W * CI;                             // floats per image row
+    constexpr int PER_THREAD = (NEL + 255) / 256;
+    float pv[PER_THREAD];
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j)
+    {
+        const int e = tid + j * 256;
+        const int py = e / PITCH, x = e - py * PITCH;
+        const int ih = ih_base + py, xe = iw_base * CI + x;
+        const bool ok = e < NEL && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
+        const float *src = ok ? img + ih * row_el + xe : g_zero_block;
+        pv[j] = *src;
+    }
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j)
+        if (tid + j * 256 < NEL) patch[tid + j * 256] = pv[j];
+    __syncthreads();
+
+    // patch position of (tap, ci) for this lane's k, relative to the lane's pixel: compile-time per lane group
+    const int lane_base = (4 * wave * S * PW + col * S) * CI;   // pixel (row 4w, column col); tile row t adds t*S*PITCH
+    int off[NS];
+    bool kvalid[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        off[s] = 0;
+        kvalid[s] = true;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+        {
+            const int k = 4 * s + g;                         // compile-time
+            const int kc = k < K ? k : 0;
+            const int tap = kc / CI, ci = kc % CI;
+            const int o = ((tap / 3) * PW + tap % 3) * CI + ci;
+            if (kq == g) { off[s] = lane_base + o; kvalid[s] = k < K; }
+        }
+    }
+    const float nscale = act_scale(a.act, a.slope);
+    const int ow = ow0 + col;
+
+    // ---- the workgroup's channel blocks, one after the other on the same patch ------------------------
+#pragma unroll
+    for (int cb_i = 0; cb_i < NCOB; ++cb_i)
+    {
+        const int cob = blockIdx.y * NCOB + cb_i;            // the launcher makes Co / 16 a multiple of NCOB
+        // filter: element k of channel co at w_blk[k * 16 + co % 16]; this lane's k in step s is 4s + kq
+        const float *w_blk = a.filt + (size_t)cob * (K * CB) + col;
+        float av[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            const int k = 4 * s + kq;
+            const float *wp = k < K ? w_blk + k * CB : g_zero_block;
+            av[s] = *wp;
+        }
+        floatx4v acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t] = floatx4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+            {
+                const float b = patch[off[s] + t * (S * PITCH)];
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], kvalid[s] ? b : 0.f, acc[t], 0, 0, 0);
+            }
+        // lane: channels cob*16 + 4*kq .. +3 of pixel (oh0 + 4w + t, ow0 + col)
+        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+        {
+            const int oh = oh0 + 4 * wave + t;
+            const bool ok = oh < a.Ho && ow < a.Wo;
+            float4 *o = reinterpret_cast<float4 *>(a.out + (((size_t)n * CoB + cob) * HoWo + (ok ? oh * a.Wo + ow : 0)) * CB + 4 * kq);
+            float4 v = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+            if (a.accumulate)
+            {
+                float4 old = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (ok) old = *o;
+                v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+            }
+            v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+            v.x = act_bf(v.x, nscale); v.y = act_bf(v.y, nscale); v.z = act_bf(v.z, nscale); v.w = act_bf(v.w, nscale);
+            if (ok) *o = v;
+        }
+    }
+}
+
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
@@ -774,6 +898,27 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
 
     if (small_ci)
     {
+        // 3x3 windows: the LDS-staged 16x16x4 MFMA kernel (tuning knob SMALL_HIP_STEM_LDS=0 switches it off)
+        static const bool stem_lds_off = [] { const char *e = std::getenv("SMALL_HIP_STEM_LDS"); return e && e[0] == '0'; }();
+        if (!stem_lds_off && kh == 3 && kw == 3 && (long)H * W * Ci < 0x7fffffffL)
+        {
+            const int tiles_x = (a.Wo + 15) / 16, tiles_y = (a.Ho + 15) / 16;
+            const long nt = (long)batch * tiles_x * tiles_y;
+            if (nt <= 0x7fffffffL)
+            {
+                const int CoB = Co / CB;
+                const int ncob = CoB % 4 == 0 ? 4 : CoB % 2 == 0 ? 2 : 1;
+                const dim3 gs((unsigned)nt, (unsigned)(CoB / ncob));
+                void (*ks)(const ConvArgs, int, int) = nullptr;
+#define SHP_STEM(CI_, S_) (ncob == 4 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 4> : ncob == 2 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 2> : conv_stem3x3_lds_f32_kernel<CI_, S_, 1>)
+                if (stride == 1) ks = Ci == 1 ? SHP_STEM(1, 1) : Ci == 2 ? SHP_STEM(2, 1) : SHP_STEM(3, 1);
+                else ks = Ci == 1 ? SHP_STEM(1, 2) : Ci == 2 ? SHP_STEM(2, 2) : SHP_STEM(3, 2);
+#undef SHP_STEM
+                hipLaunchKernelGGL(ks, gs, dim3(256), 0, s, a, tiles_x, tiles_y);
+                SHP_LAUNCH_CHECK(op);
+                return SMALL_HIP_OK;
+            }
+        }
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
         static const bool smallci_valu = [] { const char *e = std::getenv("SMALL_HIP_SMALLCI_VALU"); return e && e[0] == '1'; }();
         // measured: with 16 output channels half of every 32-row MFMA tile is idle and the vector-ALU
