@@ -68,11 +68,27 @@ def time_forward(ex, steps, warmup):
 
 
 def time_ops(ex, steps):
-    """Per-op device time (ms) from HIP events on the launch stream, averaged over `steps`."""
+    """Per-op device time (ms) from HIP events on the launch stream, averaged over `steps`.  Float32 models are
+    timed launch by launch as the forward pass issues them: a convolution that carries its 2x2 max-pool has the
+    time of the fused launch, and the pool's own row reads 0.  (uint8 models are timed op by op, unfused.)"""
     import torch
     ops = ex.model.ops
-    tot = [0.0] * len(ops)
     st = ex.stream()
+    if ex.model.dtype == "f32" and ex.fused:
+        entries = ex.plan
+        index = {op.name: i for i, op in enumerate(ops)}
+        tot = [0.0] * len(ops)
+        for _ in range(steps):
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(entries) + 1)]
+            evs[0].record()
+            for i, e in enumerate(entries):
+                ex.run_entry(e, st)
+                evs[i + 1].record()
+            torch.cuda.synchronize()
+            for i, e in enumerate(entries):
+                tot[index[e[0].name]] += evs[i].elapsed_time(evs[i + 1])
+        return [t / steps for t in tot]
+    tot = [0.0] * len(ops)
     for _ in range(steps):
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)]
         evs[0].record()
@@ -86,12 +102,25 @@ def time_ops(ex, steps):
 
 
 def layer_table(model, batch, ms):
+    """Per-op rows.  A convolution that carried the following 2x2 max-pool in its launch is priced on the fused
+    launch's own algorithmic bytes (its input + the pooled output + the filter); the pool's row is empty."""
     rows = []
-    for op, t in zip(model.ops, ms):
+    ops = model.ops
+    es = model.esize()
+    for i, (op, t) in enumerate(zip(ops, ms)):
         tb, kind = op_bound(model, op, batch)
+        nbytes = op_bytes(model, op, batch)
+        if t == 0.0 and op.kind == "maxpool":
+            rows.append({"layer": op.name, "ms": 0.0, "bound": kind, "roofline_frac": None, "GB/s": None,
+                         "TFLOP/s": None, "fused_into": "previous convolution"})
+            continue
+        if op.kind == "conv" and i + 1 < len(ops) and ops[i + 1].kind == "maxpool" and ms[i + 1] == 0.0:
+            nbytes = batch * (op.act_elems()[0] + ops[i + 1].act_elems()[1]) * es + op.weight_elems() * es
+            if kind == "hbm" or nbytes / PEAK_HBM > tb:
+                tb, kind = nbytes / PEAK_HBM, "hbm"
         rows.append({"layer": op.name, "ms": round(t, 5), "bound": kind,
                      "roofline_frac": round(tb / (t * 1e-3), 4) if t > 0 else None,
-                     "GB/s": round(op_bytes(model, op, batch) / (t * 1e-3) / 1e9, 1) if t > 0 else None,
+                     "GB/s": round(nbytes / (t * 1e-3) / 1e9, 1) if t > 0 else None,
                      "TFLOP/s": round(batch * op.flops() / (t * 1e-3) / 1e12, 2) if t > 0 and op.flops() else None})
     return rows
 

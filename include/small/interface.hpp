@@ -23,6 +23,7 @@
 
 #include "../small_hip.h"
 #include "Buffer.hpp"
+#include "utils.hpp"
 
 namespace small
 {
@@ -172,6 +173,45 @@ void Conv2D_Accum_ReLU(int batch, int kernel_height, int kernel_width, int strid
                                             input_buf.device_in(), &iq, filter_buf.device_in(), &fq, acc, &aq,
                                             relu ? 1 : 0, output_buf.device_out(), &oq, detail::st());
     detail::raise<BufferT>(rc, "Conv2D");
+}
+
+// out = MaxPool2D(act(Conv2D(in, filter) + bias)) in one launch when the pooling window is 2x2 stride 2 without
+// padding (the pooling runs on the accumulators); any other window runs the two layers through
+// inter_output_buf.  bias_buf may be empty.
+template <class BufferT, detail::if_float<BufferT> = true>
+void Conv2D_Bias_Act_Maxpool2D(int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride,
+                               uint8_t conv_t_pad, uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad,
+                               int pool_kernel_height, int pool_kernel_width, int pool_stride, uint8_t pool_t_pad,
+                               uint8_t pool_b_pad, uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels,
+                               int input_channels, int input_height, int input_width, BufferT const &input_buf,
+                               BufferT const &filter_buf, BufferT const &bias_buf, ActivationType act,
+                               float negative_slope, BufferT &inter_output_buf, BufferT &output_buf)
+{
+    const bool fusable = pool_kernel_height == 2 && pool_kernel_width == 2 && pool_stride == 2 && !pool_t_pad &&
+                         !pool_b_pad && !pool_l_pad && !pool_r_pad &&
+                         (input_channels % (int)BufferT::C_ib == 0 || (conv_kernel_height == 3 && conv_kernel_width == 3)) &&
+                         !(act == LEAKY && negative_slope < 0.f);
+    if (fusable)
+    {
+        detail::raise<BufferT>(
+            small_hip_conv2d_bias_act_maxpool2d_f32(
+                batch, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
+                conv_r_pad, 2, 2, 2, 0, 0, 0, 0, output_channels, input_channels, input_height, input_width,
+                input_buf.device_in(), filter_buf.device_in(), bias_buf.size() ? bias_buf.device_in() : nullptr,
+                (int)act, negative_slope, output_buf.device_out(), detail::st()),
+            "Conv2D_Bias_ReLU_Maxpool2D");
+        return;
+    }
+    Conv2D_Bias_Act(batch, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
+                    conv_r_pad, output_channels, input_channels, input_height, input_width, input_buf, filter_buf,
+                    bias_buf, act, negative_slope, inter_output_buf);
+    const int Ho = (int)output_dim(input_height + conv_t_pad + conv_b_pad, conv_stride, conv_kernel_height);
+    const int Wo = (int)output_dim(input_width + conv_l_pad + conv_r_pad, conv_stride, conv_kernel_width);
+    detail::raise<BufferT>(small_hip_maxpool2d_f32(batch, pool_kernel_height, pool_kernel_width, pool_stride,
+                                                   pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad, output_channels,
+                                                   Ho, Wo, inter_output_buf.device_in(), output_buf.device_out(),
+                                                   detail::st()),
+                           "MaxPool2D");
 }
 
 // ---- DepthwiseConv2D / PartialDepthwiseConv2D ------------------------------------------------------
@@ -548,6 +588,54 @@ void Dense(int output_elements, int input_elements, BufferT const &input_buf, Bu
            BufferT &output_buf)
 {
     batched::Dense(1, output_elements, input_elements, input_buf, filter_buf, output_buf);
+}
+
+// The reference's fused convolution + pooling functions (fused_interface_abstract.hpp:354, 998, 683), same
+// signatures; inter_output_buf is only written when the pooling window cannot be fused.
+template <class BufferT>
+void Conv2D_Bias_ReLU_Maxpool2D(int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad,
+                                uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad, int pool_kernel_height,
+                                int pool_kernel_width, int pool_stride, uint8_t pool_t_pad, uint8_t pool_b_pad,
+                                uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels, int input_channels,
+                                int input_height, int input_width, BufferT const &input_buf,
+                                BufferT const &filter_buf, BufferT const &bias_buf, BufferT &inter_output_buf,
+                                BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_Maxpool2D(1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad,
+                                       conv_l_pad, conv_r_pad, pool_kernel_height, pool_kernel_width, pool_stride,
+                                       pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad, output_channels,
+                                       input_channels, input_height, input_width, input_buf, filter_buf, bias_buf,
+                                       RELU, 0.f, inter_output_buf, output_buf);
+}
+
+template <class BufferT>
+void Conv2D_ReLU_Maxpool2D(int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad,
+                           uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad, int pool_kernel_height,
+                           int pool_kernel_width, int pool_stride, uint8_t pool_t_pad, uint8_t pool_b_pad,
+                           uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels, int input_channels,
+                           int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                           BufferT &inter_output_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_Maxpool2D(1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad,
+                                       conv_l_pad, conv_r_pad, pool_kernel_height, pool_kernel_width, pool_stride,
+                                       pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad, output_channels,
+                                       input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
+                                       RELU, 0.f, inter_output_buf, output_buf);
+}
+
+template <class BufferT>
+void Conv2D_Maxpool2D(int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad,
+                      uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad, int pool_kernel_height,
+                      int pool_kernel_width, int pool_stride, uint8_t pool_t_pad, uint8_t pool_b_pad,
+                      uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels, int input_channels,
+                      int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                      BufferT &inter_output_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_Maxpool2D(1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad,
+                                       conv_l_pad, conv_r_pad, pool_kernel_height, pool_kernel_width, pool_stride,
+                                       pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad, output_channels,
+                                       input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
+                                       NONE, 0.f, inter_output_buf, output_buf);
 }
 
 // small::Dense exactly as the reference writes it (interface_abstract.hpp:2113-2132):

@@ -106,6 +106,23 @@ int small_hip_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width
                                   int input_channels, int input_height, int input_width,
                                   const float *input, const float *filter, const float *bias,
                                   int act, float slope, float *output, small_hip_stream_t stream);
+/* small::Conv2D_Bias_ReLU_Maxpool2D / Conv2D_ReLU_Maxpool2D / Conv2D_Maxpool2D
+ * (include/small/fused_interface_abstract.hpp:354, 998, 683) in one launch:
+ *     out = MaxPool2D( act( Conv2D(in, filter) + bias ) )
+ * with the pooling done on the accumulators (the convolution's own output never goes to memory; no
+ * intermediate buffer is needed).  Fused here for a 2x2 stride-2 pooling window without padding (EINVAL
+ * otherwise: issue the two layers); the convolution may be any this library runs except first layers with a
+ * window other than 3x3.  output is [batch][Co/16][Ho/2][Wo/2][16].  The result equals the two layers run one
+ * after the other bit for bit (max commutes with the monotone activations; a negative LeakyReLU slope is
+ * rejected). */
+int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                            int t_pad, int b_pad, int l_pad, int r_pad, int pool_kernel_height,
+                                            int pool_kernel_width, int pool_stride, int pool_t_pad,
+                                            int pool_b_pad, int pool_l_pad, int pool_r_pad,
+                                            int output_channels, int input_channels, int input_height,
+                                            int input_width, const float *input, const float *filter,
+                                            const float *bias, int act, float negative_slope, float *output,
+                                            small_hip_stream_t stream);
 /* PartialConv2DLayer::compute_output (include/small/PartialConv2DLayer.hpp:407-463) in one pass:
  * out = act((out + conv(in, filter)) + bias), i.e. PartialConv2D + PartialBias + activation. */
 int small_hip_partial_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,

@@ -142,6 +142,45 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
     else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
+// Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 4 rows x 8
+// columns of the convolution's output (lane col = row * 8 + column), so a pooling window is this lane, lane
+// ^ 1 (next column) and lanes ^ 8 (next row): bias and activation, two shuffles and maxima per value, and
+// the lanes at even row and even column store the pooled pixel into [N][Co/16][Ho/2][Wo/2][16].
+template <int COT, int PXT>
+__device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
+                                                   const bool (&pool_ok)[PXT], const size_t (&pool_pix)[PXT])
+{
+    const float nscale = act_scale(a.act, a.slope);
+    const int HpWp = (a.Ho >> 1) * (a.Wo >> 1);
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int co4 = (cg * COT + c) * 32 + 8 * q + 4 * half;
+            float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (a.bias && co4 < a.Co) bb = *reinterpret_cast<const float4 *>(a.bias + co4);
+            const float b4[4] = {bb.x, bb.y, bb.z, bb.w};
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                float m[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    float v = act_bf(acc[c][t][4 * q + e] + b4[e], nscale);
+                    const float u = __shfl_xor(v, 1, WAVE);
+                    v = v > u ? v : u;
+                    const float w = __shfl_xor(v, 8, WAVE);
+                    m[e] = v > w ? v : w;
+                }
+                if (pool_ok[t] && co4 < a.Co)
+                    *reinterpret_cast<float4 *>(a.out + pool_pix[t] + (size_t)(co4 / CB) * HpWp * CB + (co4 % CB)) =
+                        make_float4(m[0], m[1], m[2], m[3]);
+            }
+        }
+}
+
 // ---------------------------------------------------------------------------------------------
 // The main kernel body: filter operand staged through LDS.  The four waves of a workgroup
 // multiply the same output-channel group, so the step's [16 ci][16 co] filter tiles (COT*2 KiB)
@@ -152,7 +191,7 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
 // the MFMA register, two 16-byte loads per lane and tile.
 constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks start 16 banks apart
 
-template <int COT, int PXT>
+template <int COT, int PXT, bool POOL = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
                                               const int cg, const int pxb)
 {
@@ -173,20 +212,44 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
+    bool pool_ok[PXT];           // POOL: this lane stores the pooled pixel of its window
 #pragma unroll
     for (int t = 0; t < PXT; ++t)
     {
-        const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
-        pvalid[t] = p < a.P;
-        const int pc = pvalid[t] ? p : 0;
-        const int n = pc / HoWo;
-        const int rem = pc - n * HoWo;
-        const int oh = rem / a.Wo;
-        const int ow = rem - oh * a.Wo;
+        int n, oh, ow, rem;
+        if (POOL)
+        {
+            // tiles of 4 rows x 8 columns of one image (a.P = number of tiles * 32)
+            const int tile = (pxb * 4 + wave) * PXT + t;
+            const int tiles_x = (a.Wo + 7) >> 3, tiles_y = (a.Ho + 3) >> 2;
+            const int tl = tile * 32 < a.P ? tile : 0;
+            n = tl / (tiles_x * tiles_y);
+            const int tin = tl - n * (tiles_x * tiles_y);
+            const int ty = tin / tiles_x, tx = tin - ty * tiles_x;
+            oh = ty * 4 + (col >> 3);
+            ow = tx * 8 + (col & 7);
+            pvalid[t] = tile * 32 < a.P && oh < a.Ho && ow < a.Wo;
+            if (!pvalid[t]) { oh = 0; ow = 0; }
+            rem = oh * a.Wo + ow;
+            const int Hp = a.Ho >> 1, Wp = a.Wo >> 1;
+            pool_ok[t] = pvalid[t] && ((col & 9) == 0) && (oh >> 1) < Hp && (ow >> 1) < Wp;
+            out_pix[t] = ((size_t)n * CoB * (Hp * Wp) + (size_t)((oh >> 1) * Wp + (ow >> 1))) * CB;
+        }
+        else
+        {
+            const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
+            pvalid[t] = p < a.P;
+            const int pc = pvalid[t] ? p : 0;
+            n = pc / HoWo;
+            rem = pc - n * HoWo;
+            oh = rem / a.Wo;
+            ow = rem - oh * a.Wo;
+            pool_ok[t] = false;
+            out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+        }
         ih0[t] = oh * a.stride - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
-        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
     }
 
     // ---- cooperative filter fetch: COT*2 tiles of 64 float4 each -----------------------------
@@ -308,20 +371,21 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // an odd step count leaves the last step staged in buffer 0 / B0 (the loop's invariant)
     if (nsteps & 1) multiply(0, B0);
 
-    conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix);
+    else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
 // The second launch bound (minimum waves per SIMD: 6 / 5 / 2 for one / two / four MFMA tiles per
 // wave) makes the compiler keep the accumulators in the unified register file and pack tighter
 // (2x1: 108 -> 76 registers, 2x2: 184 -> 131, no spills); measured 1-3% faster, tighter bounds spill.
-template <int COT, int PXT>
+template <int COT, int PXT, bool POOL = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a)
 {
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
-    conv_lds_tile<COT, PXT>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+    conv_lds_tile<COT, PXT, POOL>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -721,7 +785,7 @@ __global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvAr
 // A lane ends up with four consecutive channels of one pixel; a store instruction covers 16 pixels x 64
 // bytes of consecutive memory.  Wave w owns tile rows 4w .. 4w+3; a workgroup runs NCOB channel blocks on
 // the patch it staged.
-template <int CI, int S, int NCOB>
+template <int CI, int S, int NCOB, bool POOL = false>
 __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArgs a, int tiles_x, int tiles_y)
 {
     typedef float floatx4v __attribute__((ext_vector_type(4)));
@@ -814,6 +878,32 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
         // lane: channels cob*16 + 4*kq .. +3 of pixel (oh0 + 4w + t, ow0 + col)
         float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
         if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
+        if (POOL)
+        {
+            // MaxPool2D 2x2 stride 2 (no padding) of the activated result, in registers: tile rows t and
+            // t+1 are this lane's own accumulators, the neighbouring column is lane ^ 1.  Even columns
+            // store; the output tensor is [N][Co/16][Ho/2][Wo/2][16].
+            const int Hp = a.Ho >> 1, Wp = a.Wo >> 1;
+#pragma unroll
+            for (int t = 0; t < 4; t += 2)
+            {
+                float m[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    const float be = e == 0 ? bb.x : e == 1 ? bb.y : e == 2 ? bb.z : bb.w;
+                    const float v0 = act_bf(acc[t][e] + be, nscale), v1 = act_bf(acc[t + 1][e] + be, nscale);
+                    const float v = v0 > v1 ? v0 : v1;
+                    const float u = __shfl_xor(v, 1, WAVE);
+                    m[e] = v > u ? v : u;
+                }
+                const int ohp = (oh0 + 4 * wave + t) >> 1, owp = ow >> 1;
+                if ((col & 1) == 0 && ohp < Hp && owp < Wp)
+                    *reinterpret_cast<float4 *>(a.out + (((size_t)n * CoB + cob) * (Hp * Wp) + ohp * Wp + owp) * CB + 4 * kq) =
+                        make_float4(m[0], m[1], m[2], m[3]);
+            }
+            continue;
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
         {
@@ -980,6 +1070,84 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     return SMALL_HIP_OK;
 }
 
+template <int COT, int PXT>
+void launch_mfma_pool(ConvArgs &a, hipStream_t s)
+{
+    a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
+    a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
+    a.n_blocks = a.n_co_groups * a.n_px_blocks;
+    a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
+    hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+}
+
+// Conv2D + bias + activation + MaxPool2D 2x2 stride 2 (no pool padding) in one launch
+int conv_pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int pool_kh,
+                  int pool_kw, int pool_stride, int ppt, int ppb, int ppl, int ppr, int Co, int Ci, int H, int W,
+                  const float *in, const float *filt, const float *bias, int act, float slope, float *out,
+                  small_hip_stream_t stream)
+{
+    const bool blocked = Ci > 0 && Ci % CB == 0;
+    const bool small_ci = Ci == 1 || Ci == 2 || Ci == 3;
+    if (!blocked && !small_ci) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (pool_kh != 2 || pool_kw != 2 || pool_stride != 2 || ppt || ppb || ppl || ppr)
+    { set_error("%s: only a 2x2 stride-2 pooling window without padding is fused", op); return SMALL_HIP_EINVAL; }
+    if (small_ci && (kh != 3 || kw != 3))
+    { set_error("%s: first layers (1-3 input channels) are fused for 3x3 windows only", op); return SMALL_HIP_EINVAL; }
+    if (batch <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (Co % CB != 0) { set_error("%s: output_channels must be a multiple of 16 (pad the filter)", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out || !aligned16(filt) || !aligned16(out) || (blocked && !aligned16(in)) ||
+        (bias && !aligned16(bias)))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place operation is not supported", op); return SMALL_HIP_EINVAL; }
+    if (act < SMALL_HIP_ACT_NONE || act > SMALL_HIP_ACT_LEAKY) { set_error("%s: bad activation", op); return SMALL_HIP_EINVAL; }
+    if (act == SMALL_HIP_ACT_LEAKY && slope < 0.f)
+    { set_error("%s: a negative slope is not monotone; issue the layers separately", op); return SMALL_HIP_EINVAL; }
+
+    ConvArgs a{};
+    a.in = in; a.filt = filt; a.bias = bias; a.out = out;
+    a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W;
+    a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
+    a.Ho = out_dim(H, pt, pb, kh, stride);
+    a.Wo = out_dim(W, pl, pr, kw, stride);
+    a.act = act; a.slope = slope; a.accumulate = 0;
+    if (a.Ho < 2 || a.Wo < 2) return SMALL_HIP_OK;        // no pooling window fits: empty output
+    if ((long)Ci * H * W > 0x7fffffffL / 2 || (long)Ci * kh * kw * CB > 0x7fffffffL / 2)
+    { set_error("%s: one image or one filter block too large for 32-bit offsets", op); return SMALL_HIP_EINVAL; }
+    hipStream_t s = as_stream(stream);
+    if (small_ci)
+    {
+        const int tiles_x = (a.Wo + 15) / 16, tiles_y = (a.Ho + 15) / 16;
+        const long nt = (long)batch * tiles_x * tiles_y;
+        if (nt > 0x7fffffffL) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
+        a.P = batch * a.Ho * a.Wo;
+        const int CoB = Co / CB;
+        const int ncob = CoB % 4 == 0 ? 4 : CoB % 2 == 0 ? 2 : 1;
+        const dim3 gs((unsigned)nt, (unsigned)(CoB / ncob));
+        void (*ks)(const ConvArgs, int, int) = nullptr;
+#define SHP_STEM(CI_, S_) (ncob == 4 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 4, true> : ncob == 2 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 2, true> : conv_stem3x3_lds_f32_kernel<CI_, S_, 1, true>)
+        if (stride == 1) ks = Ci == 1 ? SHP_STEM(1, 1) : Ci == 2 ? SHP_STEM(2, 1) : SHP_STEM(3, 1);
+        else ks = Ci == 1 ? SHP_STEM(1, 2) : Ci == 2 ? SHP_STEM(2, 2) : SHP_STEM(3, 2);
+#undef SHP_STEM
+        hipLaunchKernelGGL(ks, gs, dim3(256), 0, s, a, tiles_x, tiles_y);
+        SHP_LAUNCH_CHECK(op);
+        return SMALL_HIP_OK;
+    }
+    // pixel tiles of 4 rows x 8 columns; P counts tile slots
+    const long ntiles = (long)batch * ((a.Ho + 3) / 4) * ((a.Wo + 7) / 8);
+    if (ntiles > 0x7fffffffL / 64) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
+    a.P = (int)(ntiles * 32);
+    const long tiles32 = (long)((Co + 31) / 32) * ntiles;
+    const long simds = 4L * NUM_CU;
+    const int nsteps = kh * kw * (Ci / CB);
+    if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) launch_mfma_pool<2, 2>(a, s);
+    else if (Co % 64 == 0 && tiles32 >= 4 * simds) launch_mfma_pool<2, 1>(a, s);
+    else launch_mfma_pool<1, 1>(a, s);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -1016,6 +1184,16 @@ int small_hip_partial_conv2d_bias_act_f32(int batch, int kh, int kw, int stride,
 {
     return conv_f32("small_hip_partial_conv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W,
                     in, filt, bias, act, slope, 1, out, stream);
+}
+
+int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                            int pool_kh, int pool_kw, int pool_stride, int ppt, int ppb, int ppl,
+                                            int ppr, int Co, int Ci, int H, int W, const float *in, const float *filt,
+                                            const float *bias, int act, float slope, float *out,
+                                            small_hip_stream_t stream)
+{
+    return conv_pool_f32("small_hip_conv2d_bias_act_maxpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, pool_kh,
+                         pool_kw, pool_stride, ppt, ppb, ppl, ppr, Co, Ci, H, W, in, filt, bias, act, slope, out, stream);
 }
 
 int small_hip_dense_f32(int batch, int No, int Ni, const float *in, const float *filt, float *out,

@@ -12,7 +12,7 @@ Topologies (synthetic weights; shapes as the benchmark configurations name them)
   layer_sweep()  single layers at C=256, 56x56
 """
 import ctypes as C
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Dict, List, Optional, Tuple
 
 import numpy as np
@@ -351,8 +351,11 @@ class HipExecutor:
         weights = weights if weights is not None else make_weights(model)
         x = x if x is not None else make_input(model, batch)
         self.w = {k: torch.from_numpy(v).to("cuda") for k, v in weights.items()}
-        self.buf = {k: torch.zeros(batch * n, dtype=self.tdtype, device="cuda")
-                    for k, n in buffer_elems(model).items()}
+        need = buffer_elems(model)
+        if fused and model.dtype == "f32":        # fused groups make buffer names trade places: one size for all
+            big = max(n for k, n in need.items() if k != "in")
+            need = {k: (n if k == "in" else big) for k, n in need.items()}
+        self.buf = {k: torch.zeros(batch * n, dtype=self.tdtype, device="cuda") for k, n in need.items()}
         self.buf["in"].copy_(torch.from_numpy(x))
         self.q = {k: capi.Quant(*v) for k, v in model.quant.items()}
         self.prep = {}
@@ -365,13 +368,32 @@ class HipExecutor:
                     capi.check(self.lib.small_hip_conv2d_u8_prepare_filter(op.kh, op.kw, op.Co, op.C,
                                                                            self._p(self.w[op.weight]), self._p(t), st))
                     self.prep[op.weight] = t
-        # uint8 residual blocks: Conv2D [+ Accum onto its output] [+ in-place ReLU] run as one launch
+        # uint8 residual blocks: Conv2D [+ Accum onto its output] [+ in-place ReLU] run as one launch;
+        # float32: Conv2D + activation followed by MaxPool2D 2x2 stride 2 (no padding) run as one launch
+        # when nothing else reads the convolution's output
         self.plan = []
         ops = model.ops
+        phys = {}                # buffer name in the model -> buffer that holds it in this plan
+        at = lambda o: replace(o, src=phys.get(o.src, o.src), dst=phys.get(o.dst, o.dst))
         i = 0
         while i < len(ops):
             op = ops[i]
             acc_op, relu, j = None, False, i + 1
+            if (fused and model.dtype == "f32" and op.kind == "conv" and j < len(ops) and ops[j].kind == "maxpool"
+                    and ops[j].src == op.dst and (ops[j].kh, ops[j].kw, ops[j].stride) == (2, 2, 2)
+                    and ops[j].pads == (0, 0, 0, 0) and (op.C % CB == 0 or (op.kh, op.kw) == (3, 3))
+                    and not self._read_before_rewritten(ops[j + 1:], op.dst, model.out)
+                    and self._pool_tiles_fill(op)):
+                # the fused launch cannot write the pooled map over the convolution's input (the model's
+                # ping-pong naming asks for that): it goes to the buffer the convolution's output had, and
+                # the two names trade buffers from here on
+                conv, pool = at(op), at(ops[j])
+                if pool.dst == conv.src:
+                    phys[ops[j].dst], phys[op.dst] = conv.dst, pool.dst
+                    pool = replace(pool, dst=conv.dst)
+                self.plan.append((conv, pool, False))
+                i = j + 1
+                continue
             if fused and model.dtype == "u8" and op.kind == "conv":
                 if j < len(ops) and ops[j].kind == "accum" and ops[j].dst == op.dst and ops[j].src != op.dst:
                     acc_op = ops[j]
@@ -379,9 +401,29 @@ class HipExecutor:
                 if j < len(ops) and ops[j].kind == "relu" and ops[j].src == op.dst and ops[j].dst == op.dst:
                     relu = True
                     j += 1
-            self.plan.append((op, acc_op, relu))
+            self.plan.append((at(op), at(acc_op) if acc_op else None, relu))
             i = j
+        self.out_name = phys.get(model.out, model.out)
         torch.cuda.synchronize()
+
+    @staticmethod
+    def _read_before_rewritten(later_ops, name, model_out):
+        """Is the tensor now in buffer `name` still needed by a later op (buffers are re-used by name)?"""
+        for o in later_ops:
+            if o.src == name or (o.kind == "accum" and o.dst == name):
+                return True
+            if o.dst == name:
+                return False
+        return model_out == name
+
+    @staticmethod
+    def _pool_tiles_fill(op):
+        """The fused convolution + pooling kernel works on 4 x 8 pixel tiles (16 x 16 for first layers) of one
+        image; on small maps the ragged tiles cost more than the saved pooling pass (measured: 26x26 loses, 52x52
+        wins), so fuse from 90% tile utilisation."""
+        th, tw = (4, 8) if op.C % CB == 0 else (16, 16)
+        ho, wo = op.Ho, op.Wo
+        return ho * wo >= 0.9 * (-(-ho // th) * th) * (-(-wo // tw) * tw)
 
     @staticmethod
     def _p(t):
@@ -394,7 +436,7 @@ class HipExecutor:
         op = self.model.ops[-1]
         c, h, w = op.out_shape()
         self.torch.cuda.synchronize()
-        return self.buf[self.model.out][: self.batch * c * h * w].cpu().numpy()
+        return self.buf[self.out_name][: self.batch * c * h * w].cpu().numpy()
 
     def run_fused_u8(self, op, acc_op, relu, st):
         """Conv2D + optional Accum + optional in-place ReLU in one launch (bit-identical to the sequence)."""
@@ -411,6 +453,25 @@ class HipExecutor:
             rc = L.small_hip_conv2d_accum_relu_u8(*args, p(b[op.src]), iq, p(self.w[op.weight]), fq,
                                                   acc_p, acc_q, int(relu), p(b[op.dst]), oq, st)
         capi.check(rc)
+
+    def run_entry(self, entry, st):
+        """One launch of the plan: a single op, or a fused group."""
+        op, acc_op, relu = entry
+        if acc_op is not None and acc_op.kind == "maxpool":
+            self.run_conv_pool_f32(op, acc_op, st)
+        elif acc_op is not None or relu:
+            self.run_fused_u8(op, acc_op, relu, st)
+        else:
+            self.run_op(op, st)
+
+    def run_conv_pool_f32(self, op, pool, st):
+        """Conv2D + activation + MaxPool2D 2x2 stride 2 in one launch."""
+        L, p, b = self.lib, self._p, self.buf
+        act = {None: capi.ACT_NONE, "relu": capi.ACT_RELU, "leaky": capi.ACT_LEAKY}[op.act]
+        t_, b_, l_, r_ = op.pads
+        capi.check(L.small_hip_conv2d_bias_act_maxpool2d_f32(
+            self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 2, 2, 2, 0, 0, 0, 0, op.Co, op.C, op.H, op.W,
+            p(b[op.src]), p(self.w[op.weight]), None, act, op.slope, p(b[pool.dst]), st))
 
     def run_op(self, op: Op, st):
         L, p, B, b = self.lib, self._p, self.batch, self.buf
@@ -480,11 +541,8 @@ class HipExecutor:
 
     def forward(self):
         st = self.stream()
-        for op, acc_op, relu in self.plan:
-            if acc_op is not None or relu:
-                self.run_fused_u8(op, acc_op, relu, st)
-            else:
-                self.run_op(op, st)
+        for entry in self.plan:
+            self.run_entry(entry, st)
 
     def capture(self):
         """Record one forward pass into a HIP graph (the launches go to the capture stream through the

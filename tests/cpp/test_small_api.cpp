@@ -353,6 +353,37 @@ static void test_quint8_and_batched()
     for (int i = 0; i < 32; ++i) CHECK(dy[i] == cy[i]);
 }
 
+static void test_fused_conv_pool_dropout_softmax()
+{
+    std::printf("fused convolution + pooling, dropout, softmax\n");
+    // Conv2D_Bias_ReLU_Maxpool2D == Conv2D_Bias_Act, then MaxPool2D: 2x2 stride 2 (one launch) and 3x3 stride 2
+    // (runs through the intermediate buffer)
+    const int Ci = 16, Co = 32, H = 12, W = 20;
+    FloatBuffer x(Ci * H * W), f(Co * Ci * 9), bias(Co), mid(Co * H * W), inter(Co * H * W);
+    small::init(x, x.size());
+    small::init(f, f.size());
+    small::init(bias, Co);
+    small::batched::Conv2D_Bias_Act(1, 3, 3, 1, 1, 1, 1, 1, Co, Ci, H, W, x, f, bias, small::RELU, 0.f, mid);
+    for (int pk = 2; pk <= 3; ++pk)
+    {
+        const int Hp = (H - pk) / 2 + 1, Wp = (W - pk) / 2 + 1;
+        FloatBuffer want(Co * Hp * Wp), got(Co * Hp * Wp);
+        small::MaxPool2D(pk, pk, 2, 0, 0, 0, 0, Co, H, W, mid, want);
+        small::Conv2D_Bias_ReLU_Maxpool2D(3, 3, 1, 1, 1, 1, 1, pk, pk, 2, 0, 0, 0, 0, Co, Ci, H, W, x, f, bias, inter, got);
+        for (size_t i = 0; i < want.size(); ++i) CHECK(almost_equal(got[i], want[i], 1e-4f));
+    }
+    // Dropout = multiplication by filter[0]; SoftMax sums to one over the whole tensor
+    FloatBuffer rate(1), d(Ci * H * W), sm(Ci * H * W);
+    rate[0] = 0.75f;
+    small::Dropout(Ci, H, W, x, rate, d);
+    for (size_t i = 0; i < d.size(); ++i) CHECK(d[i] == x[i] * 0.75f);
+    small::SoftMax(Ci, H, W, x, sm);
+    double total = 0;
+    for (size_t i = 0; i < sm.size(); ++i) total += sm[i];
+    CHECK(std::fabs(total - 1.0) < 1e-5);
+    CHECK(almost_equal(sm[5] / sm[6], std::exp(x[5] - x[6]), 1e-4f));
+}
+
 int main(int argc, char **argv)
 {
     const std::string dir = argc > 1 ? argv[1] : "tests/golden/ref_regression";
@@ -364,6 +395,7 @@ int main(int argc, char **argv)
     test_conv2d_fixtures(dir);
     test_window_fixtures(dir);
     test_quint8_and_batched();
+    test_fused_conv_pool_dropout_softmax();
     std::printf(g_fail ? "FAILED: %d checks\n" : "ALL PASSED\n", g_fail);
     return g_fail ? 1 : 0;
 }
