@@ -270,6 +270,29 @@ void DepthwiseConv2D_Bias_Act(int batch, int kernel_height, int kernel_width, in
         "DepthwiseConv2D_Bias_Act");
 }
 
+// Conv2D [+ bias] [+ act] followed by DepthwiseConv2D [+ bias] [+ act] (the reference's Conv2D_*_DepthwiseConv2D_*
+// family, fused_interface_abstract.hpp:1513-2500): two launches through inter_output_buf, which ends up holding
+// the whole first layer's output.  A one-launch form (depthwise inside the matrix kernel) was measured slower
+// than the two launches on this machine, so none is built.  Bias buffers may be empty.
+template <class BufferT, detail::if_float<BufferT> = true>
+void Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
+    int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad, uint8_t conv_b_pad,
+    uint8_t conv_l_pad, uint8_t conv_r_pad, int dw_kernel_height, int dw_kernel_width, int dw_stride,
+    uint8_t dw_t_pad, uint8_t dw_b_pad, uint8_t dw_l_pad, uint8_t dw_r_pad, int output_channels, int input_channels,
+    int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT const &bias_buf,
+    BufferT &inter_output_buf, BufferT const &dwise_filter_buf, BufferT const &dwise_bias_buf, ActivationType act,
+    float negative_slope, BufferT &output_buf)
+{
+    Conv2D_Bias_Act(batch, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
+                    conv_r_pad, output_channels, input_channels, input_height, input_width, input_buf, filter_buf,
+                    bias_buf, act, negative_slope, inter_output_buf);
+    const int Ho = (int)output_dim(input_height + conv_t_pad + conv_b_pad, conv_stride, conv_kernel_height);
+    const int Wo = (int)output_dim(input_width + conv_l_pad + conv_r_pad, conv_stride, conv_kernel_width);
+    DepthwiseConv2D_Bias_Act(batch, dw_kernel_height, dw_kernel_width, dw_stride, dw_t_pad, dw_b_pad, dw_l_pad,
+                             dw_r_pad, output_channels, Ho, Wo, inter_output_buf, dwise_filter_buf, dwise_bias_buf,
+                             act, negative_slope, output_buf);
+}
+
 // ---- pooling -----------------------------------------------------------------------------------------
 template <class BufferT, detail::if_float<BufferT> = true>
 void MaxPool2D(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
@@ -636,6 +659,98 @@ void Conv2D_Maxpool2D(int conv_kernel_height, int conv_kernel_width, int conv_st
                                        pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad, output_channels,
                                        input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
                                        NONE, 0.f, inter_output_buf, output_buf);
+}
+
+// The reference's single-layer "fused" functions (fused_interface_abstract.hpp:55, 217, 1332, 1419): one launch.
+template <class BufferT>
+void Conv2D_ReLU(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+                 uint8_t r_pad, int output_channels, int input_channels, int input_height, int input_width,
+                 BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, output_channels,
+                             input_channels, input_height, input_width, input_buf, filter_buf, BufferT(), RELU, 0.f,
+                             output_buf);
+}
+
+template <class BufferT>
+void Conv2D_Bias_ReLU(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad, uint8_t l_pad,
+                      uint8_t r_pad, int output_channels, int input_channels, int input_height, int input_width,
+                      BufferT const &input_buf, BufferT const &filter_buf, BufferT const &bias_buf,
+                      BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, output_channels,
+                             input_channels, input_height, input_width, input_buf, filter_buf, bias_buf, RELU, 0.f,
+                             output_buf);
+}
+
+template <class BufferT>
+void DepthwiseConv2D_ReLU(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                          uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                          BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::DepthwiseConv2D_Bias_Act(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad,
+                                      input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
+                                      RELU, 0.f, output_buf);
+}
+
+template <class BufferT>
+void DepthwiseConv2D_Bias_ReLU(int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
+                               uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                               BufferT const &input_buf, BufferT const &filter_buf, BufferT const &bias_buf,
+                               BufferT &output_buf)
+{
+    batched::DepthwiseConv2D_Bias_Act(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad,
+                                      input_channels, input_height, input_width, input_buf, filter_buf, bias_buf,
+                                      RELU, 0.f, output_buf);
+}
+
+// The reference's convolution + depthwise convolution functions (fused_interface_abstract.hpp:1513, 1840, 2170),
+// same signatures (the reference names the depthwise window "pool_*").
+template <class BufferT>
+void Conv2D_DepthwiseConv2D(int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad,
+                            uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad, int pool_kernel_height,
+                            int pool_kernel_width, int pool_stride, uint8_t pool_t_pad, uint8_t pool_b_pad,
+                            uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels, int input_channels,
+                            int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                            BufferT &inter_output_buf, BufferT const &dwise_filter_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
+        1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad, conv_r_pad,
+        pool_kernel_height, pool_kernel_width, pool_stride, pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad,
+        output_channels, input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
+        inter_output_buf, dwise_filter_buf, BufferT(), NONE, 0.f, output_buf);
+}
+
+template <class BufferT>
+void Conv2D_ReLU_DepthwiseConv2D_ReLU(int conv_kernel_height, int conv_kernel_width, int conv_stride,
+                                      uint8_t conv_t_pad, uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad,
+                                      int pool_kernel_height, int pool_kernel_width, int pool_stride,
+                                      uint8_t pool_t_pad, uint8_t pool_b_pad, uint8_t pool_l_pad, uint8_t pool_r_pad,
+                                      int output_channels, int input_channels, int input_height, int input_width,
+                                      BufferT const &input_buf, BufferT const &filter_buf, BufferT &inter_output_buf,
+                                      BufferT const &dwise_filter_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
+        1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad, conv_r_pad,
+        pool_kernel_height, pool_kernel_width, pool_stride, pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad,
+        output_channels, input_channels, input_height, input_width, input_buf, filter_buf, BufferT(),
+        inter_output_buf, dwise_filter_buf, BufferT(), RELU, 0.f, output_buf);
+}
+
+template <class BufferT>
+void Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU(
+    int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad, uint8_t conv_b_pad,
+    uint8_t conv_l_pad, uint8_t conv_r_pad, int pool_kernel_height, int pool_kernel_width, int pool_stride,
+    uint8_t pool_t_pad, uint8_t pool_b_pad, uint8_t pool_l_pad, uint8_t pool_r_pad, int output_channels,
+    int input_channels, int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+    BufferT const &bias_buf, BufferT &inter_output_buf, BufferT const &dwise_filter_buf,
+    BufferT const &dwise_bias_buf, BufferT &output_buf)
+{
+    batched::Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
+        1, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad, conv_r_pad,
+        pool_kernel_height, pool_kernel_width, pool_stride, pool_t_pad, pool_b_pad, pool_l_pad, pool_r_pad,
+        output_channels, input_channels, input_height, input_width, input_buf, filter_buf, bias_buf,
+        inter_output_buf, dwise_filter_buf, dwise_bias_buf, RELU, 0.f, output_buf);
 }
 
 // small::Dense exactly as the reference writes it (interface_abstract.hpp:2113-2132):

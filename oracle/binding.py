@@ -322,6 +322,10 @@ class RefLib:
             L.sref_upsample2d_f32.argtypes = [c_int] * 4 + [c_vp] * 2
             L.sref_concat_f32.argtypes = [C.c_uint32] * 4 + [c_vp] * 3
             L.sref_dense_f32.argtypes = [c_int] * 2 + [c_vp] * 3
+            if hasattr(L, "sref_fused_conv_pool_f32"):
+                L.sref_fused_conv_pool_f32.argtypes = [c_int] * 17 + [c_vp] * 5
+                L.sref_fused_conv_dw_f32.argtypes = [c_int] * 17 + [c_vp] * 7
+                L.sref_fused_single_f32.argtypes = [c_int] * 11 + [c_vp] * 4
         if has_q:
             L.sref_qbuf_new.restype = c_vp
             L.sref_qbuf_new.argtypes = [C.c_size_t]

@@ -13,6 +13,11 @@ Pinned (CPU suite) against the reference's own classes compiled into oracle/_ref
 The quantised variants have no counterpart that runs in the reference (its Layer classes call
 small::Bias / the float-only activations): they compose the quantised functions that are pinned one by
 one, and PartialConv2DLayer / AddLayer follow this build's own definition: parity unpinned.
+
+fused_two_layers_f32 / fused_single_f32 restate the reference's "fused" functions
+(include/small/fused_interface_abstract.hpp) as what they compute: the plain layer sequence.  Pinned
+against those functions in oracle/_ref (sref_fused_*; identical on the scalar build without bias,
+float32 tolerance with bias, where the reference adds the bias at another point of the summation).
 """
 import numpy as np
 
@@ -299,3 +304,49 @@ def resnet8_tiny_u8(oracle, q, x, iq, filters, fq, aq):
     assert rc == 0
     y = _unpack_images(oracle, y, n, c, 1, 1)
     return cl(0, y, aq, f[i], NONE, 1, 1, 0)
+
+
+# ---- the reference's two-layer functions (packed arrays, batch images back to back) -------------------------
+def fused_single_f32(oracle, batch, cb, depthwise, k, s, pads, Co, Ci, H, W, x, f, bias):
+    """Conv2D_ReLU / Conv2D_Bias_ReLU (fused_interface_abstract.hpp:55, 217) and DepthwiseConv2D_ReLU /
+    DepthwiseConv2D_Bias_ReLU (:1332, :1419): [bias +] convolution, ReLU.  bias None = the form without."""
+    if not depthwise:
+        rc, y = oracle.conv2d_bias_act_f32(batch, cb, k, k, s, *pads, Co, Ci, H, W, x, f, bias, RELU, 0.0)
+        assert rc == 0
+        return y
+    Ho, Wo = oracle.out_hw(k, k, s, *pads, H, W)
+    if bias is not None:
+        rc, y = oracle.bias_f32(batch, cb, Ci, Ho, Wo, bias)
+        assert rc == 0
+        rc, y = oracle.dwconv2d_f32(batch, cb, k, k, s, *pads, Ci, H, W, x, f, out=y, accumulate=1)
+    else:
+        rc, y = oracle.dwconv2d_f32(batch, cb, k, k, s, *pads, Ci, H, W, x, f)
+    assert rc == 0
+    return np.maximum(y, np.float32(0))
+
+
+def fused_two_layers_f32(oracle, batch, cb, second, variant, ck, cs, cpads, k2, s2, pads2, Co, Ci, H, W, x, f, bias=None,
+                         dwf=None, dwbias=None):
+    """second = "pool": Conv2D_Maxpool2D / Conv2D_ReLU_Maxpool2D / Conv2D_Bias_ReLU_Maxpool2D
+    (fused_interface_abstract.hpp:683, 998, 354); second = "dw": Conv2D_DepthwiseConv2D /
+    Conv2D_ReLU_DepthwiseConv2D_ReLU / Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU (:1513, 1840, 2170).
+    variant 0: neither bias nor ReLU, 1: ReLU after each convolution, 2: bias and ReLU.
+    -> (output of the second layer, output of the first)."""
+    act = NONE if variant == 0 else RELU
+    rc, mid = oracle.conv2d_bias_act_f32(batch, cb, ck, ck, cs, *cpads, Co, Ci, H, W, x, f,
+                                         bias if variant == 2 else None, act, 0.0)
+    assert rc == 0
+    Ho, Wo = oracle.out_hw(ck, ck, cs, *cpads, H, W)
+    if second == "pool":
+        rc, y = oracle.maxpool2d_f32(batch, cb, k2, k2, s2, *pads2, Co, Ho, Wo, mid)
+        assert rc == 0
+        return y, mid
+    H2, W2 = oracle.out_hw(k2, k2, s2, *pads2, Ho, Wo)
+    if variant == 2:
+        rc, y = oracle.bias_f32(batch, cb, Co, H2, W2, dwbias)
+        assert rc == 0
+        rc, y = oracle.dwconv2d_f32(batch, cb, k2, k2, s2, *pads2, Co, Ho, Wo, mid, dwf, out=y, accumulate=1)
+    else:
+        rc, y = oracle.dwconv2d_f32(batch, cb, k2, k2, s2, *pads2, Co, Ho, Wo, mid, dwf)
+    assert rc == 0
+    return (np.maximum(y, np.float32(0)) if act else y), mid

@@ -208,6 +208,60 @@ int sref_dense_f32(int No, int Ni, void *in, void *filt, void *out)
 {
     return guarded([&] { small::Dense(No, Ni, F(in), F(filt), F(out)); });
 }
+
+// ---- the reference's two-layer ("fused") functions, include/small/fused_interface_abstract.hpp ------------
+// variant 0: Conv2D_Maxpool2D, 1: Conv2D_ReLU_Maxpool2D, 2: Conv2D_Bias_ReLU_Maxpool2D
+int sref_fused_conv_pool_f32(int variant, int ck, int cs, int ct, int cb, int cl, int cr, int pk, int ps, int pt,
+                             int pb, int pl, int pr, int Co, int Ci, int H, int W, void *in, void *filt, void *bias,
+                             void *inter, void *out)
+{
+    return guarded([&] {
+        if (variant == 0)
+            small::Conv2D_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, pk, pk, ps, pt, pb, pl, pr, Co, Ci, H, W, F(in),
+                                    F(filt), F(inter), F(out));
+        else if (variant == 1)
+            small::Conv2D_ReLU_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, pk, pk, ps, pt, pb, pl, pr, Co, Ci, H, W, F(in),
+                                         F(filt), F(inter), F(out));
+        else
+            small::Conv2D_Bias_ReLU_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, pk, pk, ps, pt, pb, pl, pr, Co, Ci, H, W,
+                                              F(in), F(filt), F(bias), F(inter), F(out));
+    });
+}
+// variant 0: Conv2D_DepthwiseConv2D, 1: Conv2D_ReLU_DepthwiseConv2D_ReLU,
+//         2: Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU
+int sref_fused_conv_dw_f32(int variant, int ck, int cs, int ct, int cb, int cl, int cr, int dk, int ds, int dt,
+                           int db, int dl, int dr, int Co, int Ci, int H, int W, void *in, void *filt, void *bias,
+                           void *inter, void *dwfilt, void *dwbias, void *out)
+{
+    return guarded([&] {
+        if (variant == 0)
+            small::Conv2D_DepthwiseConv2D(ck, ck, cs, ct, cb, cl, cr, dk, dk, ds, dt, db, dl, dr, Co, Ci, H, W,
+                                          F(in), F(filt), F(inter), F(dwfilt), F(out));
+        else if (variant == 1)
+            small::Conv2D_ReLU_DepthwiseConv2D_ReLU(ck, ck, cs, ct, cb, cl, cr, dk, dk, ds, dt, db, dl, dr, Co, Ci,
+                                                    H, W, F(in), F(filt), F(inter), F(dwfilt), F(out));
+        else
+            small::Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU(ck, ck, cs, ct, cb, cl, cr, dk, dk, ds, dt, db, dl, dr,
+                                                              Co, Ci, H, W, F(in), F(filt), F(bias), F(inter),
+                                                              F(dwfilt), F(dwbias), F(out));
+    });
+}
+// variant 0: DepthwiseConv2D_ReLU, 1: DepthwiseConv2D_Bias_ReLU, 2: Conv2D_ReLU, 3: Conv2D_Bias_ReLU
+// (Co is ignored by the depthwise variants)
+int sref_fused_single_f32(int variant, int k, int s, int t, int b, int l, int r, int Co, int Ci, int H, int W,
+                          void *in, void *filt, void *bias, void *out)
+{
+    return guarded([&] {
+        if (variant == 0)
+            small::DepthwiseConv2D_ReLU(k, k, s, t, b, l, r, Ci, H, W, F(in), F(filt), F(out));
+        else if (variant == 1)
+            small::DepthwiseConv2D_Bias_ReLU(k, k, s, t, b, l, r, Ci, H, W, F(in), F(filt), F(bias), F(out));
+        else if (variant == 2)
+            small::Conv2D_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, F(in), F(filt), F(out));
+        else
+            small::Conv2D_Bias_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, F(in), F(filt), F(bias), F(out));
+    });
+}
 #endif // float
 
 #if defined(SMALL_HAS_QUINT8_SUPPORT)

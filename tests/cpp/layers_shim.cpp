@@ -311,4 +311,54 @@ int stest_resnet8_u8(int batch, const uint8_t *const *filters, const size_t *siz
     });
 }
 
+// The reference-named two-layer functions of small/interface.hpp on PACKED batch-1 arrays.
+// second 0: Conv2D_*_Maxpool2D, 1: Conv2D_*_DepthwiseConv2D_*; variant 0 plain, 1 ReLU, 2 bias + ReLU.
+// inter / out: packed first-layer and second-layer outputs (inter is only defined where the library says so).
+int stest_fused_two_layers_f32(int second, int variant, int ck, int cs, int ct, int cb, int cl, int cr, int k2, int s2,
+                               int t2, int b2, int l2, int r2, int Co, int Ci, int H, int W, const float *in,
+                               size_t n_in, const float *filt, size_t n_filt, const float *bias, const float *dwfilt,
+                               size_t n_dwfilt, const float *dwbias, float *out, size_t n_out, size_t n_inter)
+{
+    using FB = small::FloatBuffer;
+    return guarded([&] {
+        FB x = from_host<FB>(in, n_in), f = from_host<FB>(filt, n_filt), b = from_host<FB>(bias, Co);
+        FB df = from_host<FB>(dwfilt, n_dwfilt), db = from_host<FB>(dwbias, Co), inter(n_inter), o(n_out);
+        if (second == 0 && variant == 0)
+            small::Conv2D_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co, Ci, H, W, x, f, inter, o);
+        else if (second == 0 && variant == 1)
+            small::Conv2D_ReLU_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co, Ci, H, W, x, f,
+                                         inter, o);
+        else if (second == 0)
+            small::Conv2D_Bias_ReLU_Maxpool2D(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co, Ci, H, W, x, f,
+                                              b, inter, o);
+        else if (variant == 0)
+            small::Conv2D_DepthwiseConv2D(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co, Ci, H, W, x, f,
+                                          inter, df, o);
+        else if (variant == 1)
+            small::Conv2D_ReLU_DepthwiseConv2D_ReLU(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co, Ci, H, W,
+                                                    x, f, inter, df, o);
+        else
+            small::Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co,
+                                                              Ci, H, W, x, f, b, inter, df, db, o);
+        std::memcpy(out, o.data(), n_out * sizeof(float));
+    });
+}
+
+// variant 0: DepthwiseConv2D_ReLU, 1: DepthwiseConv2D_Bias_ReLU, 2: Conv2D_ReLU, 3: Conv2D_Bias_ReLU (packed arrays)
+int stest_fused_single_f32(int variant, int k, int s, int t, int b, int l, int r, int Co, int Ci, int H, int W,
+                           const float *in, size_t n_in, const float *filt, size_t n_filt, const float *bias,
+                           float *out, size_t n_out)
+{
+    using FB = small::FloatBuffer;
+    return guarded([&] {
+        FB x = from_host<FB>(in, n_in), f = from_host<FB>(filt, n_filt), bb = from_host<FB>(bias, variant < 2 ? Ci : Co);
+        FB o(n_out);
+        if (variant == 0) small::DepthwiseConv2D_ReLU(k, k, s, t, b, l, r, Ci, H, W, x, f, o);
+        else if (variant == 1) small::DepthwiseConv2D_Bias_ReLU(k, k, s, t, b, l, r, Ci, H, W, x, f, bb, o);
+        else if (variant == 2) small::Conv2D_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, x, f, o);
+        else small::Conv2D_Bias_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, x, f, bb, o);
+        std::memcpy(out, o.data(), n_out * sizeof(float));
+    });
+}
+
 } // extern "C"

@@ -124,6 +124,26 @@ class HipLayers(_Shim):
         self._check(rc)
         return ms.value
 
+    def fused_two_layers_f32(self, second, variant, ck, cs, cp, k2, s2, p2, Co, Ci, H, W, x, f, bias, dwf, dwbias, n_out,
+                             n_inter):
+        """The reference-named Conv2D_*_Maxpool2D (second "pool") / Conv2D_*_DepthwiseConv2D_* ("dw") functions of
+        small/interface.hpp on packed batch-1 arrays -> packed output."""
+        out = np.zeros(n_out, np.float32)
+        ints = [0 if second == "pool" else 1, variant, ck, cs, *cp, k2, s2, *p2, Co, Ci, H, W]
+        rc = self.lib.stest_fused_two_layers_f32(*[C.c_int(v) for v in ints], _f32p(x), C.c_size_t(x.size), _f32p(f),
+                                                 C.c_size_t(f.size), _f32p(bias), _f32p(dwf), C.c_size_t(dwf.size),
+                                                 _f32p(dwbias), _f32p(out), C.c_size_t(n_out), C.c_size_t(n_inter))
+        self._check(rc)
+        return out
+
+    def fused_single_f32(self, variant, k, s, p, Co, Ci, H, W, x, f, bias, n_out):
+        out = np.zeros(n_out, np.float32)
+        ints = [variant, k, s, *p, Co, Ci, H, W]
+        rc = self.lib.stest_fused_single_f32(*[C.c_int(v) for v in ints], _f32p(x), C.c_size_t(x.size), _f32p(f),
+                                             C.c_size_t(f.size), _f32p(bias), _f32p(out), C.c_size_t(n_out))
+        self._check(rc)
+        return out
+
     def conv_layer_u8(self, kind, x, iq, filters, fq, oq, act, kh, kw, stride, padding, out_init=None):
         n, c, h, w = x.shape
         co = filters.shape[0]

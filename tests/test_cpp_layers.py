@@ -114,6 +114,42 @@ def test_models(hip, oracle, name):
     assert_close_f32(one[0], got[1], atol=1e-5 * scale, what=name + " batch-1 vs batched")
 
 
+# ---- the reference-named two-layer ("fused") functions ---------------------------------------------------
+from test_oracle_fused_vs_ref import SINGLE_CASES, TWO_LAYER_CASES, two_layer_inputs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", [0, 1, 2], ids=["plain", "relu", "bias_relu"])
+@pytest.mark.parametrize("second", ["pool", "dw"])
+@pytest.mark.parametrize("case", TWO_LAYER_CASES, ids=str)
+def test_two_layer_functions(hip, oracle, case, second, variant):
+    ck, cs, cp, k2, s2, p2, Co, Ci, H, W = case
+    x, f, bias, dwf, dwbias = two_layer_inputs(case, 16, oracle)
+    want, mid = ol.fused_two_layers_f32(oracle, 1, 16, second, variant, ck, cs, cp, k2, s2, p2, Co, Ci, H, W, x, f, bias,
+                                        dwf, dwbias)
+    got = hip.fused_two_layers_f32(second, variant, ck, cs, cp, k2, s2, p2, Co, Ci, H, W, x, f, bias, dwf, dwbias,
+                                   want.size, mid.size)
+    assert_close_f32(got, want, what="%s %s %d" % (case, second, variant))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", [0, 1, 2, 3], ids=["dw_relu", "dw_bias_relu", "conv_relu", "conv_bias_relu"])
+@pytest.mark.parametrize("case", SINGLE_CASES, ids=str)
+def test_single_layer_fused_functions(hip, oracle, case, variant):
+    k, s, p, Co, Ci, H, W = case
+    dw = variant < 2
+    if dw and Ci % 16:
+        pytest.skip("depthwise needs whole channel blocks")
+    Cout = Ci if dw else Co
+    x = oracle.pack(synth.normal(1, Ci * H * W), 0, 1, Ci, H, W, 16, 16)
+    f = (oracle.pack(synth.he_normal(5, Ci * k * k, k * k), 2, Ci, 1, k, k, 16, 16) if dw else
+         oracle.pack(synth.he_normal(2, Co * Ci * k * k, Ci * k * k), 3, Co, Ci, k, k, 16, 16))
+    bias = synth.normal(4, Cout)
+    want = ol.fused_single_f32(oracle, 1, 16, dw, k, s, p, Co, Ci, H, W, x, f, bias if variant in (1, 3) else None)
+    got = hip.fused_single_f32(variant, k, s, p, Co, Ci, H, W, x, f, bias, want.size)
+    assert_close_f32(got, want, what="%s %d" % (case, variant))
+
+
 # ---- quantised layers -------------------------------------------------------------------------------------
 DEFAULT_Q = (128, 1077952576, 0, 6)       # the fields of a fresh QUInt8Buffer
 QMAX = (1 << 31) - 1                      # multiplier ~ 1.0: ReLU and Accum requantise with the output's scale again
