@@ -14,3 +14,4 @@
 #include "small/utils.hpp"
 #include "small/buffers.hpp"
 #include "small/interface.hpp"
+#include "small/interface_1D.hpp"

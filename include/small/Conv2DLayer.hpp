@@ -56,6 +56,7 @@ struct BatchNormRefs
 //     scale = gamma / sqrt(var + eps);  filter[co] *= scale;
 //     bias[co] = beta - mean * scale               (no bias given)
 //              = beta + scale * (bias[co] - mean)  (bias given)
+// (conv1d_folding: scale = gamma / sqrt(var + eps), bias = scale * bias + beta - mean * scale, as Conv1DLayer.hpp does)
 // the reference's initialize_conv2d_buffers (Conv2DLayer.hpp:135-341) with the same float expressions.
 // `who` is the message prefix ("*Conv2DLayer" there).  Depthwise filters: num_input_channels = 1 and
 // depthwise = true (tensor type FILTER_DW).
@@ -64,7 +65,7 @@ void build_conv_weights(std::string const &who, bool depthwise, uint32_t num_out
                         uint32_t num_effective_output_channels, uint32_t num_input_channels, uint32_t kernel_height,
                         uint32_t kernel_width, BufferT const &filters, BufferT const &bias,
                         BatchNormRefs<BufferT> const &bn, bool buffers_are_packed, BufferT &packed_filters,
-                        BufferT &packed_bias)
+                        BufferT &packed_bias, bool conv1d_folding = false)
 {
     typedef typename BufferT::value_type T;
     const size_t taps = (size_t)num_input_channels * kernel_height * kernel_width;
@@ -118,10 +119,20 @@ void build_conv_weights(std::string const &who, bool depthwise, uint32_t num_out
     T *pb = packed_bias.data();
     for (size_t co = 0; co < num_effective_output_channels; ++co)
     {
-        const float rsq = 1.0f / std::sqrt(bn.variance[co] + bn.eps);
-        const float filter_scale = bn.weight[co] * rsq;
-        if (no_bias) pb[co] = bn.bias[co] - bn.mean[co] * filter_scale;
-        else pb[co] = bn.bias[co] + filter_scale * (pb[co] - bn.mean[co]);
+        float filter_scale;
+        if (conv1d_folding)     // Conv1DLayer.hpp:262-277 divides and sums in another order
+        {
+            filter_scale = bn.weight[co] / std::sqrt(bn.variance[co] + bn.eps);
+            if (no_bias) pb[co] = bn.bias[co] - bn.mean[co] * filter_scale;
+            else pb[co] = filter_scale * pb[co] + bn.bias[co] - bn.mean[co] * filter_scale;
+        }
+        else
+        {
+            const float rsq = 1.0f / std::sqrt(bn.variance[co] + bn.eps);
+            filter_scale = bn.weight[co] * rsq;
+            if (no_bias) pb[co] = bn.bias[co] - bn.mean[co] * filter_scale;
+            else pb[co] = bn.bias[co] + filter_scale * (pb[co] - bn.mean[co]);
+        }
         for (size_t ci = 0; ci < num_input_channels; ++ci)
             for (size_t fh = 0; fh < kernel_height; ++fh)
                 for (size_t fw = 0; fw < kernel_width; ++fw)

@@ -61,6 +61,13 @@ inline void raise(int status, const char *op)
     }
 }
 
+// "Conv2D<float> ERROR: ..." -> "Conv1D<float> ERROR: ..." for the 1-D functions built on the 2-D ones
+inline std::string rename_op(std::string msg, std::string const &from, std::string const &to)
+{
+    if (msg.compare(0, from.size(), from) == 0) msg.replace(0, from.size(), to);
+    return msg;
+}
+
 template <class BufferT>
 using if_float = std::enable_if_t<std::is_same<FloatBuffer, BufferT>::value, bool>;
 template <class BufferT>

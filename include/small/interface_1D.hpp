@@ -1,0 +1,192 @@
+// The 1-D layer functions of the reference (include/small/interface_abstract_1D.hpp:47-1700 and the single-launch
+// members of fused_interface_abstract_1D.hpp), same names and argument order.
+//
+// A 1-D tensor is the packed 2-D tensor [C/16][rows][W][16] whose rows are independent signals: the
+// reference's `batch_size` argument is that row count (its Conv1DLayer passes shape[HEIGHT],
+// Conv1DLayer.hpp:671-690).  Every function here is therefore the 2-D kernel with a 1 x kernel_width window
+// and no vertical padding.  The 2-D kernels stride both axes alike, so more than one row is accepted with
+// stride 1 only (any stride when rows == 1); other combinations raise std::invalid_argument.
+// small::batched::<Fn>(batch, ...) takes `batch` such tensors back to back.
+#pragma once
+
+#include "interface.hpp"
+
+namespace small
+{
+namespace detail
+{
+template <class BufferT>
+inline void check_rows(const char *op, int stride, int rows)
+{
+    if (rows > 1 && stride != 1)
+        throw std::invalid_argument(std::string(op) + "<" + type_tag<BufferT>::name() +
+                                    "> ERROR: more than one row needs stride 1 on this platform.");
+}
+} // namespace detail
+
+namespace batched
+{
+// interface_abstract_1D.hpp:47 (float), :229 (quint8)
+template <class BufferT>
+void Conv1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels,
+            int input_channels, int batch_size, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+            BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("Conv1D", stride, batch_size);
+    try
+    {
+        Conv2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
+               input_width, input_buf, filter_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e) { throw std::invalid_argument(detail::rename_op(e.what(), "Conv2D", "Conv1D")); }
+}
+
+// interface_abstract_1D.hpp:415
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialConv1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels,
+                   int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                   BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("PartialConv1D", stride, batch_size);
+    try
+    {
+        PartialConv2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
+                      input_width, input_buf, filter_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e)
+    {
+        throw std::invalid_argument(detail::rename_op(e.what(), "PartialConv2D", "PartialConv1D"));
+    }
+}
+
+// bias + convolution + activation in one launch (Conv1D_ReLU / Conv1D_Bias_ReLU, fused_interface_abstract_1D.hpp:55, 216,
+// and what Conv1DLayer::compute_output issues as three calls); bias_buf may be empty
+template <class BufferT, detail::if_float<BufferT> = true>
+void Conv1D_Bias_Act(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels,
+                     int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                     BufferT const &filter_buf, BufferT const &bias_buf, ActivationType act, float negative_slope,
+                     BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("Conv1D", stride, batch_size);
+    Conv2D_Bias_Act(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
+                    input_width, input_buf, filter_buf, bias_buf, act, negative_slope, output_buf);
+}
+
+// interface_abstract_1D.hpp:776 (float), :840 (quint8)
+template <class BufferT>
+void MaxPool1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels,
+               int batch_size, int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("MaxPool1D", stride, batch_size);
+    try
+    {
+        MaxPool2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, input_channels, batch_size, input_width,
+                  input_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e) { throw std::invalid_argument(detail::rename_op(e.what(), "MaxPool2D", "MaxPool1D")); }
+}
+
+// interface_abstract_1D.hpp:906
+template <class BufferT, detail::if_float<BufferT> = true>
+void AveragePool1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels,
+                   int batch_size, int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("AveragePool1D", stride, batch_size);
+    try
+    {
+        AveragePool2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, input_channels, batch_size, input_width,
+                      input_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e)
+    {
+        throw std::invalid_argument(detail::rename_op(e.what(), "AveragePool2D", "AveragePool1D"));
+    }
+}
+
+// interface_abstract_1D.hpp:1526 (float), :1562 (quint8)
+template <class BufferT>
+void ReLUActivation1D(int batch, int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                      BufferT &output_buf)
+{
+    ReLUActivation(batch, input_channels, batch_size, input_width, input_buf, output_buf);
+}
+
+// interface_abstract_1D.hpp:1614: nearest neighbour along the width
+template <class BufferT, detail::if_float<BufferT> = true>
+void UpSample1D(int batch, int scale_factor, int input_channels, int batch_size, int input_width,
+                BufferT const &input_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_upsample1d_f32(batch, scale_factor, input_channels, batch_size, input_width,
+                                                    input_buf.device_in(), output_buf.device_out(), detail::st()),
+                           "Upsample");
+}
+} // namespace batched
+
+// ---- the reference's signatures ---------------------------------------------------------------------------------
+template <class BufferT>
+void Conv1D(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels,
+            int batch_size, int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::Conv1D(1, kernel_width, stride, l_pad, r_pad, output_channels, input_channels, batch_size, input_width,
+                    input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialConv1D(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels,
+                   int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                   BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::PartialConv1D(1, kernel_width, stride, l_pad, r_pad, output_channels, input_channels, batch_size,
+                           input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void MaxPool1D(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels, int batch_size,
+               int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::MaxPool1D(1, kernel_width, stride, l_pad, r_pad, input_channels, batch_size, input_width, input_buf,
+                       output_buf);
+}
+
+template <class BufferT>
+void AveragePool1D(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels, int batch_size,
+                   int input_width, BufferT const &input_buf, BufferT &output_buf)
+{
+    batched::AveragePool1D(1, kernel_width, stride, l_pad, r_pad, input_channels, batch_size, input_width, input_buf,
+                           output_buf);
+}
+
+template <class BufferT>
+void ReLUActivation1D(int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                      BufferT &output_buf)
+{
+    batched::ReLUActivation1D(1, input_channels, batch_size, input_width, input_buf, output_buf);
+}
+
+template <class BufferT>
+void UpSample1D(int scale_factor, int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                BufferT &output_buf)
+{
+    batched::UpSample1D(1, scale_factor, input_channels, batch_size, input_width, input_buf, output_buf);
+}
+
+// fused_interface_abstract_1D.hpp:55, 216: one launch
+template <class BufferT>
+void Conv1D_ReLU(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels, int input_channels,
+                 int batch_size, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                 BufferT &output_buf)
+{
+    batched::Conv1D_Bias_Act(1, kernel_width, stride, l_pad, r_pad, output_channels, input_channels, batch_size,
+                             input_width, input_buf, filter_buf, BufferT(), RELU, 0.f, output_buf);
+}
+
+template <class BufferT>
+void Conv1D_Bias_ReLU(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int output_channels,
+                      int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                      BufferT const &filter_buf, BufferT const &bias_buf, BufferT &output_buf)
+{
+    batched::Conv1D_Bias_Act(1, kernel_width, stride, l_pad, r_pad, output_channels, input_channels, batch_size,
+                             input_width, input_buf, filter_buf, bias_buf, RELU, 0.f, output_buf);
+}
+
+} // namespace small

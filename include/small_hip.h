@@ -190,6 +190,11 @@ int small_hip_partial_bias_f32(int batch, int num_channels, int output_height, i
 int small_hip_upsample2d_f32(int batch, int scale_factor, int input_channels, int input_height,
                              int input_width, const float *input, float *output,
                              small_hip_stream_t stream);
+
+/* small::UpSample1D<FloatBuffer>      interface_abstract_1D.hpp:1614-1660: nearest neighbour x2 along the width only;
+ * `rows` is the reference's batch_size argument (independent rows of a [C/16][rows][W][16] tensor). */
+int small_hip_upsample1d_f32(int batch, int scale_factor, int input_channels, int rows, int input_width,
+                             const float *in, float *out, small_hip_stream_t stream);
 /* small::Concat<BufferT>              interface.hpp:475-481, interface_abstract.hpp:2072-2105
  * (element_size = 4 for FloatBuffer, 1 for QUInt8Buffer) */
 int small_hip_concat(int batch, uint32_t input0_channels, uint32_t input1_channels,

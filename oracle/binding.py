@@ -69,6 +69,7 @@ class Oracle:
         L.so_accum_f32.argtypes = [c_int] * 5 + [c_vp, c_vp]
         L.so_bias_f32.argtypes = [c_int] * 5 + [c_vp, c_vp, c_int]
         L.so_upsample2d_f32.argtypes = [c_int] * 6 + [c_vp, c_vp]
+        L.so_upsample1d_f32.argtypes = [c_int] * 6 + [c_vp, c_vp]
         L.so_concat.argtypes = [c_int] + [C.c_uint32] * 4 + [c_vp, c_vp, c_vp, C.c_size_t]
         L.so_dense_f32.argtypes = [c_int] * 4 + [c_vp, c_vp, c_vp]
         L.so_dense_literal_f32.argtypes = [c_int] * 3 + [c_vp, c_vp, c_vp]
@@ -177,6 +178,10 @@ class Oracle:
     def upsample2d_f32(self, batch, cb, scale, Cn, H, W, x):
         out = np.zeros(batch * Cn * H * W * max(scale, 1) ** 2, np.float32)
         return self.lib.so_upsample2d_f32(batch, cb, scale, Cn, H, W, _p(x), _p(out)), out
+
+    def upsample1d_f32(self, batch, cb, scale, Cn, rows, W, x):
+        out = np.zeros(batch * Cn * rows * W * (scale if scale in (1, 2) else 1), np.float32)
+        return self.lib.so_upsample1d_f32(batch, cb, scale, Cn, rows, W, _p(x), _p(out)), out
 
     def concat(self, batch, C0, C1, H, W, a, b):
         out = np.empty(a.size + b.size, a.dtype)
@@ -322,6 +327,8 @@ class RefLib:
             L.sref_upsample2d_f32.argtypes = [c_int] * 4 + [c_vp] * 2
             L.sref_concat_f32.argtypes = [C.c_uint32] * 4 + [c_vp] * 3
             L.sref_dense_f32.argtypes = [c_int] * 2 + [c_vp] * 3
+            if hasattr(L, "sref_1d_f32"):
+                L.sref_1d_f32.argtypes = [c_int] * 9 + [c_vp] * 3
             if hasattr(L, "sref_fused_conv_pool_f32"):
                 L.sref_fused_conv_pool_f32.argtypes = [c_int] * 17 + [c_vp] * 5
                 L.sref_fused_conv_dw_f32.argtypes = [c_int] * 17 + [c_vp] * 7

@@ -44,20 +44,25 @@ def pad_up(c, cb=None):
     return (c + cb - 1) // cb * cb
 
 
-def fold_weights(filters, bias, bn, eps, co_padded):
+def fold_weights(filters, bias, bn, eps, co_padded, conv1d=False):
     """filters [Co, ...] float32, bias [Co] or None, bn [4, Co] (gamma, beta, mean, variance) or None
-    -> (filters [co_padded, ...], bias [co_padded] or None), float32 arithmetic in the reference's order."""
+    -> (filters [co_padded, ...], bias [co_padded] or None), float32 arithmetic in the reference's order
+    (conv1d: the expressions of Conv1DLayer.hpp:262-277, which divide where Conv2DLayer multiplies by 1/sqrt)."""
     f = np.array(filters, np.float32)
     co = f.shape[0]
     b = None if bias is None else np.array(bias, np.float32)
     if bn is not None:
         gamma, beta, mean, var = (np.asarray(a, np.float32) for a in bn)
-        rsq = np.float32(1.0) / np.sqrt(var + np.float32(eps), dtype=np.float32)
-        scale = (gamma * rsq).astype(np.float32)
-        if b is None:
-            b = (beta - mean * scale).astype(np.float32)
+        if conv1d:
+            scale = (gamma / np.sqrt(var + np.float32(eps), dtype=np.float32)).astype(np.float32)
+            b = (beta - mean * scale if b is None else scale * b + beta - mean * scale).astype(np.float32)
         else:
-            b = (beta + scale * (b - mean)).astype(np.float32)
+            rsq = np.float32(1.0) / np.sqrt(var + np.float32(eps), dtype=np.float32)
+            scale = (gamma * rsq).astype(np.float32)
+            if b is None:
+                b = (beta - mean * scale).astype(np.float32)
+            else:
+                b = (beta + scale * (b - mean)).astype(np.float32)
         f = (f * scale.reshape((-1,) + (1,) * (f.ndim - 1))).astype(np.float32)
     if co_padded != co:
         f = np.concatenate([f, np.zeros((co_padded - co,) + f.shape[1:], np.float32)], 0)
@@ -78,8 +83,25 @@ def _unpack_images(oracle, p, n, c, h, w):
 
 
 def conv_layer_f32(oracle, kind, x, filters, bias, bn, eps, act, slope, kh, kw, stride, padding, out_init=None):
-    """kind 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer on x [N, C, H, W];
-    filters [Co, Ci, kh, kw] (depthwise [C, kh, kw]).  -> [N, Co_padded, Ho, Wo]."""
+    """kind 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer, 3 Conv1DLayer (kh unused) on x [N, C, H, W];
+    filters [Co, Ci, kh, kw] (depthwise [C, kh, kw], 1-D [Co, Ci, kw]).  -> [N, Co_padded, Ho, Wo]."""
+    if kind == 3:
+        # Conv1DLayer (Conv1DLayer.hpp:647-724): the rows (HEIGHT) are independent signals, the window and the
+        # padding run along the width only.  Restated as Conv2DLayer with a 1 x kw window on every row taken as
+        # an image of its own, which also covers stride 2 on several rows.
+        n, c, h, w = x.shape
+        rows = np.ascontiguousarray(x.transpose(0, 2, 1, 3).reshape(n * h, c, 1, w))
+        f4, b1 = fold_weights(np.asarray(filters, np.float32).reshape(filters.shape[0], c, 1, kw), bias, bn, eps,
+                              filters.shape[0], conv1d=True)
+        y = conv_layer_f32(oracle, 0, rows, f4, b1, None, eps, NONE if act == SOFTMAX else act, slope, 1, kw, stride,
+                           padding)
+        y = np.ascontiguousarray(y.reshape(n, h, y.shape[1], y.shape[3]).transpose(0, 2, 1, 3))
+        if act == SOFTMAX:
+            yp = _pack_images(oracle, y, OUTPUT)
+            rc, yp = oracle.softmax_f32(n, CB, y.shape[1], h, y.shape[3], yp)
+            assert rc == 0
+            y = _unpack_images(oracle, yp, n, y.shape[1], h, y.shape[3])
+        return y
     n, c, h, w = x.shape
     co = filters.shape[0]
     cop = pad_up(co)
@@ -350,3 +372,37 @@ def fused_two_layers_f32(oracle, batch, cb, second, variant, ck, cs, cpads, k2, 
         rc, y = oracle.dwconv2d_f32(batch, cb, k2, k2, s2, *pads2, Co, Ho, Wo, mid, dwf)
     assert rc == 0
     return (np.maximum(y, np.float32(0)) if act else y), mid
+
+
+# ---- 1-D functions (packed arrays [C/cb][rows][W][cb]; rows = the reference's batch_size argument) --------------
+def one_d_f32(oracle, kind, cb, k, s, l, r, Co, Ci, rows, W, x, f=None, out_init=None):
+    """interface_abstract_1D.hpp: kind 0 Conv1D (:47), 1 PartialConv1D (:415), 2 MaxPool1D (:776), 3 AveragePool1D
+    (:906), 4 ReLUActivation1D (:1526), 5 UpSample1D (:1614, k = scale).  Every row is an independent signal: the 2-D
+    function with a 1 x k window on that row alone."""
+    if kind == 5:
+        rc, y = oracle.upsample1d_f32(1, cb, k, Ci, rows, W, x)
+        assert rc == 0
+        return y
+    if kind == 4:
+        rc, y = oracle.relu_f32(1, cb, Ci, rows, W, x)
+        assert rc == 0
+        return y
+    Wo = 1 + (W + l + r - k) // s
+    Cout = Co if kind < 2 else Ci
+    xin = np.asarray(x, np.float32).reshape(-1, rows, W * cb) if Ci >= cb else None
+    y = np.zeros((Cout // cb, rows, Wo * cb), np.float32)
+    init = None if out_init is None else np.asarray(out_init, np.float32).reshape(Cout // cb, rows, Wo * cb)
+    for row in range(rows):
+        # a first layer (Ci < cb) is stored [rows][W][Ci]
+        xr = (np.ascontiguousarray(xin[:, row]).ravel() if xin is not None else
+              np.ascontiguousarray(np.asarray(x, np.float32).reshape(rows, W * Ci)[row]))
+        if kind in (0, 1):
+            o0 = None if kind == 0 else np.ascontiguousarray(init[:, row]).ravel()
+            rc, yr = oracle.conv2d_f32(1, cb, 1, k, s, 0, 0, l, r, Co, Ci, 1, W, xr, f, out=o0, accumulate=kind)
+        elif kind == 2:
+            rc, yr = oracle.maxpool2d_f32(1, cb, 1, k, s, 0, 0, l, r, Ci, 1, W, xr)
+        else:
+            rc, yr = oracle.avgpool2d_f32(1, cb, 1, k, s, 0, 0, l, r, Ci, 1, W, xr)
+        assert rc == 0
+        y[:, row] = yr.reshape(Cout // cb, Wo * cb)
+    return y.ravel()

@@ -25,6 +25,7 @@
 #include <omp.h>
 
 #include <small.h>
+#include <small/Conv1DLayer.hpp>
 #include <small/Conv2DLayer.hpp>
 #include <small/PartialConv2DLayer.hpp>
 #include <small/DepthwiseConv2DLayer.hpp>
@@ -209,6 +210,23 @@ int sref_dense_f32(int No, int Ni, void *in, void *filt, void *out)
     return guarded([&] { small::Dense(No, Ni, F(in), F(filt), F(out)); });
 }
 
+// ---- 1-D functions, include/small/interface_abstract_1D.hpp (rows = their batch_size argument) -----------------
+// kind 0 Conv1D, 1 PartialConv1D, 2 MaxPool1D, 3 AveragePool1D, 4 ReLUActivation1D, 5 UpSample1D (k = scale)
+int sref_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows, int W, void *in, void *filt, void *out)
+{
+    return guarded([&] {
+        switch (kind)
+        {
+        case 0: small::Conv1D(k, s, l, r, Co, Ci, rows, W, F(in), F(filt), F(out)); break;
+        case 1: small::PartialConv1D(k, s, l, r, Co, Ci, rows, W, F(in), F(filt), F(out)); break;
+        case 2: small::MaxPool1D(k, s, l, r, Ci, rows, W, F(in), F(out)); break;
+        case 3: small::AveragePool1D(k, s, l, r, Ci, rows, W, F(in), F(out)); break;
+        case 4: small::ReLUActivation1D(Ci, rows, W, F(in), F(out)); break;
+        default: small::UpSample1D(k, Ci, rows, W, F(in), F(out)); break;
+        }
+    });
+}
+
 // ---- the reference's two-layer ("fused") functions, include/small/fused_interface_abstract.hpp ------------
 // variant 0: Conv2D_Maxpool2D, 1: Conv2D_ReLU_Maxpool2D, 2: Conv2D_Bias_ReLU_Maxpool2D
 int sref_fused_conv_pool_f32(int variant, int ck, int cs, int ct, int cb, int cl, int cr, int pk, int ps, int pt,
@@ -346,7 +364,7 @@ void unpack_tensor(small::Tensor<FB> const &t, float *flat, int *out_shape)
 } // namespace
 extern "C" {
 
-// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer; batch 1 (the reference computes one
+// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer, 3 Conv1DLayer; batch 1 (the reference computes one
 // image).  filters [Co][Ci][kh][kw] (depthwise [C][kh][kw]); bias Co or NULL; bn 4 x Co (gamma, beta, mean,
 // variance) or NULL; out is in/out, flat [Co_padded][Ho][Wo].
 int sref_conv_layer_f32(int kind, int C, int H, int W, int kh, int kw, int stride, int padding, int Co,
@@ -363,7 +381,13 @@ int sref_conv_layer_f32(int kind, int C, int H, int W, int kh, int kw, int strid
         const auto pad = padding ? small::PADDING_F : small::PADDING_V;
         const auto a = (small::ActivationType)act;
         std::unique_ptr<small::Layer<FB>> layer;
-        if (kind == 2)
+        if (kind == 3)      // Conv1DLayer: kh is ignored; it has no constructor taking bias and batch normalisation
+        {
+            if (bn) layer.reset(new small::Conv1DLayer<FB>(is, kw, stride, pad, Co, f, g, be, mu, var, eps, false, a, slope));
+            else if (bias) layer.reset(new small::Conv1DLayer<FB>(is, kw, stride, pad, Co, f, b, false, a, slope));
+            else layer.reset(new small::Conv1DLayer<FB>(is, kw, stride, pad, Co, f, false, a, slope));
+        }
+        else if (kind == 2)
         {
             if (bn) layer.reset(new small::DepthwiseConv2DLayer<FB>(is, kh, kw, stride, pad, f, b, g, be, mu, var, eps, false, a, slope));
             else if (bias) layer.reset(new small::DepthwiseConv2DLayer<FB>(is, kh, kw, stride, pad, f, b, false, a, slope));

@@ -22,7 +22,7 @@
  *        not usable there (abstract_layer.hpp:1269-1349), so this is the textbook result
  *   so_maxpool2d_f32 (incl. "padding counts as 0" quirk), so_avgpool2d_f32 (count_include_pad)
  *        reference fixtures, REF/ZEN2 builds with negative inputs on padded borders
- *   so_relu_f32, so_leaky_relu_f32, so_accum_f32, so_bias_f32, so_upsample2d_f32, so_concat
+ *   so_relu_f32, so_leaky_relu_f32, so_accum_f32, so_bias_f32, so_upsample2d_f32, so_upsample1d_f32, so_concat
  *        closed forms (exact), reference fixtures (relu), REF/ZEN2 builds
  *   so_dropout_f32, so_softmax_f32   REF/ZEN2 builds (dropout exact; softmax within 1e-6 relative:
  *        the reduction order of the global sum differs), closed form sum(out) == 1
@@ -458,6 +458,24 @@ int so_upsample2d_f32(int batch, int cb, int scale, int C, int H, int W, const f
                     for (int c = 0; c < cb; c++)
                         O[((size_t)i * Wo + j) * cb + c] = I[((size_t)(i / 2) * W + (j / 2)) * cb + c];
         }
+    return SO_OK;
+}
+
+/* UpSample1D (interface_abstract_1D.hpp:1614-1655): x2 along the width only; rows = its batch_size argument */
+int so_upsample1d_f32(int batch, int cb, int scale, int C, int rows, int W, const float *in, float *out)
+{
+    if (scale == 1)
+    {
+        memmove(out, in, (size_t)batch * C * rows * W * sizeof(float));
+        return SO_OK;
+    }
+    if (scale != 2) return SO_ESCALE;
+    if (C <= 0 || C % cb != 0) return SO_ECHANNELS;
+    const size_t planes = (size_t)batch * (C / cb) * rows;
+    for (size_t p = 0; p < planes; p++)
+        for (int j = 0; j < 2 * W; j++)
+            for (int c = 0; c < cb; c++)
+                out[(p * 2 * W + j) * cb + c] = in[(p * W + j / 2) * cb + c];
     return SO_OK;
 }
 

@@ -87,6 +87,7 @@ int so_bias_f32(int batch, int cb, int C, int H, int W, const float *bias, float
                 int accumulate);
 int so_upsample2d_f32(int batch, int cb, int scale, int C, int H, int W, const float *in,
                       float *out);
+int so_upsample1d_f32(int batch, int cb, int scale, int C, int rows, int W, const float *in, float *out);
 int so_concat(int batch, uint32_t C0, uint32_t C1, uint32_t H, uint32_t W, const void *in0,
               const void *in1, void *out, size_t esize);
 /* y = W x : Conv2D(1,1,...) on a 1x1 image (how every reference model spells a

@@ -93,13 +93,13 @@ __global__ __launch_bounds__(TPB) void bias_f32_kernel(const float4 *__restrict_
     }
 }
 
-// nearest-neighbour x2: one lane per output float4
+// nearest-neighbour x2 (along the width, and along the height too when hshift is 1): one lane per output float4
 __global__ __launch_bounds__(TPB) void upsample2_f32_kernel(const float4 *__restrict__ in,
                                                             float4 *__restrict__ out, size_t n4out,
-                                                            int H, int W)
+                                                            int H, int W, int hshift)
 {
     const size_t base = (size_t)blockIdx.x * (TPB * UNROLL) + threadIdx.x;
-    const int Wo = 2 * W, Ho = 2 * H;
+    const int Wo = 2 * W, Ho = H << hshift;
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
     {
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(TPB) void upsample2_f32_kernel(const float4 *__rest
             const PixelPos pp = split_pixel(i >> 2, Wo, Ho);
             const int ow = pp.ow, oh = pp.oh;
             const size_t plane = pp.plane;                    // n * cblocks + cb
-            out[i] = in[((plane * H + (oh >> 1)) * W + (ow >> 1)) * 4 + q];
+            out[i] = in[((plane * H + (oh >> hshift)) * W + (ow >> 1)) * 4 + q];
         }
     }
 }
@@ -295,26 +295,41 @@ int small_hip_partial_bias_f32(int batch, int C, int H, int W, const float *bias
     return bias_impl(true, batch, C, H, W, bias, out, stream);
 }
 
+static int upsample_impl(const char *name, int hshift, int batch, int scale, int C, int H, int W, const float *in,
+                         float *out, small_hip_stream_t stream);
+
 int small_hip_upsample2d_f32(int batch, int scale, int C, int H, int W, const float *in, float *out,
                              small_hip_stream_t stream)
+{
+    return upsample_impl("small_hip_upsample2d_f32", 1, batch, scale, C, H, W, in, out, stream);
+}
+
+int small_hip_upsample1d_f32(int batch, int scale, int C, int rows, int W, const float *in, float *out,
+                             small_hip_stream_t stream)
+{
+    return upsample_impl("small_hip_upsample1d_f32", 0, batch, scale, C, rows, W, in, out, stream);
+}
+
+static int upsample_impl(const char *name, int hshift, int batch, int scale, int C, int H, int W, const float *in,
+                         float *out, small_hip_stream_t stream)
 {
     // interface_abstract.hpp:1858-1886: scale 1 copies whatever the channel count is, scale 2
     // checks the channel count, anything else is a scale error
     if (scale == 1)
     {
-        if (batch <= 0 || C <= 0 || H <= 0 || W <= 0 || !in || !out) return einval("small_hip_upsample2d_f32: bad argument");
+        if (batch <= 0 || C <= 0 || H <= 0 || W <= 0 || !in || !out) { set_error("%s: bad argument", name); return SMALL_HIP_EINVAL; }
         if (in != out)
             SHP_HIP(hipMemcpyAsync(out, in, (size_t)batch * C * H * W * sizeof(float),
                                    hipMemcpyDeviceToDevice, as_stream(stream)));
         return SMALL_HIP_OK;
     }
     if (scale != 2) return SMALL_HIP_ESCALE;
-    if (int rc = check_act_args("small_hip_upsample2d_f32", batch, C, H, W, in, out)) return rc;
-    if (in == out) return einval("small_hip_upsample2d_f32: in-place upsampling is not possible");
-    const size_t n4 = (size_t)batch * C * H * W;  // 4x the elements, /4 per vector
+    if (int rc = check_act_args(name, batch, C, H, W, in, out)) return rc;
+    if (in == out) { set_error("%s: in-place upsampling is not possible", name); return SMALL_HIP_EINVAL; }
+    const size_t n4 = ((size_t)batch * C * H * W) << hshift >> 1;  // 2x or 4x the elements, /4 per vector
     hipLaunchKernelGGL(upsample2_f32_kernel, dim3(blocks_for(n4)), dim3(TPB), 0, as_stream(stream),
-                       reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out), n4, H, W);
-    SHP_LAUNCH_CHECK("small_hip_upsample2d_f32");
+                       reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out), n4, H, W, hshift);
+    SHP_LAUNCH_CHECK(name);
     return SMALL_HIP_OK;
 }
 

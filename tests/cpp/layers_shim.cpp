@@ -15,6 +15,7 @@
 #include <small.h>
 #include <small/AddLayer.hpp>
 #include <small/AveragePool2DLayer.hpp>
+#include <small/Conv1DLayer.hpp>
 #include <small/Conv2DLayer.hpp>
 #include <small/DepthwiseConv2DLayer.hpp>
 #include <small/DummyLayer.hpp>
@@ -94,7 +95,7 @@ void set_quant(small::QUInt8Buffer &b, int32_t const *q)
     b.rshift = q[3];
 }
 
-// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer
+// kind: 0 Conv2DLayer, 1 PartialConv2DLayer, 2 DepthwiseConv2DLayer, 3 Conv1DLayer
 template <class BufferT>
 std::unique_ptr<small::Layer<BufferT>> make_conv_layer(int kind, small::shape_type const &in_shape, int kh, int kw,
                                                        int stride, int padding, int Co, BufferT const &filt,
@@ -104,7 +105,16 @@ std::unique_ptr<small::Layer<BufferT>> make_conv_layer(int kind, small::shape_ty
     const auto pad = padding ? small::PADDING_F : small::PADDING_V;
     const auto a = (small::ActivationType)act;
     small::Layer<BufferT> *l = nullptr;
-    if (kind == 2)
+    if (kind == 3)      // Conv1DLayer (float only): kh is ignored
+    {
+        if constexpr (std::is_same<BufferT, small::FloatBuffer>::value)
+        {
+            if (bn) l = new small::Conv1DLayer<BufferT>(in_shape, kw, stride, pad, Co, filt, bn[0], bn[1], bn[2], bn[3], eps, false, a, slope);
+            else if (bias.size()) l = new small::Conv1DLayer<BufferT>(in_shape, kw, stride, pad, Co, filt, bias, false, a, slope);
+            else l = new small::Conv1DLayer<BufferT>(in_shape, kw, stride, pad, Co, filt, false, a, slope);
+        }
+    }
+    else if (kind == 2)
     {
         if (bn) l = new small::DepthwiseConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, filt, bias, bn[0], bn[1], bn[2], bn[3], eps, false, a, slope);
         else if (bias.size()) l = new small::DepthwiseConv2DLayer<BufferT>(in_shape, kh, kw, stride, pad, filt, bias, false, a, slope);
@@ -340,6 +350,31 @@ int stest_fused_two_layers_f32(int second, int variant, int ck, int cs, int ct, 
         else
             small::Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU(ck, ck, cs, ct, cb, cl, cr, k2, k2, s2, t2, b2, l2, r2, Co,
                                                               Ci, H, W, x, f, b, inter, df, db, o);
+        std::memcpy(out, o.data(), n_out * sizeof(float));
+    });
+}
+
+// The 1-D functions of small/interface_1D.hpp on PACKED arrays (batch-1 signatures of the reference; rows = its
+// batch_size).  kind 0 Conv1D, 1 PartialConv1D (out is in/out), 2 MaxPool1D, 3 AveragePool1D, 4 ReLUActivation1D,
+// 5 UpSample1D (k = scale), 6 Conv1D_ReLU, 7 Conv1D_Bias_ReLU (bias = 4th array)
+int stest_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows, int W, const float *in, size_t n_in,
+                 const float *filt, size_t n_filt, const float *bias, float *out, size_t n_out)
+{
+    using FB = small::FloatBuffer;
+    return guarded([&] {
+        FB x = from_host<FB>(in, n_in), f = from_host<FB>(filt, n_filt), b = from_host<FB>(bias, bias ? Co : 0);
+        FB o = from_host<FB>(out, n_out);
+        switch (kind)
+        {
+        case 0: small::Conv1D(k, s, l, r, Co, Ci, rows, W, x, f, o); break;
+        case 1: small::PartialConv1D(k, s, l, r, Co, Ci, rows, W, x, f, o); break;
+        case 2: small::MaxPool1D(k, s, l, r, Ci, rows, W, x, o); break;
+        case 3: small::AveragePool1D(k, s, l, r, Ci, rows, W, x, o); break;
+        case 4: small::ReLUActivation1D(Ci, rows, W, x, o); break;
+        case 5: small::UpSample1D(k, Ci, rows, W, x, o); break;
+        case 6: small::Conv1D_ReLU(k, s, l, r, Co, Ci, rows, W, x, f, o); break;
+        default: small::Conv1D_Bias_ReLU(k, s, l, r, Co, Ci, rows, W, x, f, b, o); break;
+        }
         std::memcpy(out, o.data(), n_out * sizeof(float));
     });
 }

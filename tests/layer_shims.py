@@ -136,6 +136,16 @@ class HipLayers(_Shim):
         self._check(rc)
         return out
 
+    def one_d_f32(self, kind, k, s, l, r, Co, Ci, rows, W, x, f, bias, out_init, n_out):
+        """The 1-D functions of small/interface_1D.hpp on packed arrays (kinds: tests/cpp/layers_shim.cpp)."""
+        out = np.zeros(n_out, np.float32) if out_init is None else np.ascontiguousarray(out_init, np.float32).copy()
+        f = np.zeros(1, np.float32) if f is None else f
+        rc = self.lib.stest_1d_f32(*[C.c_int(v) for v in (kind, k, s, l, r, Co, Ci, rows, W)], _f32p(x),
+                                   C.c_size_t(x.size), _f32p(f), C.c_size_t(f.size), _f32p(bias), _f32p(out),
+                                   C.c_size_t(n_out))
+        self._check(rc)
+        return out
+
     def fused_single_f32(self, variant, k, s, p, Co, Ci, H, W, x, f, bias, n_out):
         out = np.zeros(n_out, np.float32)
         ints = [variant, k, s, *p, Co, Ci, H, W]

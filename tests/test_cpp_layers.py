@@ -150,6 +150,38 @@ def test_single_layer_fused_functions(hip, oracle, case, variant):
     assert_close_f32(got, want, what="%s %d" % (case, variant))
 
 
+# ---- 1-D functions ------------------------------------------------------------------------------------------------
+from test_oracle_1d_vs_ref import KINDS, ONE_D_CASES, one_d_inputs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", range(8), ids=KINDS + ["conv_relu", "conv_bias_relu"])
+@pytest.mark.parametrize("case", ONE_D_CASES, ids=str)
+def test_one_d_functions(hip, oracle, case, kind):
+    k, s, l, r, Co, Ci, rows, W = case
+    okind = 0 if kind >= 6 else kind              # Conv1D_ReLU / Conv1D_Bias_ReLU: convolution, then the epilogue
+    if okind >= 2 and Ci % 16:
+        pytest.skip("needs whole channel blocks")
+    x, f, init, n_out = one_d_inputs(case, okind, 16, oracle)
+    kk = 2 if kind == 5 else k
+    bias = synth.normal(4, Co) if kind == 7 else None
+    if rows > 1 and s != 1 and kind not in (4, 5):
+        with pytest.raises(ValueError, match="more than one row needs stride 1"):
+            hip.one_d_f32(kind, kk, s, l, r, Co, Ci, rows, W, x, f, bias, init, n_out)
+        return
+    got = hip.one_d_f32(kind, kk, s, l, r, Co, Ci, rows, W, x, f, bias, init, n_out)
+    if kind >= 6:
+        Wo = 1 + (W + l + r - k) // s
+        rc, want = oracle.conv2d_bias_act_f32(1, 16, 1, k, s, 0, 0, l, r, Co, Ci, rows, W, x, f, bias, ol.RELU, 0.0)
+        assert rc == 0 and want.size == Co * rows * Wo
+    else:
+        want = ol.one_d_f32(oracle, kind, 16, kk, s, l, r, Co, Ci, rows, W, x, f, init)
+    if okind in (0, 1, 3):
+        assert_close_f32(got, want, what="%s %s" % (kind, case))
+    else:
+        assert_equal_exact(got, want, "%s %s" % (kind, case))
+
+
 # ---- quantised layers -------------------------------------------------------------------------------------
 DEFAULT_Q = (128, 1077952576, 0, 6)       # the fields of a fresh QUInt8Buffer
 QMAX = (1 << 31) - 1                      # multiplier ~ 1.0: ReLU and Accum requantise with the output's scale again

@@ -50,12 +50,20 @@ CONV_LAYER_CASES = [
     (2, 16, 8, 8, 3, 3, 2, 0, 16, False, True, ol.LEAKY),
     (0, 64, 1, 1, 1, 1, 1, 0, 16, True, False, ol.SOFTMAX),     # classifier head with the softmax attached
     (0, 16, 4, 4, 3, 3, 1, 1, 16, False, False, ol.SOFTMAX),
+    # Conv1DLayer (kind 3; kh unused; H = rows): the reference's own test shape first (test_conv1d.cpp:41)
+    (3, 16, 1, 13, 1, 3, 1, 1, 64, False, False, ol.NONE),
+    (3, 16, 1, 13, 1, 3, 2, 1, 32, True, False, ol.RELU),
+    (3, 32, 3, 12, 1, 3, 1, 1, 20, False, True, ol.LEAKY),       # three rows, 20 -> 32 outputs
+    (3, 3, 1, 24, 1, 5, 1, 0, 16, True, False, ol.RELU),
+    (3, 16, 2, 9, 1, 1, 1, 0, 16, False, False, ol.SOFTMAX),
 ]
 
 
 def conv_layer_inputs(case, batch=1, seed=0):
     kind, C, H, W, kh, kw, stride, padding, Co, has_bias, has_bn, act = case
     ci = 1 if kind == 2 else C
+    if kind == 3:
+        kh = 1
     x = synth.normal(seed + 1, batch * C * H * W).reshape(batch, C, H, W)
     f = synth.he_normal(seed + 2, Co * ci * kh * kw, ci * kh * kw).reshape((Co, kh, kw) if kind == 2 else (Co, C, kh, kw))
     bias = synth.normal(seed + 3, Co) if has_bias else None
@@ -73,6 +81,8 @@ def conv_layer_inputs(case, batch=1, seed=0):
 def test_conv_layers(oracle, plat, case):
     name, ref = plat
     kind, C, H, W, kh, kw, stride, padding, Co, has_bias, has_bn, act = case
+    if kind == 3 and H > 1 and name == "ZEN2":
+        pytest.skip("the reference's ZEN2 build aborts in Conv1D on more than one row; its scalar build runs it")
     x, f, bias, bn, init = conv_layer_inputs(case)
     eps, slope = 1e-3, 0.1
     want = ref.conv_layer_f32(kind, x, f, bias, bn, eps, act, slope, kh, kw, stride, padding, out_init=init)
