@@ -223,6 +223,23 @@ def dscnn_tiny(oracle, x, filters, stem=(3, 1), average_pool=False):
     return conv_layer_f32(oracle, 0, y, next(f), None, None, 0, NONE, 0, 1, 1, 1, 0)
 
 
+def autoencoder_specs(in_channels=128, bottleneck=16, layers=9):
+    """AutoencoderTiny.hpp:176-205: 1x1 convolutions, 128 outputs each but layer 4 (the bottleneck)."""
+    specs, ci = [], in_channels
+    for ix in range(layers):
+        co = bottleneck if ix == 4 else 128
+        specs.append(("conv", co, ci, 1, 1))
+        ci = pad_up(co)
+    return specs
+
+
+def autoencoder_tiny(oracle, x, filters):
+    y = x
+    for f in filters:
+        y = conv_layer_f32(oracle, 0, y, f, None, None, 0, RELU, 0, 1, 1, 1, 0)
+    return y
+
+
 def yolo_specs():
     specs, c, ci = [], 16, 3
     for _ in range(6):

@@ -41,6 +41,8 @@
 #include <small/models/Resnet8Tiny.hpp>
 #include <small/models/DSCNNTiny.hpp>
 #include <small/models/TinyYoloV2.hpp>
+#include <small/models/AutoencoderTiny.hpp>
+#include <small/models/DSCNNSquareTiny.hpp>
 
 #include <memory>
 #include <vector>
@@ -469,6 +471,8 @@ int sref_model_f32(int which, int C, int H, int W, const float *const *filters, 
         case 1: m.reset(new small::Resnet8Tiny<FB>(is, fl, false)); break;
         case 2: m.reset(new small::DSCNNTiny<FB>(is, fl, false)); break;
         case 3: m.reset(new small::TinyYoloV2<FB>(is, fl, false)); break;
+        case 4: m.reset(new small::AutoencoderTiny<FB>(is, 16, fl, false)); break;
+        case 5: m.reset(new small::DSCNNSquareTiny<FB>(is, fl, false)); break;
         default: throw std::invalid_argument("sref_model_f32: unknown model");
         }
         auto x = packed_tensor(in, is);

@@ -26,6 +26,8 @@
 #include <small/RouteLayer.hpp>
 #include <small/SoftMaxLayer.hpp>
 #include <small/UpSample2DLayer.hpp>
+#include <small/models/AutoencoderTiny.hpp>
+#include <small/models/DSCNNSquareTiny.hpp>
 #include <small/models/DSCNNTiny.hpp>
 #include <small/models/MobileNetTiny.hpp>
 #include <small/models/Resnet8Tiny.hpp>
@@ -249,6 +251,8 @@ int stest_model_f32(int which, int variant, int batch, int C, int H, int W, cons
                                 : new small::DSCNNTiny<FB>(is, fl, false)); break;
         case 3: m.reset(variant ? new small::TinyYoloV2<FB>(is, fl, false, small::LEAKY, 0.1f, 125, false)
                                 : new small::TinyYoloV2<FB>(is, fl, false)); break;
+        case 4: m.reset(new small::AutoencoderTiny<FB>(is, 16, fl, false)); break;
+        case 5: m.reset(new small::DSCNNSquareTiny<FB>(is, fl, false)); break;
         default: throw std::invalid_argument("stest_model_f32: unknown model");
         }
         auto x = packed_tensor<FB>(in, is);

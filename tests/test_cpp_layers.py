@@ -95,12 +95,18 @@ def _model_case(name):
     if name == "TinyYoloV2_leaky_125":
         fl = ol.make_filters(synth, ol.yolo_specs(), 125)
         return 3, 1, lambda o, x, f: ol.tiny_yolo_v2(o, x, f, ol.LEAKY, 0.1, False), fl, (2, 3, 160, 160)
+    if name == "AutoencoderTiny":
+        return 4, 0, ol.autoencoder_tiny, ol.make_filters(synth, ol.autoencoder_specs(), 16), (3, 128, 1, 1)
+    if name == "DSCNNSquareTiny":
+        fl = ol.make_filters(synth, ol.dscnn_specs((3, 3)), 16)
+        return 5, 0, lambda o, x, f: ol.dscnn_tiny(o, x, f, stem=(3, 3)), fl, (3, 3, 49, 10)
     raise KeyError(name)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["MobileNetTiny", "MobileNetV1_224_1000", "Resnet8Tiny", "Resnet8_10", "DSCNNTiny",
-                                  "DSCNN_10x4_12", "TinyYoloV2", "TinyYoloV2_leaky_125"])
+                                  "DSCNN_10x4_12", "TinyYoloV2", "TinyYoloV2_leaky_125", "AutoencoderTiny",
+                                  "DSCNNSquareTiny"])
 def test_models(hip, oracle, name):
     which, variant, fn, filters, shape = _model_case(name)
     x = synth.normal(55, int(np.prod(shape))).reshape(shape)

@@ -140,6 +140,9 @@ MODEL_CASES = [
     (1, "Resnet8Tiny", ol.resnet8_specs, ol.resnet8_tiny, (3, 32, 32)),
     (2, "DSCNNTiny", ol.dscnn_specs, ol.dscnn_tiny, (3, 49, 10)),
     (3, "TinyYoloV2", ol.yolo_specs, ol.tiny_yolo_v2, (3, 96, 96)),
+    (4, "AutoencoderTiny", ol.autoencoder_specs, ol.autoencoder_tiny, (128, 1, 1)),
+    (5, "DSCNNSquareTiny", lambda: ol.dscnn_specs((3, 3)), lambda o, x, f: ol.dscnn_tiny(o, x, f, stem=(3, 3)),
+     (3, 49, 10)),
 ]
 
 
