@@ -178,6 +178,14 @@ int small_hip_dropout_f32(int batch, int input_channels, int input_height, int i
  * In place allowed.  No quantised version in the reference. */
 int small_hip_softmax_f32(int batch, int input_channels, int input_height, int input_width,
                           const float *input, float *output, small_hip_stream_t stream);
+/* small::YOLOLayer<FloatBuffer>::compute_output   YOLOLayer.hpp:150-222: decodes a detection head.
+ * input: packed [padded_channels/16][H][W][16], channel a*(5+classes)+f = field f of anchor a;
+ * output: flat [batch][num_anchors*H*W][5+classes] records {cx, cy, w, h, objectness, class scores}:
+ *   cx = s*(sigmoid(x)+col), cy = s*(sigmoid(x)+row), w = exp(x)*anchor_w, h = exp(x)*anchor_h, rest sigmoid(x),
+ *   s = image_size / H (integer division).  anchors_wh: HOST array {w0,h0,w1,h1,...}, at most 8 anchors. */
+int small_hip_yolo_decode_f32(int batch, int padded_channels, int input_height, int input_width, int num_anchors,
+                              const uint32_t *anchors_wh, int num_classes, int image_size, const float *input,
+                              float *output, small_hip_stream_t stream);
 /* small::Accum<FloatBuffer>           interface.hpp:451-455, interface_abstract.hpp:1950-1978 */
 int small_hip_accum_f32(int batch, int input_channels, int input_height, int input_width,
                         const float *input, float *output, small_hip_stream_t stream);

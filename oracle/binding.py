@@ -70,6 +70,7 @@ class Oracle:
         L.so_bias_f32.argtypes = [c_int] * 5 + [c_vp, c_vp, c_int]
         L.so_upsample2d_f32.argtypes = [c_int] * 6 + [c_vp, c_vp]
         L.so_upsample1d_f32.argtypes = [c_int] * 6 + [c_vp, c_vp]
+        L.so_yolo_decode_f32.argtypes = [c_int] * 6 + [c_vp, c_int, c_int, c_vp, c_vp]
         L.so_concat.argtypes = [c_int] + [C.c_uint32] * 4 + [c_vp, c_vp, c_vp, C.c_size_t]
         L.so_dense_f32.argtypes = [c_int] * 4 + [c_vp, c_vp, c_vp]
         L.so_dense_literal_f32.argtypes = [c_int] * 3 + [c_vp, c_vp, c_vp]
@@ -182,6 +183,12 @@ class Oracle:
     def upsample1d_f32(self, batch, cb, scale, Cn, rows, W, x):
         out = np.zeros(batch * Cn * rows * W * (scale if scale in (1, 2) else 1), np.float32)
         return self.lib.so_upsample1d_f32(batch, cb, scale, Cn, rows, W, _p(x), _p(out)), out
+
+    def yolo_decode_f32(self, batch, cb, Cn, H, W, anchors, classes, image_size, x):
+        """anchors: [(w, h), ...] -> flat [batch][len(anchors) * H * W][5 + classes]"""
+        an = np.ascontiguousarray(np.asarray(anchors, np.uint32).ravel())
+        out = np.zeros(batch * len(anchors) * H * W * (classes + 5), np.float32)
+        return self.lib.so_yolo_decode_f32(batch, cb, Cn, H, W, len(anchors), _p(an), classes, image_size, _p(x), _p(out)), out
 
     def concat(self, batch, C0, C1, H, W, a, b):
         out = np.empty(a.size + b.size, a.dtype)

@@ -461,6 +461,37 @@ int so_upsample2d_f32(int batch, int cb, int scale, int C, int H, int W, const f
     return SO_OK;
 }
 
+/* YOLOLayer::compute_output (YOLOLayer.hpp:150-222; sigmoid :21-24 is evaluated in double around a float exp) */
+int so_yolo_decode_f32(int batch, int cb, int C, int H, int W, int num_anchors, const uint32_t *anchors_wh,
+                       int num_classes, int image_size, const float *in, float *out)
+{
+    const int nrec = num_classes + 5;
+    if (C <= 0 || C % cb != 0) return SO_ECHANNELS;
+    if (num_anchors * nrec > C) return SO_EINVAL;
+    const float stride = (float)(image_size / H);
+    size_t o = 0;
+    for (int n = 0; n < batch; n++)
+        for (int a = 0; a < num_anchors; a++)
+            for (int i = 0; i < H; i++)
+                for (int j = 0; j < W; j++)
+                    for (int f = 0; f < nrec; f++)
+                    {
+                        const int c = a * nrec + f;
+                        const float x = in[((((size_t)n * (C / cb) + c / cb) * H + i) * W + j) * cb + c % cb];
+                        float r;
+                        if (f == 2) r = expf(x) * (float)anchors_wh[2 * a];
+                        else if (f == 3) r = expf(x) * (float)anchors_wh[2 * a + 1];
+                        else
+                        {
+                            r = (float)(1.0 / (1.0 + expf(-x)));
+                            if (f == 0) r = stride * (r + (float)j);
+                            else if (f == 1) r = stride * (r + (float)i);
+                        }
+                        out[o++] = r;
+                    }
+    return SO_OK;
+}
+
 /* UpSample1D (interface_abstract_1D.hpp:1614-1655): x2 along the width only; rows = its batch_size argument */
 int so_upsample1d_f32(int batch, int cb, int scale, int C, int rows, int W, const float *in, float *out)
 {

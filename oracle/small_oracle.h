@@ -87,6 +87,8 @@ int so_bias_f32(int batch, int cb, int C, int H, int W, const float *bias, float
                 int accumulate);
 int so_upsample2d_f32(int batch, int cb, int scale, int C, int H, int W, const float *in,
                       float *out);
+int so_yolo_decode_f32(int batch, int cb, int C, int H, int W, int num_anchors, const uint32_t *anchors_wh,
+                       int num_classes, int image_size, const float *in, float *out);
 int so_upsample1d_f32(int batch, int cb, int scale, int C, int rows, int W, const float *in, float *out);
 int so_concat(int batch, uint32_t C0, uint32_t C1, uint32_t H, uint32_t W, const void *in0,
               const void *in1, void *out, size_t esize);

@@ -115,6 +115,41 @@ __global__ __launch_bounds__(TPB) void upsample2_f32_kernel(const float4 *__rest
     }
 }
 
+// YOLO head decode (include/small/YOLOLayer.hpp:150-222): packed [C/16][H][W][16] scores -> [anchor][h][w][5 + classes]
+// box records.  One lane per output element; consecutive lanes write consecutive floats of a record.
+struct YoloAnchors
+{
+    float w[8], h[8];
+};
+
+__global__ __launch_bounds__(TPB) void yolo_decode_f32_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                              size_t n_out, int C, int H, int W, int na, int nrec,
+                                                              float stride, YoloAnchors anchors)
+{
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n_out) return;
+    const int field = (int)(i % (size_t)nrec);
+    size_t pred = i / (size_t)nrec;
+    const int ow = (int)(pred % (size_t)W);
+    pred /= (size_t)W;
+    const int oh = (int)(pred % (size_t)H);
+    pred /= (size_t)H;                       // n * anchors + anchor
+    const int a = (int)(pred % (size_t)na);
+    const size_t n = pred / (size_t)na;
+    const int c = a * nrec + field;
+    const float x = in[((n * (size_t)(C / CB) + (size_t)(c / CB)) * H + oh) * (size_t)W * CB + (size_t)ow * CB + (c % CB)];
+    float r;
+    if (field == 2) r = expf(x) * anchors.w[a];
+    else if (field == 3) r = expf(x) * anchors.h[a];
+    else
+    {
+        r = (float)(1.0 / (1.0 + (double)expf(-x)));
+        if (field == 0) r = stride * (r + (float)ow);
+        else if (field == 1) r = stride * (r + (float)oh);
+    }
+    out[i] = r;
+}
+
 // concat: per image two contiguous copies, 16-byte granules
 __global__ __launch_bounds__(TPB) void concat_kernel(const uint4 *__restrict__ in0,
                                                      const uint4 *__restrict__ in1,
@@ -329,6 +364,33 @@ static int upsample_impl(const char *name, int hshift, int batch, int scale, int
     const size_t n4 = ((size_t)batch * C * H * W) << hshift >> 1;  // 2x or 4x the elements, /4 per vector
     hipLaunchKernelGGL(upsample2_f32_kernel, dim3(blocks_for(n4)), dim3(TPB), 0, as_stream(stream),
                        reinterpret_cast<const float4 *>(in), reinterpret_cast<float4 *>(out), n4, H, W, hshift);
+    SHP_LAUNCH_CHECK(name);
+    return SMALL_HIP_OK;
+}
+
+int small_hip_yolo_decode_f32(int batch, int padded_channels, int H, int W, int num_anchors,
+                              const uint32_t *anchors_wh, int num_classes, int image_size, const float *in,
+                              float *out, small_hip_stream_t stream)
+{
+    const char *name = "small_hip_yolo_decode_f32";
+    if (int rc = check_act_args(name, batch, padded_channels, H, W, in, out)) return rc;
+    if (num_anchors <= 0 || num_anchors > 8 || num_classes < 0 || !anchors_wh || image_size < H)
+    {
+        set_error("%s: 1..8 anchors, a class count >= 0 and an image at least as high as the map are needed", name);
+        return SMALL_HIP_EINVAL;
+    }
+    const int nrec = num_classes + 5;
+    if ((long)num_anchors * nrec > padded_channels)
+    {
+        set_error("%s: %d anchors x %d fields do not fit %d channels", name, num_anchors, nrec, padded_channels);
+        return SMALL_HIP_EINVAL;
+    }
+    if (in == out) { set_error("%s: in-place decode is not possible", name); return SMALL_HIP_EINVAL; }
+    YoloAnchors an{};
+    for (int a = 0; a < num_anchors; ++a) { an.w[a] = (float)anchors_wh[2 * a]; an.h[a] = (float)anchors_wh[2 * a + 1]; }
+    const size_t n_out = (size_t)batch * num_anchors * H * W * nrec;
+    hipLaunchKernelGGL(yolo_decode_f32_kernel, dim3((unsigned)((n_out + TPB - 1) / TPB)), dim3(TPB), 0, as_stream(stream),
+                       in, out, n_out, padded_channels, H, W, num_anchors, nrec, (float)(image_size / H), an);
     SHP_LAUNCH_CHECK(name);
     return SMALL_HIP_OK;
 }

@@ -29,6 +29,7 @@
 #include <small/models/AutoencoderTiny.hpp>
 #include <small/models/DSCNNSquareTiny.hpp>
 #include <small/models/DSCNNTiny.hpp>
+#include <small/models/Darknet.hpp>
 #include <small/models/MobileNetTiny.hpp>
 #include <small/models/Resnet8Tiny.hpp>
 #include <small/models/TinyYoloV2.hpp>
@@ -397,6 +398,99 @@ int stest_fused_single_f32(int variant, int k, int s, int t, int b, int l, int r
         else if (variant == 2) small::Conv2D_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, x, f, o);
         else small::Conv2D_Bias_ReLU(k, k, s, t, b, l, r, Co, Ci, H, W, x, f, bb, o);
         std::memcpy(out, o.data(), n_out * sizeof(float));
+    });
+}
+
+// ---- Darknet cfg / weights model, YOLO decode, non-maximum suppression -------------------------------------------
+// Runs the model the two files describe on one flat [C][H][W] image.  out receives the YOLO heads' records one
+// after the other (each head is [predictions][5 + classes]); out_preds[i] = predictions of head i.
+// det (may be NULL): detections after process_outputs(conf, iou), 7 floats each {x, y, w, h, objectness, class
+// score, class id}; *n_det in: capacity, out: count.
+int stest_darknet_f32(const char *cfg, const char *weights, const float *in, size_t n_in, float *out, size_t out_cap,
+                       int *out_preds, int *n_heads, int *record_len, float conf, float iou, float *det, int *n_det)
+{
+    return guarded([&] {
+        small::Darknet<FB> model(cfg, weights);
+        auto const &is = model.get_input_shape();
+        if (small::compute_size(is) != n_in) throw std::invalid_argument("darknet shim: input size mismatch");
+        auto x = packed_tensor<FB>(in, is);
+        auto outs = model.inference(&x);
+        size_t at = 0;
+        *n_heads = (int)outs.size();
+        for (size_t i = 0; i < outs.size(); ++i)
+        {
+            auto const &s = outs[i]->shape();
+            out_preds[i] = (int)s[2];
+            *record_len = (int)s[3];
+            const size_t n = s[2] * s[3];
+            if (at + n > out_cap) throw std::invalid_argument("darknet shim: output capacity");
+            for (size_t k = 0; k < n; ++k) out[at + k] = outs[i]->buffer()[k];
+            at += n;
+        }
+        if (det)
+        {
+            auto d = model.process_outputs(outs, conf, iou);
+            const int cap = *n_det;
+            *n_det = (int)d.size();
+            for (int i = 0; i < (int)d.size() && i < cap; ++i)
+            {
+                float *r = det + 7 * i;
+                r[0] = d[i].bbox.x; r[1] = d[i].bbox.y; r[2] = d[i].bbox.w; r[3] = d[i].bbox.h;
+                r[4] = d[i].objectness; r[5] = d[i].class_score; r[6] = (float)d[i].class_id;
+            }
+        }
+    });
+}
+
+// basic_nms on n records of 7 floats (layout as above); kept records are written to out, their count returned in *n_out
+int stest_nms(const float *pred, int n, float iou, float *out, int *n_out)
+{
+    return guarded([&] {
+        std::vector<small::Detection> p;
+        for (int i = 0; i < n; ++i)
+        {
+            const float *r = pred + 7 * i;
+            p.push_back(small::Detection{{r[0], r[1], r[2], r[3]}, r[4], r[5], (size_t)r[6]});
+        }
+        auto k = small::basic_nms(p, iou);
+        *n_out = (int)k.size();
+        for (size_t i = 0; i < k.size(); ++i)
+        {
+            float *r = out + 7 * i;
+            r[0] = k[i].bbox.x; r[1] = k[i].bbox.y; r[2] = k[i].bbox.w; r[3] = k[i].bbox.h;
+            r[4] = k[i].objectness; r[5] = k[i].class_score; r[6] = (float)k[i].class_id;
+        }
+    });
+}
+
+// YOLOLayer on a flat [C][H][W] input (C is padded to the channel block with zeros by the caller)
+int stest_yolo_layer_f32(int C, int H, int W, const uint32_t *anchors_wh, int num_anchors, int classes, int image_size,
+                          const float *in, float *out)
+{
+    return guarded([&] {
+        const small::shape_type is{1UL, (size_t)C, (size_t)H, (size_t)W};
+        std::vector<std::pair<uint32_t, uint32_t>> an;
+        for (int a = 0; a < num_anchors; ++a) an.emplace_back(anchors_wh[2 * a], anchors_wh[2 * a + 1]);
+        small::YOLOLayer<FB> layer(is, an, classes, image_size);
+        auto x = packed_tensor<FB>(in, is);
+        small::Tensor<FB> y(layer.output_shape());
+        layer.compute_output({&x}, &y);
+        for (size_t k = 0; k < layer.output_size(); ++k) out[k] = y.buffer()[k];
+    });
+}
+
+// Milliseconds per Darknet::inference() call at `batch` images (input left as allocated; resident on the device).
+int stest_darknet_time(const char *cfg, const char *weights, int batch, int steps, int warmup, double *ms_per_call)
+{
+    return guarded([&] {
+        small::Darknet<FB> model(cfg, weights, false, (uint32_t)batch);
+        small::Tensor<FB> x(model.get_input_shape());
+        for (int i = 0; i < warmup; ++i) model.inference(&x);
+        small::synchronize();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < steps; ++i) model.inference(&x);
+        small::synchronize();
+        *ms_per_call = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
     });
 }
 

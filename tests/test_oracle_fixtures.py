@@ -8,8 +8,10 @@ reference's REF platform) and 16 (its ZEN2 platform and the HIP library).
 import numpy as np
 import pytest
 
+import os
+
 import fixtures
-from util import assert_close_f32, assert_equal_exact
+from util import GOLDEN, assert_close_f32, assert_equal_exact, read_ref_bin
 
 CBS = [1, 16]
 REF_RTOL, REF_ATOL = 5e-3, 1e-5  # almost_equal() in the reference's test_utils.hpp
@@ -110,3 +112,17 @@ def test_relu_exact(oracle, case, cb):
     rc, out = oracle.relu_f32(1, cb, Cn, H, W, oracle.pack(x, 0, 1, Cn, H, W, cb, cb))
     assert rc == 0
     assert_equal_exact(out, oracle.pack(y, 1, 1, Cn, H, W, cb, cb), what=case["id"])
+
+
+def test_yolo_decode_fixture(oracle):
+    """The reference's YOLO-head fixture (test/test_yolo.cpp:132-141: 255 channels on a 19x19 map of a 608x608 image,
+    anchors (116,90) (156,198) (373,326), 80 classes) against the restatement of YOLOLayer::compute_output."""
+    x = read_ref_bin(os.path.join(GOLDEN, "ref_regression", "in__yolo_Ci255_H19_W19_k0_s0_f_92055.bin"))
+    want = read_ref_bin(os.path.join(GOLDEN, "ref_regression", "out__yolo_Ci255_H19_W19_k0_s0_f_92055.bin"))
+    padded = np.zeros(256 * 19 * 19, np.float32)
+    padded[:x.size] = x
+    for cb in (1, 16):
+        xp = oracle.pack(padded, 0, 1, 256, 19, 19, cb, cb)
+        rc, got = oracle.yolo_decode_f32(1, cb, 256, 19, 19, [(116, 90), (156, 198), (373, 326)], 80, 608, xp)
+        assert rc == 0
+        assert_close_f32(got, want, what="yolo decode, channel block %d" % cb)
