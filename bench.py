@@ -125,6 +125,33 @@ def layer_table(model, batch, ms):
     return rows
 
 
+def library_gemm_ms(model, batch, steps, warmup):
+    """Calibration, not part of the product path: the contraction of every MFMA-sized convolution as a plain
+    float32 GEMM [Co x K] . [K x pixels] through torch.mm (the vendor BLAS; no im2col cost counted, TF32 off).
+    -> {layer name: milliseconds}.  It shows what a tuned library reaches on this machine for the same shapes."""
+    import torch
+    torch.backends.cuda.matmul.allow_tf32 = False
+    out = {}
+    for op in model.ops:
+        if op.kind not in ("conv", "dense") or op.C % 16 != 0:
+            continue
+        M, K = op.Co, op.C * op.kh * op.kw
+        N = batch * op.Ho * op.Wo
+        a = torch.randn(M, K, device="cuda")
+        b = torch.randn(K, N, device="cuda")
+        c = torch.empty(M, N, device="cuda")
+        for _ in range(warmup):
+            torch.mm(a, b, out=c)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            torch.mm(a, b, out=c)
+        e1.record()
+        torch.cuda.synchronize()
+        out[op.name] = e0.elapsed_time(e1) / steps
+    return out
+
+
 def cpu_threads():
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
     threads = min(threads, os.cpu_count() or threads)
@@ -270,6 +297,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="headline model only")
     ap.add_argument("--unfused", action="store_true", help="issue Conv2D and the activation as separate calls")
+    ap.add_argument("--library-gemm", action="store_true",
+                    help="calibration: also time every MFMA-sized convolution's contraction as a torch.mm float32 GEMM")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build measures one GPU; the path shards by image with no collective, "
@@ -299,8 +328,15 @@ def main():
     # per-op device times (HIP events on the launch stream) over the same number of steps
     ms = time_ops(ex, args.steps)
     table = layer_table(model, batch, ms)
+    if args.library_gemm:
+        lib_ms = library_gemm_ms(model, batch, args.steps, args.warmup)
+        for r in table:
+            if r["layer"] in lib_ms:
+                r["library_gemm_ms"] = round(lib_ms[r["layer"]], 5)
     for r in table:
-        log("  %-28s %9.4f ms  %-4s %6.1f%%" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0)))
+        log("  %-28s %9.4f ms  %-4s %6.1f%%%s" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0),
+                                                  "   library GEMM %.4f ms" % r["library_gemm_ms"]
+                                                  if "library_gemm_ms" in r else ""))
 
     # dominant kernel = the one with the largest summed time
     def kernel_of(op):
