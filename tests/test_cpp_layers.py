@@ -188,6 +188,22 @@ def test_one_d_functions(hip, oracle, case, kind):
         assert_equal_exact(got, want, "%s %s" % (kind, case))
 
 
+@pytest.mark.gpu
+def test_one_d_errors(hip, oracle):
+    """Same exception texts as the reference's 1-D functions (interface_abstract_1D.hpp:100-103, 160-163, 1650-1653)."""
+    x = np.zeros(16 * 12, np.float32)
+    f = np.zeros(16 * 16 * 3, np.float32)
+    with pytest.raises(ValueError, match=r"Conv1D<float> ERROR: stride unsupported\."):
+        hip.one_d_f32(0, 3, 3, 0, 0, 16, 16, 1, 12, x, f, None, None, 16 * 4)
+    with pytest.raises(ValueError, match=r"Conv1D<float> ERROR: in_channels unsupported\."):
+        hip.one_d_f32(0, 3, 1, 1, 1, 16, 5, 1, 12, np.zeros(5 * 12, np.float32), np.zeros(16 * 5 * 3, np.float32), None,
+                      None, 16 * 12)
+    with pytest.raises(ValueError, match=r"MaxPool1D<float> ERROR: stride unsupported\."):
+        hip.one_d_f32(2, 3, 3, 0, 0, 16, 16, 1, 12, x, None, None, None, 16 * 4)
+    with pytest.raises(ValueError, match=r"Upsample<float> ERROR: scale factor unsupported \(only 1 or 2\)\."):
+        hip.one_d_f32(5, 3, 1, 0, 0, 16, 16, 1, 12, x, None, None, None, 16 * 36)
+
+
 # ---- quantised layers -------------------------------------------------------------------------------------
 DEFAULT_Q = (128, 1077952576, 0, 6)       # the fields of a fresh QUInt8Buffer
 QMAX = (1 << 31) - 1                      # multiplier ~ 1.0: ReLU and Accum requantise with the output's scale again
