@@ -495,6 +495,7 @@ int sref_darknet_f32(const char *cfg, const char *weights, const float *in, size
         auto const &is = model.get_input_shape();
         if (small::compute_size(is) != n_in) throw std::invalid_argument("darknet shim: input size mismatch");
         auto x = packed_tensor(in, is);
+        model.inference(&x);                     // the second pass runs on recycled pool tensors
         auto outs = model.inference(&x);
         size_t at = 0;
         *n_heads = (int)outs.size();

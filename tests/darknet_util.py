@@ -11,6 +11,7 @@ from util import GOLDEN
 
 CFG = os.path.join(GOLDEN, "darknet", "yolov3-tiny.cfg")
 CFG_BUG = os.path.join(GOLDEN, "darknet", "yolov3-tiny_wbug.cfg")
+CFG_MINI = os.path.join(GOLDEN, "darknet", "mini_shortcut.cfg")      # written for these tests: shortcuts, routes, two heads
 
 
 def small_cfg(tmpdir, size, src=CFG):

@@ -43,6 +43,21 @@ def test_darknet_model(hip, oracle, tmp_path, size):
     assert_equal_exact(du.sorted_rows(det), du.sorted_rows(got_det), "detections")
 
 
+def test_darknet_shortcuts_and_routes(hip, oracle, tmp_path):
+    text = open(du.CFG_MINI).read()
+    weights = du.synthetic_weights(tmp_path, text, seed=900)
+    x = synth.uniform_f32(8, 3 * 64 * 64, 0.0, 1.0).reshape(1, 3, 64, 64)
+    got, _ = hip.run(du.CFG_MINI, weights, x)
+    want = od.Model(text, weights).inference(oracle, x)
+    assert [a.shape for a in got] == [w.shape for w in want] == [(1, 3 * 16 * 16, 7), (1, 2 * 32 * 32, 7)]
+    for a, w in zip(got, want):
+        assert_close_f32(a, w, atol=1e-5 * max(1.0, float(np.abs(w).max())), what="yolo head %s" % (w.shape,))
+    # a second pass recycles the pooled tensors and must reproduce the first
+    again, _ = hip.run(du.CFG_MINI, weights, x)
+    for a, b in zip(got, again):
+        assert_equal_exact(a, b, "second model instance")
+
+
 def test_unsupported_block_is_an_error(hip, tmp_path):
     cfg, _ = du.small_cfg(tmp_path, 96, du.CFG_BUG)
     weights = du.synthetic_weights(tmp_path, open(du.CFG).read())

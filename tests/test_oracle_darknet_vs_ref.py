@@ -54,6 +54,23 @@ def test_darknet_model(oracle, plat, tmp_path):
     assert_equal_exact(du.sorted_rows(det), du.sorted_rows(want_det), "detections")
 
 
+def test_darknet_shortcuts_and_routes(oracle, plat, tmp_path):
+    """A small residual network (tests/golden/darknet/mini_shortcut.cfg): [shortcut] accumulates into its first
+    parent's tensor in DAGModel, a layer output feeds two consumers, routes take one and two layers."""
+    name, ref = plat
+    text = open(du.CFG_MINI).read()
+    weights = du.synthetic_weights(tmp_path, text, seed=900)
+    x = synth.uniform_f32(8, 3 * 64 * 64, 0.0, 1.0).reshape(1, 3, 64, 64)
+    want, _ = ref.run(du.CFG_MINI, weights, x)
+    got = od.Model(text, weights).inference(oracle, x)
+    assert [g.shape for g in got] == [w.shape for w in want] == [(1, 3 * 16 * 16, 7), (1, 2 * 32 * 32, 7)]
+    for g, w in zip(got, want):
+        if name == "REF":
+            assert_equal_exact(g, w, "yolo head")
+        else:
+            assert_close_f32(g, w, atol=1e-5 * max(1.0, float(np.abs(w).max())), what="yolo head")
+
+
 def test_unsupported_block_is_an_error(oracle, ref_REF, tmp_path):
     cfg, text = du.small_cfg(tmp_path, 96, du.CFG_BUG)
     weights = du.synthetic_weights(tmp_path, open(du.CFG).read())
