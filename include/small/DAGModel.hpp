@@ -110,6 +110,25 @@ protected:
         m_cached.assign(this->m_layers.size(), nullptr);
     }
 
+    // Takes over a finished layer list as the graph's vertices 0..n-1 and initialises the DAG.  parents[i] lists
+    // the layers feeding layer i, in input order (for an accumulating layer: the tensor it adds onto first);
+    // an empty list means the previous layer, so an empty `parents` describes a plain chain.
+    void adopt_layers(std::vector<Layer<BufferT> *> layers, std::vector<std::vector<size_t>> const &parents = {})
+    {
+        size_t max_size = compute_size(this->m_input_shape);
+        for (size_t i = 0; i < layers.size(); ++i)
+        {
+            this->add(layers[i]);
+            max_size = std::max(max_size, layers[i]->output_size());
+            m_graph.add_vertex(i);
+            if (i < parents.size() && !parents[i].empty())
+                for (size_t p : parents[i]) m_graph.add_edge(p, i);
+            else if (i > 0)
+                m_graph.add_edge(i - 1, i);
+        }
+        initializeDAG(max_size);
+    }
+
     Graph m_graph;
 
 private:

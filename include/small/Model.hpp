@@ -35,6 +35,15 @@ public:
         return m_layers[idx];
     }
 
+    // hands the layers (and their ownership) to the caller and leaves the model empty; used to re-host a
+    // model's layer list in another executor (DAGModel::adopt_layers)
+    std::vector<Layer<BufferT> *> release_layers()
+    {
+        std::vector<Layer<BufferT> *> out;
+        out.swap(m_layers);
+        return out;
+    }
+
 protected:
     // takes ownership; returns the layer for chaining on its output_shape()
     Layer<BufferT> *add(Layer<BufferT> *layer)

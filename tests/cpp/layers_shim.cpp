@@ -27,6 +27,12 @@
 #include <small/SoftMaxLayer.hpp>
 #include <small/UpSample2DLayer.hpp>
 #include <small/models/AutoencoderTiny.hpp>
+#include <small/models/AutoencoderTinyDAG.hpp>
+#include <small/models/DSCNNSquareTinyDAG.hpp>
+#include <small/models/DSCNNTinyDAG.hpp>
+#include <small/models/MobileNetTinyDAG.hpp>
+#include <small/models/Resnet8TinyDAG.hpp>
+#include <small/models/TinyYoloV2DAG.hpp>
 #include <small/models/DSCNNSquareTiny.hpp>
 #include <small/models/DSCNNTiny.hpp>
 #include <small/models/Darknet.hpp>
@@ -254,9 +260,17 @@ int stest_model_f32(int which, int variant, int batch, int C, int H, int W, cons
                                 : new small::TinyYoloV2<FB>(is, fl, false)); break;
         case 4: m.reset(new small::AutoencoderTiny<FB>(is, 16, fl, false)); break;
         case 5: m.reset(new small::DSCNNSquareTiny<FB>(is, fl, false)); break;
+        // 10 + which: the same model on the DAG executor
+        case 10: m.reset(new small::MobileNetTinyDAG<FB>(is, fl, false)); break;
+        case 11: m.reset(new small::Resnet8TinyDAG<FB>(is, fl, false)); break;
+        case 12: m.reset(new small::DSCNNTinyDAG<FB>(is, fl, false)); break;
+        case 13: m.reset(new small::TinyYoloV2DAG<FB>(is, fl, false)); break;
+        case 14: m.reset(new small::AutoencoderTinyDAG<FB>(is, 16, fl, false)); break;
+        case 15: m.reset(new small::DSCNNSquareTinyDAG<FB>(is, fl, false)); break;
         default: throw std::invalid_argument("stest_model_f32: unknown model");
         }
         auto x = packed_tensor<FB>(in, is);
+        if (which >= 10) m->inference(&x);       // the second pass of a DAG model runs on recycled pool tensors
         auto outs = m->inference(&x);
         unpack_tensor<FB>(*outs[0], out, out_shape);
     });

@@ -120,6 +120,19 @@ def test_models(hip, oracle, name):
     assert_close_f32(one[0], got[1], atol=1e-5 * scale, what=name + " batch-1 vs batched")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["MobileNetTiny", "Resnet8Tiny", "DSCNNTiny", "TinyYoloV2", "AutoencoderTiny",
+                                  "DSCNNSquareTiny"])
+def test_dag_twins_equal_the_sequential_models(hip, name):
+    """<Model>DAG runs the same layers through DAGModel (pooled tensors, graph order, residual joins that
+    accumulate into the first parent's tensor): bit-identical to the sequential class."""
+    which, variant, fn, filters, shape = _model_case(name)
+    x = synth.normal(56, int(np.prod(shape))).reshape(shape)
+    seq = hip.model_f32(which, x, filters, 0)
+    dag = hip.model_f32(which + 10, x, filters, 0)
+    assert_equal_exact(dag, seq, name + "DAG")
+
+
 # ---- the reference-named two-layer ("fused") functions ---------------------------------------------------
 from test_oracle_fused_vs_ref import SINGLE_CASES, TWO_LAYER_CASES, two_layer_inputs
 
