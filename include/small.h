@@ -15,3 +15,4 @@
 #include "small/buffers.hpp"
 #include "small/interface.hpp"
 #include "small/interface_1D.hpp"
+#include "small/utils/Timer.hpp"

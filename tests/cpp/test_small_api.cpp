@@ -372,6 +372,12 @@ static void test_fused_conv_pool_dropout_softmax()
         small::Conv2D_Bias_ReLU_Maxpool2D(3, 3, 1, 1, 1, 1, 1, pk, pk, 2, 0, 0, 0, 0, Co, Ci, H, W, x, f, bias, inter, got);
         for (size_t i = 0; i < want.size(); ++i) CHECK(almost_equal(got[i], want[i], 1e-4f));
     }
+    // Timer brackets device work: a launch between start() and stop() shows up as a positive interval
+    small::Timer timer;
+    timer.start();
+    small::batched::Conv2D_Bias_Act(1, 3, 3, 1, 1, 1, 1, 1, Co, Ci, H, W, x, f, bias, small::RELU, 0.f, mid);
+    timer.stop();
+    CHECK(timer.elapsed() > 0.0 && timer.elapsed() < 5.0e9);
     // Dropout = multiplication by filter[0]; SoftMax sums to one over the whole tensor
     FloatBuffer rate(1), d(Ci * H * W), sm(Ci * H * W);
     rate[0] = 0.75f;
