@@ -66,7 +66,15 @@ public:
                 for (size_t p : parents) ins.push_back(m_cached[p]);
                 out = m_pool.pop_buffer();
             }
-            this->m_layers[cur]->compute_output(ins, out);
+            try
+            {
+                this->m_layers[cur]->compute_output(ins, out);
+            }
+            catch (...)
+            {
+                m_pool.push_buffer(out);     // nothing refers to it yet: back to the pool, then let the caller see the error
+                throw;
+            }
             // a parent's tensor returns to the pool after its last consumer; the stream orders the reuse
             if (step != 0)
                 for (size_t k = accumulates(cur) ? 1 : 0; k < parents.size(); ++k)
