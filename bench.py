@@ -125,6 +125,28 @@ def layer_table(model, batch, ms):
     return rows
 
 
+def mfma_probe_tflops(steps=5):
+    """Calibration: float32 MFMA instructions on registers only (small_hip_mfma_f32_probe), 8 workgroups per CU.
+    -> sustained TFLOP/s of the matrix pipes on this machine (to set beside the published 157.3)."""
+    import ctypes as C
+    import torch
+    from smallframework_amd import capi
+    lib = capi.load()
+    sink = torch.zeros(4, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    wgs, iters = 256 * 8, 20000
+    call = lambda: capi.check(lib.small_hip_mfma_f32_probe(wgs, iters, C.c_void_p(sink.data_ptr()), st))
+    call()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    torch.cuda.synchronize()
+    flops = steps * float(wgs) * 4 * iters * 4 * 4096
+    return flops / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+
 def library_gemm_ms(model, batch, steps, warmup):
     """Calibration, not part of the product path: the contraction of every MFMA-sized convolution as a plain
     float32 GEMM [Co x K] . [K x pixels] through torch.mm (the vendor BLAS; no im2col cost counted, TF32 off).
@@ -329,6 +351,7 @@ def main():
     ms = time_ops(ex, args.steps)
     table = layer_table(model, batch, ms)
     if args.library_gemm:
+        log("float32 MFMA on registers only: %.1f TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
         lib_ms = library_gemm_ms(model, batch, args.steps, args.warmup)
         for r in table:
             if r["layer"] in lib_ms:
@@ -376,6 +399,9 @@ def main():
 
     extras = {"per_kernel_ms": {k: round(v["ms"], 4) for k, v in per_kernel.items()},
               "sum_of_layer_ms": round(sum(ms), 4)}
+    if model.dtype == "f32":
+        # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
+        extras["mfma_f32_sustained_TFLOPs"] = round(mfma_probe_tflops(), 1)
     if not args.no_extras and args.model == "mobilenet_v1":
         for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
             m2 = getattr(models, name)()

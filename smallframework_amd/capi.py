@@ -70,6 +70,7 @@ SIGNATURES = {
     "small_hip_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_partial_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_upsample2d_f32": (_i, [_i] * 5 + [_p, _p, _p]),
+    "small_hip_mfma_f32_probe": (_i, [_i, _i, _p, _p]),
     "small_hip_upsample1d_f32": (_i, [_i] * 5 + [_p, _p, _p]),
     "small_hip_yolo_decode_f32": (_i, [_i] * 5 + [_p, _i, _i, _p, _p, _p]),
     "small_hip_concat": (_i, [_i, _u32, _u32, _u32, _u32, _p, _p, _p, _sz, _p]),
