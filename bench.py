@@ -147,6 +147,21 @@ def mfma_probe_tflops(steps=5):
     return flops / (e0.elapsed_time(e1) * 1e-3) / 1e12
 
 
+def hbm_copy_gbs(nbytes=822083584, steps=10):
+    """Calibration: a device-to-device copy of `nbytes` through the runtime (read + write counted), GB/s."""
+    import torch
+    x = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda").normal_()
+    y = torch.empty_like(x)
+    y.copy_(x)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        y.copy_(x)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * nbytes * steps / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+
 def library_gemm_ms(model, batch, steps, warmup):
     """Calibration, not part of the product path: the contraction of every MFMA-sized convolution as a plain
     float32 GEMM [Co x K] . [K x pixels] through torch.mm (the vendor BLAS; no im2col cost counted, TF32 off).
@@ -352,6 +367,7 @@ def main():
     table = layer_table(model, batch, ms)
     if args.library_gemm:
         log("float32 MFMA on registers only: %.1f TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
+        log("device-to-device copy of 822 MB: %.0f GB/s read + write (published peak 8000)" % hbm_copy_gbs())
         lib_ms = library_gemm_ms(model, batch, args.steps, args.warmup)
         for r in table:
             if r["layer"] in lib_ms:
@@ -402,6 +418,7 @@ def main():
     if model.dtype == "f32":
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         extras["mfma_f32_sustained_TFLOPs"] = round(mfma_probe_tflops(), 1)
+        extras["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
     if not args.no_extras and args.model == "mobilenet_v1":
         for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
             m2 = getattr(models, name)()
