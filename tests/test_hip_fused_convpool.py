@@ -59,6 +59,35 @@ def test_conv_pool_vs_oracle(lib, oracle, case):
     assert_close_f32(hu.host(do)[: want.size], want, what=str(case))
 
 
+def _random_cases(seed, n):
+    """Seeded random shapes: both kernels (first layers with 3x3 windows, 16-multiple inputs with any window), ragged
+    tiles, odd output extents (the pool drops the last row / column), many pixels (2x1 / 2x2 wave tiles)."""
+    import random
+    rng = random.Random(seed)
+    cases = []
+    while len(cases) < n:
+        first = rng.random() < 0.3
+        ci = rng.choice([1, 2, 3]) if first else CB * rng.choice([1, 2, 3, 4])
+        k = 3 if first else rng.choice([1, 3, 3, 5])
+        s = rng.choice([1, 1, 2])
+        co = CB * rng.choice([1, 2, 2, 4, 6, 8])
+        h, w = rng.randint(2, 45), rng.randint(2, 45)
+        pads = tuple(rng.randint(0, min(2, k - 1)) if k > 1 else 0 for _ in range(4))
+        batch = rng.choice([1, 2, 3, 9, 40])
+        if h + pads[0] + pads[1] < k or w + pads[2] + pads[3] < k:
+            continue
+        if batch * h * w * co * ci * k * k > 3e9:
+            continue
+        cases.append((batch, k, s, pads, co, ci, h, w, rng.random() < 0.5,
+                      rng.choice([capi.ACT_NONE, capi.ACT_RELU, capi.ACT_LEAKY])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(31, 36), ids=str)
+def test_conv_pool_random_shapes(lib, oracle, case):
+    test_conv_pool_vs_oracle(lib, oracle, case)
+
+
 def test_conv_pool_full_size_vs_unfused(lib):
     """Tiny-YOLOv2's pooled layers at batch 16: the fused launch against this library's two launches."""
     import torch
