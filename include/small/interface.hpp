@@ -183,8 +183,8 @@ void Conv2D_Accum_ReLU(int batch, int kernel_height, int kernel_width, int strid
 }
 
 // out = MaxPool2D(act(Conv2D(in, filter) + bias)) in one launch when the pooling window is 2x2 stride 2 without
-// padding (the pooling runs on the accumulators); any other window runs the two layers through
-// inter_output_buf.  bias_buf may be empty.
+// padding (the pooling runs on the accumulators) when the kernel's pixel tiles fill the map well; any other
+// window or a ragged map runs the two layers through inter_output_buf.  bias_buf may be empty.
 template <class BufferT, detail::if_float<BufferT> = true>
 void Conv2D_Bias_Act_Maxpool2D(int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride,
                                uint8_t conv_t_pad, uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad,
@@ -194,10 +194,21 @@ void Conv2D_Bias_Act_Maxpool2D(int batch, int conv_kernel_height, int conv_kerne
                                BufferT const &filter_buf, BufferT const &bias_buf, ActivationType act,
                                float negative_slope, BufferT &inter_output_buf, BufferT &output_buf)
 {
-    const bool fusable = pool_kernel_height == 2 && pool_kernel_width == 2 && pool_stride == 2 && !pool_t_pad &&
-                         !pool_b_pad && !pool_l_pad && !pool_r_pad &&
-                         (input_channels % (int)BufferT::C_ib == 0 || (conv_kernel_height == 3 && conv_kernel_width == 3)) &&
-                         !(act == LEAKY && negative_slope < 0.f);
+    bool fusable = pool_kernel_height == 2 && pool_kernel_width == 2 && pool_stride == 2 && !pool_t_pad &&
+                   !pool_b_pad && !pool_l_pad && !pool_r_pad &&
+                   (input_channels % (int)BufferT::C_ib == 0 || (conv_kernel_height == 3 && conv_kernel_width == 3)) &&
+                   !(act == LEAKY && negative_slope < 0.f);
+    if (fusable)
+    {
+        // the fused kernel works on 4 x 8 pixel tiles of one image (16 x 16 for first layers): on small maps the
+        // ragged tiles cost more than the saved pooling pass (measured: 26x26 loses, 52x52 wins): fuse from 90% fill
+        const long Hc = (long)output_dim(input_height + conv_t_pad + conv_b_pad, conv_stride, conv_kernel_height);
+        const long Wc = (long)output_dim(input_width + conv_l_pad + conv_r_pad, conv_stride, conv_kernel_width);
+        const bool first = input_channels % (int)BufferT::C_ib != 0;
+        const long th = first ? 16 : 4, tw = first ? 16 : 8;
+        const long slots = ((Hc + th - 1) / th * th) * ((Wc + tw - 1) / tw * tw);
+        fusable = Hc > 0 && Wc > 0 && 10 * Hc * Wc >= 9 * slots;
+    }
     if (fusable)
     {
         detail::raise<BufferT>(

@@ -358,7 +358,7 @@ static void test_fused_conv_pool_dropout_softmax()
     std::printf("fused convolution + pooling, dropout, softmax\n");
     // Conv2D_Bias_ReLU_Maxpool2D == Conv2D_Bias_Act, then MaxPool2D: 2x2 stride 2 (one launch) and 3x3 stride 2
     // (runs through the intermediate buffer)
-    const int Ci = 16, Co = 32, H = 12, W = 20;
+    const int Ci = 16, Co = 32, H = 12, W = 16;      // 4 x 8 pixel tiles fill this map: the 2x2 pool is fused
     FloatBuffer x(Ci * H * W), f(Co * Ci * 9), bias(Co), mid(Co * H * W), inter(Co * H * W);
     small::init(x, x.size());
     small::init(f, f.size());

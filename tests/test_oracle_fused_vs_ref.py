@@ -22,6 +22,8 @@ TWO_LAYER_CASES = [
     (3, 1, (1, 1, 1, 1), 2, 2, (0, 0, 0, 0), 16, 3, 12, 12),
     (1, 1, (0, 0, 0, 0), 3, 1, (1, 1, 1, 1), 48, 32, 13, 9),
     (3, 1, (1, 1, 1, 1), 2, 2, (0, 0, 0, 0), 16, 16, 13, 11),      # odd map: the pool drops the last row / column
+    (3, 1, (1, 1, 1, 1), 2, 2, (0, 0, 0, 0), 32, 16, 16, 24),      # whole 4 x 8 pixel tiles (one-launch path on the GPU)
+    (3, 1, (1, 1, 1, 1), 2, 2, (0, 0, 0, 0), 16, 3, 32, 32),       # first layer, whole 16 x 16 tiles
 ]
 
 
