@@ -295,6 +295,35 @@ public:
         output->set_shape(os);
     }
 
+    // This layer followed by a MaxPool2DLayer with window `pool` in one call (small::batched::
+    // Conv2D_Bias_Act_Maxpool2D: one launch for a 2x2 stride-2 un-padded pool on a map the kernel's tiles fill,
+    // else the two launches through `inter`).  float32, ReLU / LeakyReLU / no activation; the caller checks
+    // fusable_with_pool() first.  `pooled` receives the pooling layer's output shape.
+    bool fusable_with_pool() const
+    {
+        return std::is_same<BufferT, FloatBuffer>::value && m_activation_type != SOFTMAX;
+    }
+
+    void compute_output_pooled(Tensor<BufferT> const *input, detail::Window const &pool, shape_type const &pooled_shape,
+                               Tensor<BufferT> *inter, Tensor<BufferT> *pooled) const
+    {
+        if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        {
+            this->check_single_input("Conv2DLayer", {input}, m_input_shape, inter);
+            if (pooled->capacity() < compute_size(pooled_shape))
+                throw std::invalid_argument("Conv2DLayer::compute_output_pooled() ERROR: insufficient output buffer space.");
+            auto const &os = this->output_shape();
+            batched::Conv2D_Bias_Act_Maxpool2D(
+                (int)m_input_shape[BATCH], m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b, m_window.l,
+                m_window.r, pool.kh, pool.kw, pool.stride, pool.t, pool.b, pool.l, pool.r, (int)os[CHANNEL],
+                (int)m_input_shape[CHANNEL], (int)m_input_shape[HEIGHT], (int)m_input_shape[WIDTH], input->buffer(),
+                m_packed_filters, m_packed_bias, m_activation_type, m_slope, inter->buffer(), pooled->buffer());
+            pooled->set_shape(pooled_shape);
+        }
+        else
+            throw std::invalid_argument("Conv2DLayer::compute_output_pooled() ERROR: float32 only.");
+    }
+
 private:
     shape_type const m_input_shape;
     detail::Window const m_window;

@@ -34,6 +34,9 @@ public:
         output->set_shape(this->output_shape());
     }
 
+    // window geometry (kernel, stride, pads from the padding type)
+    detail::Window const &window() const { return m_window; }
+
 private:
     shape_type const m_input_shape;
     detail::Window const m_window;

@@ -57,21 +57,36 @@ public:
         cap0 = std::max(cap0, cap1);   // the tail swaps the two tensors
         m_buffer_0.reset(new Tensor<BufferT>(cap0));
         m_buffer_1.reset(new Tensor<BufferT>(cap0));
+        m_buffer_2.reset(new Tensor<BufferT>(cap0));
     }
 
     virtual ~TinyYoloV2() {}
 
     virtual std::vector<Tensor<BufferT> *> inference(Tensor<BufferT> const *input_tensor)
     {
-        Tensor<BufferT> *a = m_buffer_0.get(), *b = m_buffer_1.get();
+        // b takes convolution outputs; the pooled maps alternate between a and c, so that the one-launch
+        // convolution + pooling never writes over its own input
+        Tensor<BufferT> *a = m_buffer_0.get(), *b = m_buffer_1.get(), *c = m_buffer_2.get();
         size_t l = 0;
         Tensor<BufferT> const *src = input_tensor;
         for (int blk = 0; blk < 6; ++blk)
         {
-            this->m_layers[l++]->compute_output({src}, b);   // convolution + activation
-            this->m_layers[l++]->compute_output({b}, a);     // pooling
+            // convolution + activation + pooling: one call (one launch where the pool is 2x2 stride 2 on a map the
+            // kernel's tiles fill; the wrapper falls back to the two launches through b otherwise)
+            auto *conv = static_cast<Conv2DLayer<BufferT> *>(this->m_layers[l]);
+            auto *pool = static_cast<MaxPool2DLayer<BufferT> *>(this->m_layers[l + 1]);
+            if (conv->fusable_with_pool())
+                conv->compute_output_pooled(src, pool->window(), pool->output_shape(), b, a);
+            else
+            {
+                conv->compute_output({src}, b);
+                pool->compute_output({b}, a);
+            }
+            l += 2;
             src = a;
+            std::swap(a, c);          // the next block reads what was just written (now c) and writes the other one
         }
+        std::swap(a, c);              // a = the last pooled map
         for (int tail = 0; tail < 3; ++tail)
         {
             this->m_layers[l++]->compute_output({a}, b);
@@ -81,7 +96,7 @@ public:
     }
 
 private:
-    std::unique_ptr<Tensor<BufferT>> m_buffer_0, m_buffer_1;
+    std::unique_ptr<Tensor<BufferT>> m_buffer_0, m_buffer_1, m_buffer_2;
 };
 
 } // namespace small

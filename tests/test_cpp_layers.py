@@ -125,12 +125,18 @@ def test_models(hip, oracle, name):
                                   "DSCNNSquareTiny"])
 def test_dag_twins_equal_the_sequential_models(hip, name):
     """<Model>DAG runs the same layers through DAGModel (pooled tensors, graph order, residual joins that
-    accumulate into the first parent's tensor): bit-identical to the sequential class."""
+    accumulate into the first parent's tensor): bit-identical to the sequential class where both issue the same
+    launches."""
     which, variant, fn, filters, shape = _model_case(name)
     x = synth.normal(56, int(np.prod(shape))).reshape(shape)
     seq = hip.model_f32(which, x, filters, 0)
     dag = hip.model_f32(which + 10, x, filters, 0)
-    assert_equal_exact(dag, seq, name + "DAG")
+    if name == "TinyYoloV2":
+        # the sequential class runs convolution + pooling pairs as one launch, the DAG executor layer by layer:
+        # another kernel variant, another (fixed) summation order in the last tiles
+        assert_close_f32(dag, seq, atol=1e-5 * max(1.0, float(np.abs(seq).max())), what=name + "DAG")
+    else:
+        assert_equal_exact(dag, seq, name + "DAG")
 
 
 # ---- the reference-named two-layer ("fused") functions ---------------------------------------------------
@@ -272,3 +278,10 @@ def test_model_class_throughput(hip):
     print("MobileNetTiny<FloatBuffer> (MobileNetV1 224x224, 1000 classes) batch 64: %.3f ms per inference, %.0f images/s"
           % (ms, 64 / ms * 1e3))
     assert ms < 2.2
+    # TinyYoloV2<FloatBuffer> as Tiny-YOLOv2 (416x416, LeakyReLU, 125 outputs) at batch 16: the class fuses its
+    # convolution + pooling pairs like the benchmark's executor (recorded: ~1.2 ms)
+    sizes = [int(np.prod(f.shape)) for f in ol.make_filters(synth, ol.yolo_specs(), 125)]
+    ms = hip.model_time_f32(3, 1, (16, 3, 416, 416), sizes)
+    print("TinyYoloV2<FloatBuffer> (416x416, LeakyReLU, 125 outputs) batch 16: %.3f ms per inference, %.0f images/s"
+          % (ms, 16 / ms * 1e3))
+    assert ms < 2.6
