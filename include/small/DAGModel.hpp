@@ -3,6 +3,7 @@
 // run in topological order, each output lives in a pooled tensor until its last consumer has run, and a layer
 // that accumulates (AddLayer, PartialConv2DLayer) writes into the tensor of its FIRST parent, which must have
 // no other consumer.  With save_outputs every layer's output stays readable until the next inference().
+// A float32 convolution whose only consumer is a max-pooling layer runs together with it (not with save_outputs).
 #pragma once
 
 #include <deque>
@@ -10,6 +11,8 @@
 #include <vector>
 
 #include "AddLayer.hpp"
+#include "Conv2DLayer.hpp"
+#include "MaxPool2DLayer.hpp"
 #include "Model.hpp"
 #include "PartialConv2DLayer.hpp"
 #include "utils/BufferPool.hpp"
@@ -66,6 +69,34 @@ public:
                 for (size_t p : parents) ins.push_back(m_cached[p]);
                 out = m_pool.pop_buffer();
             }
+            if (!m_save_outputs && m_pool_after[cur] != NO_POOL && step + 1 < m_order.size() &&
+                m_order[step + 1] == m_pool_after[cur])
+            {
+                // convolution whose only consumer is a max-pooling layer: both in one call (one launch for a 2x2
+                // stride-2 pool on a map the kernel's tiles fill); the convolution's own output is never cached
+                const size_t pl = m_pool_after[cur];
+                auto *conv = static_cast<Conv2DLayer<BufferT> *>(this->m_layers[cur]);
+                auto *pool = static_cast<MaxPool2DLayer<BufferT> *>(this->m_layers[pl]);
+                Tensor<BufferT> *inter = m_pool.pop_buffer();
+                try
+                {
+                    conv->compute_output_pooled(ins[0], pool->window(), pool->output_shape(), inter, out);
+                }
+                catch (...)
+                {
+                    m_pool.push_buffer(inter);
+                    m_pool.push_buffer(out);
+                    throw;
+                }
+                m_pool.push_buffer(inter);
+                if (step != 0)
+                    for (size_t k = 0; k < parents.size(); ++k)
+                        if (m_count[parents[k]] > 0 && --m_count[parents[k]] == 0) release(parents[k]);
+                m_count[pl] = m_graph.out_neighbors(pl).size();
+                m_cached[pl] = out;
+                ++step;                  // the pooling layer has run
+                continue;
+            }
             try
             {
                 this->m_layers[cur]->compute_output(ins, out);
@@ -116,6 +147,17 @@ protected:
         m_pool = BufferPool<BufferT>(max_buffer_size, num_bufs);
         m_count.assign(this->m_layers.size(), 0);
         m_cached.assign(this->m_layers.size(), nullptr);
+        // convolution -> max-pool pairs that can run as one call: the pool is the convolution's only consumer
+        // and the convolution the pool's only input
+        m_pool_after.assign(this->m_layers.size(), NO_POOL);
+        for (size_t i = 0; i < this->m_layers.size(); ++i)
+        {
+            auto *conv = dynamic_cast<Conv2DLayer<BufferT> *>(this->m_layers[i]);
+            auto const &outs = m_graph.out_neighbors(i);
+            if (!conv || !conv->fusable_with_pool() || outs.size() != 1) continue;
+            if (dynamic_cast<MaxPool2DLayer<BufferT> *>(this->m_layers[outs[0]]) && m_graph.in_neighbors(outs[0]).size() == 1)
+                m_pool_after[i] = outs[0];
+        }
     }
 
     // Takes over a finished layer list as the graph's vertices 0..n-1 and initialises the DAG.  parents[i] lists
@@ -153,7 +195,10 @@ private:
         m_count[idx] = 0;
     }
 
+    static constexpr size_t NO_POOL = (size_t)-1;
+
     bool m_save_outputs;
+    std::vector<size_t> m_pool_after;          // per layer: the max-pooling layer fused behind it, or NO_POOL
     std::deque<size_t> m_order;
     BufferPool<BufferT> m_pool;
     std::vector<size_t> m_count;
