@@ -7,6 +7,9 @@
 // and no vertical padding.  The 2-D kernels stride both axes alike, so more than one row is accepted with
 // stride 1 only (any stride when rows == 1); other combinations raise std::invalid_argument.
 // small::batched::<Fn>(batch, ...) takes `batch` such tensors back to back.
+// The QUInt8Buffer forms (Conv1D, MaxPool1D, ReLUActivation1D) are the quantised 2-D functions on the same
+// 1 x kernel_width window; the reference's own quantised 1-D functions write unrelated bytes on its scalar build
+// (its only quantised platform), so there is nothing to compare them with.
 #pragma once
 
 #include "interface.hpp"
