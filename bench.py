@@ -419,6 +419,18 @@ def main():
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         extras["mfma_f32_sustained_TFLOPs"] = round(mfma_probe_tflops(), 1)
         extras["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
+        # the same forward pass replayed from a HIP graph (no host work between the launches)
+        ex.capture()
+        for _ in range(args.warmup):
+            ex.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            ex.replay()
+        torch.cuda.synchronize()
+        sg = (time.perf_counter() - t0) / args.steps
+        extras["hip_graph_ms_per_step"] = round(sg * 1e3, 4)
+        log("%s: HIP graph replay %.3f ms/step (eager %.3f)" % (model.name, sg * 1e3, sec * 1e3))
     if not args.no_extras and args.model == "mobilenet_v1":
         for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
             m2 = getattr(models, name)()
