@@ -1048,7 +1048,9 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
     else if (Co % 64 == 0 && (tiles32 >= 4 * simds || (tiles32 >= 2 * simds && nsteps >= 128))) { cot = 2; pxt = 1; }
     // few tiles and a long reduction: split K over the four waves of a workgroup
-    bool splitk = tiles32 < 2 * simds && nsteps >= 16;
+    // (measured: from one tile per SIMD the whole-rounds + tail kernel with 1x1 wave tiles is ahead, e.g. 256->512 3x3
+    // @13x13 batch 16, 1360 tiles: 81 us against 91 us)
+    bool splitk = tiles32 < simds && nsteps >= 16;
     if (const char *e = std::getenv("SMALL_HIP_CONV_SPLITK")) splitk = e[0] == '1';
     if (splitk)
     {
