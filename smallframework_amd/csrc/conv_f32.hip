@@ -1039,14 +1039,14 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
 
     // Wave tile (in 32-channel x 32-pixel MFMA tiles).  Measured on MI355X inside whole-model runs with
     // the balanced tail in place: 2x2 only pays with many tiles per SIMD and a long reduction (big
-    // 3x3 layers), 2x1 from 4 tiles per SIMD (from 2 when the reduction has at least 128 steps), 1x1 below (few tiles: balance matters more than
+    // 3x3 layers), 2x1 from 4 tiles per SIMD (from 2 when the reduction has at least 72 steps: 128->256 3x3 @26x26 b16, 2.6 tiles per SIMD, 74 -> 69 us; 1024->1024 1x1 @7x7 b64 with 64 steps stays 1x1: 69 against 73 us), 1x1 below (few tiles: balance matters more than
     // operand re-use).
     const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32);
     const long simds = 4L * NUM_CU;
     const int nsteps = kh * kw * (Ci / CB);
     int cot = 1, pxt = 1;
     if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
-    else if (Co % 64 == 0 && (tiles32 >= 4 * simds || (tiles32 >= 2 * simds && nsteps >= 128))) { cot = 2; pxt = 1; }
+    else if (Co % 64 == 0 && (tiles32 >= 4 * simds || (tiles32 >= 2 * simds && nsteps >= 72))) { cot = 2; pxt = 1; }
     // few tiles and a long reduction: split K over the four waves of a workgroup
     // (measured: from one tile per SIMD the whole-rounds + tail kernel with 1x1 wave tiles is ahead, e.g. 256->512 3x3
     // @13x13 batch 16, 1360 tiles: 81 us against 91 us)
