@@ -415,7 +415,7 @@ def main():
 
     extras = {"per_kernel_ms": {k: round(v["ms"], 4) for k, v in per_kernel.items()},
               "sum_of_layer_ms": round(sum(ms), 4)}
-    if model.dtype == "f32":
+    if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         extras["mfma_f32_sustained_TFLOPs"] = round(mfma_probe_tflops(), 1)
         extras["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
