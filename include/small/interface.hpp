@@ -119,6 +119,48 @@ void PartialConv2D(int batch, int kernel_height, int kernel_width, int stride, u
                            "PartialConv2D");
 }
 
+// ---- GroupConv2D / PartialGroupConv2D (interface_abstract.hpp:1265-1533) ---------------------------------
+// `output_groups` convolutions of input_channels -> input_channels, one per slab of input_channels channels
+// of the packed tensors; filter_buf holds one packed Conv2D filter per group, group after group.
+template <class BufferT, detail::if_float<BufferT> = true>
+void GroupConv2D(int batch, int kernel_height, int kernel_width, int stride, int output_groups, uint8_t t_pad,
+                 uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height,
+                 int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_group_conv2d_f32(batch, kernel_height, kernel_width, stride, output_groups,
+                                                      t_pad, b_pad, l_pad, r_pad, input_channels, input_height,
+                                                      input_width, input_buf.device_in(), filter_buf.device_in(),
+                                                      0, output_buf.device_out(), detail::st()),
+                           "GroupConv2D");
+}
+
+template <class BufferT, detail::if_quint8<BufferT> = true>
+void GroupConv2D(int batch, int kernel_height, int kernel_width, int stride, int output_groups, uint8_t t_pad,
+                 uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height,
+                 int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    const small_hip_quant iq = input_buf.quant(), fq = filter_buf.quant(), oq = output_buf.quant();
+    detail::raise<BufferT>(small_hip_group_conv2d_u8(batch, kernel_height, kernel_width, stride, output_groups,
+                                                     t_pad, b_pad, l_pad, r_pad, input_channels, input_height,
+                                                     input_width, input_buf.device_in(), &iq,
+                                                     filter_buf.device_in(), &fq, output_buf.device_out(), &oq,
+                                                     detail::st()),
+                           "GroupConv2D");
+}
+
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialGroupConv2D(int batch, int kernel_height, int kernel_width, int stride, int output_groups,
+                        uint8_t t_pad, uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels,
+                        int input_height, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                        BufferT &output_buf)
+{
+    detail::raise<BufferT>(small_hip_group_conv2d_f32(batch, kernel_height, kernel_width, stride, output_groups,
+                                                      t_pad, b_pad, l_pad, r_pad, input_channels, input_height,
+                                                      input_width, input_buf.device_in(), filter_buf.device_in(),
+                                                      1, output_buf.device_out(), detail::st()),
+                           "PartialGroupConv2D");
+}
+
 // bias_buf may be empty (size 0): no bias
 template <class BufferT, detail::if_float<BufferT> = true>
 void Conv2D_Bias_Act(int batch, int kernel_height, int kernel_width, int stride, uint8_t t_pad, uint8_t b_pad,
@@ -524,6 +566,24 @@ void PartialConv2D(int kernel_height, int kernel_width, int stride, uint8_t t_pa
 {
     batched::PartialConv2D(1, kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad, output_channels,
                            input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void GroupConv2D(int kernel_height, int kernel_width, int stride, int output_groups, uint8_t t_pad, uint8_t b_pad,
+                 uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height, int input_width,
+                 BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::GroupConv2D(1, kernel_height, kernel_width, stride, output_groups, t_pad, b_pad, l_pad, r_pad,
+                         input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialGroupConv2D(int kernel_height, int kernel_width, int stride, int output_groups, uint8_t t_pad,
+                        uint8_t b_pad, uint8_t l_pad, uint8_t r_pad, int input_channels, int input_height,
+                        int input_width, BufferT const &input_buf, BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::PartialGroupConv2D(1, kernel_height, kernel_width, stride, output_groups, t_pad, b_pad, l_pad, r_pad,
+                                input_channels, input_height, input_width, input_buf, filter_buf, output_buf);
 }
 
 template <class BufferT>

@@ -62,6 +62,40 @@ void PartialConv1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8
     }
 }
 
+// interface_abstract_1D.hpp:1255 (float), :1320 (quint8): output_groups convolutions of input_channels -> input_channels,
+// one per slab of input_channels channels
+template <class BufferT>
+void GroupConv1D(int batch, int kernel_width, int stride, int output_groups, uint8_t l_pad, uint8_t r_pad,
+                 int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                 BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("GroupConv1D", stride, batch_size);
+    try
+    {
+        GroupConv2D(batch, 1, kernel_width, stride, output_groups, 0, 0, l_pad, r_pad, input_channels, batch_size,
+                    input_width, input_buf, filter_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e) { throw std::invalid_argument(detail::rename_op(e.what(), "GroupConv2D", "GroupConv1D")); }
+}
+
+// interface_abstract_1D.hpp:1388
+template <class BufferT, detail::if_float<BufferT> = true>
+void PartialGroupConv1D(int batch, int kernel_width, int stride, int output_groups, uint8_t l_pad, uint8_t r_pad,
+                        int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                        BufferT const &filter_buf, BufferT &output_buf)
+{
+    detail::check_rows<BufferT>("PartialGroupConv1D", stride, batch_size);
+    try
+    {
+        PartialGroupConv2D(batch, 1, kernel_width, stride, output_groups, 0, 0, l_pad, r_pad, input_channels,
+                           batch_size, input_width, input_buf, filter_buf, output_buf);
+    }
+    catch (std::invalid_argument const &e)
+    {
+        throw std::invalid_argument(detail::rename_op(e.what(), "PartialGroupConv2D", "PartialGroupConv1D"));
+    }
+}
+
 // bias + convolution + activation in one launch (Conv1D_ReLU / Conv1D_Bias_ReLU, fused_interface_abstract_1D.hpp:55, 216,
 // and what Conv1DLayer::compute_output issues as three calls); bias_buf may be empty
 template <class BufferT, detail::if_float<BufferT> = true>
@@ -141,6 +175,24 @@ void PartialConv1D(int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, i
 {
     batched::PartialConv1D(1, kernel_width, stride, l_pad, r_pad, output_channels, input_channels, batch_size,
                            input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void GroupConv1D(int kernel_width, int stride, int output_groups, uint8_t l_pad, uint8_t r_pad, int input_channels,
+                 int batch_size, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
+                 BufferT &output_buf)
+{
+    batched::GroupConv1D(1, kernel_width, stride, output_groups, l_pad, r_pad, input_channels, batch_size,
+                         input_width, input_buf, filter_buf, output_buf);
+}
+
+template <class BufferT>
+void PartialGroupConv1D(int kernel_width, int stride, int output_groups, uint8_t l_pad, uint8_t r_pad,
+                        int input_channels, int batch_size, int input_width, BufferT const &input_buf,
+                        BufferT const &filter_buf, BufferT &output_buf)
+{
+    batched::PartialGroupConv1D(1, kernel_width, stride, output_groups, l_pad, r_pad, input_channels, batch_size,
+                                input_width, input_buf, filter_buf, output_buf);
 }
 
 template <class BufferT>

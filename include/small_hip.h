@@ -214,6 +214,25 @@ int small_hip_concat(int batch, uint32_t input0_channels, uint32_t input1_channe
                      uint32_t input_height, uint32_t input_width, const void *input0,
                      const void *input1, void *output, size_t element_size,
                      small_hip_stream_t stream);
+/* small::GroupConv2D<FloatBuffer> / small::PartialGroupConv2D<FloatBuffer>
+ *                                      interface_abstract.hpp:1265-1328, 1402-1466
+ * `groups` convolutions of `channels` -> `channels`: group g reads channels [g*channels, (g+1)*channels) of
+ * the packed input, writes the same channels of the packed output and uses filter block g, each block a
+ * packed Conv2D filter of channels x channels (the reference's layout on its scalar platform, where every
+ * block is one element; its blocked platforms interleave 16 groups per block and feed every lane the first
+ * group's input, which no caller or test of the reference relies on).  `channels` must be a multiple of 16
+ * (SMALL_HIP_ECHANNELS), stride 1 or 2 (SMALL_HIP_ESTRIDE).  accumulate != 0 is the Partial form (adds into
+ * the output).  One launch per image and group. */
+int small_hip_group_conv2d_f32(int batch, int kernel_height, int kernel_width, int stride, int groups,
+                               int t_pad, int b_pad, int l_pad, int r_pad, int channels, int input_height,
+                               int input_width, const float *input, const float *filter, int accumulate,
+                               float *output, small_hip_stream_t stream);
+/* small::GroupConv2D<QUInt8Buffer>     interface_abstract.hpp:1332-1395 */
+int small_hip_group_conv2d_u8(int batch, int kernel_height, int kernel_width, int stride, int groups,
+                              int t_pad, int b_pad, int l_pad, int r_pad, int channels, int input_height,
+                              int input_width, const uint8_t *input, const small_hip_quant *input_q,
+                              const uint8_t *filter, const small_hip_quant *filter_q, uint8_t *output,
+                              const small_hip_quant *output_q, small_hip_stream_t stream);
 /* Fully connected layer y = W x, i.e. Conv2D(1,1,1,0,0,0,0,No,Ni,1,1,...) on a 1x1 image, the way
  * every reference model spells it (include/small/models/MobileNetTiny.hpp:531-538).  The
  * reference's own small::Dense (interface_abstract.hpp:2113-2132) is a per-channel scale with no

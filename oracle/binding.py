@@ -122,6 +122,44 @@ class Oracle:
                                     _p(f), _p(out), accumulate, acc64)
         return rc, out
 
+    def group_conv2d_f32(self, batch, cb, kh, kw, s, pt, pb, pl, pr, G, Cg, H, W, x, f, out=None,
+                         accumulate=0):
+        """small::GroupConv2D / PartialGroupConv2D (interface_abstract.hpp:1265-1328, 1402-1466;
+        layout comment abstract_layer.hpp:1420-1434): group g is a convolution of Cg -> Cg channels on
+        channels [g*Cg, (g+1)*Cg) with filter block g.  With Cg a multiple of cb the slab of one group
+        is contiguous in the packed tensors, so each group is one packed Conv2D."""
+        assert Cg % cb == 0
+        Ho, Wo = self.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
+        if out is None:
+            out = np.zeros(batch * G * Cg * Ho * Wo, np.float32)
+        si, so, sf = Cg * H * W, Cg * Ho * Wo, Cg * Cg * kh * kw
+        for i in range(batch * G):
+            g = i % G
+            o = np.ascontiguousarray(out[i * so:(i + 1) * so])
+            rc, o = self.conv2d_f32(1, cb, kh, kw, s, pt, pb, pl, pr, Cg, Cg, H, W,
+                                    np.ascontiguousarray(x[i * si:(i + 1) * si]),
+                                    np.ascontiguousarray(f[g * sf:(g + 1) * sf]), out=o, accumulate=accumulate)
+            if rc:
+                return rc, out
+            out[i * so:(i + 1) * so] = o
+        return 0, out
+
+    def group_conv2d_u8(self, batch, cb, kh, kw, s, pt, pb, pl, pr, G, Cg, H, W, x, iq, f, fq, oq):
+        """small::GroupConv2D<QUInt8Buffer> (interface_abstract.hpp:1332-1395), group by group."""
+        assert Cg % cb == 0
+        Ho, Wo = self.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
+        out = np.zeros(batch * G * Cg * Ho * Wo, np.uint8)
+        si, so, sf = Cg * H * W, Cg * Ho * Wo, Cg * Cg * kh * kw
+        for i in range(batch * G):
+            g = i % G
+            rc, o = self.conv2d_u8(1, cb, kh, kw, s, pt, pb, pl, pr, Cg, Cg, H, W,
+                                   np.ascontiguousarray(x[i * si:(i + 1) * si]), iq,
+                                   np.ascontiguousarray(f[g * sf:(g + 1) * sf]), fq, oq)
+            if rc:
+                return rc, out
+            out[i * so:(i + 1) * so] = o
+        return 0, out
+
     def conv2d_bias_act_f32(self, batch, cb, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, f, bias,
                             act, slope):
         Ho, Wo = self.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
@@ -323,6 +361,8 @@ class RefLib:
             L.sref_conv2d_f32.argtypes = conv
             L.sref_partial_conv2d_f32.argtypes = conv
             L.sref_dwconv2d_f32.argtypes = win3
+            if hasattr(L, "sref_group_conv2d_f32"):
+                L.sref_group_conv2d_f32.argtypes = [c_int] * 12 + [c_vp] * 3
             L.sref_partial_dwconv2d_f32.argtypes = win3
             L.sref_maxpool2d_f32.argtypes = win2
             L.sref_avgpool2d_f32.argtypes = win2
@@ -350,6 +390,8 @@ class RefLib:
             L.sref_qbuf_get_quant.argtypes = [c_vp, c_vp, c_vp]
             L.sref_conv2d_u8.argtypes = conv
             L.sref_dwconv2d_u8.argtypes = win3
+            if hasattr(L, "sref_group_conv2d_u8"):
+                L.sref_group_conv2d_u8.argtypes = [c_int] * 11 + [c_vp] * 3
             L.sref_maxpool2d_u8.argtypes = win2
             L.sref_relu_u8.argtypes = [c_int] * 3 + [c_vp] * 2
             L.sref_concat_u8.argtypes = [C.c_uint32] * 4 + [c_vp] * 3

@@ -394,8 +394,18 @@ def fused_two_layers_f32(oracle, batch, cb, second, variant, ck, cs, cpads, k2, 
 # ---- 1-D functions (packed arrays [C/cb][rows][W][cb]; rows = the reference's batch_size argument) --------------
 def one_d_f32(oracle, kind, cb, k, s, l, r, Co, Ci, rows, W, x, f=None, out_init=None):
     """interface_abstract_1D.hpp: kind 0 Conv1D (:47), 1 PartialConv1D (:415), 2 MaxPool1D (:776), 3 AveragePool1D
-    (:906), 4 ReLUActivation1D (:1526), 5 UpSample1D (:1614, k = scale).  Every row is an independent signal: the 2-D
+    (:906), 4 ReLUActivation1D (:1526), 5 UpSample1D (:1614, k = scale), 6 GroupConv1D, 7 PartialGroupConv1D (Co = groups,
+    Ci = channels per group).  Every row is an independent signal: the 2-D
     function with a 1 x k window on that row alone."""
+    if kind in (6, 7):
+        # GroupConv1D (:1255) / PartialGroupConv1D (:1388): Co groups, each a Conv1D of Ci -> Ci on its slab of Ci channels
+        G, Wo = Co, 1 + (W + l + r - k) // s
+        si, so, sf = Ci * rows * W, Ci * rows * Wo, Ci * Ci * k
+        x, f = np.asarray(x, np.float32), np.asarray(f, np.float32)
+        return np.concatenate([
+            one_d_f32(oracle, kind - 6, cb, k, s, l, r, Ci, Ci, rows, W, x[g * si:(g + 1) * si], f[g * sf:(g + 1) * sf],
+                      None if out_init is None else np.asarray(out_init, np.float32)[g * so:(g + 1) * so])
+            for g in range(G)])
     if kind == 5:
         rc, y = oracle.upsample1d_f32(1, cb, k, Ci, rows, W, x)
         assert rc == 0

@@ -149,6 +149,15 @@ int sref_partial_conv2d_f32(int kh, int kw, int s, int t, int b, int l, int r,
     return guarded([&] { small::PartialConv2D(kh, kw, s, t, b, l, r, Co, Ci, H, W,
                                               F(in), F(filt), F(out)); });
 }
+// small::GroupConv2D / small::PartialGroupConv2D (interface_abstract.hpp:1265-1533); C = channels per group
+int sref_group_conv2d_f32(int partial, int kh, int kw, int s, int G, int t, int b, int l, int r,
+                          int C, int H, int W, void *in, void *filt, void *out)
+{
+    return guarded([&] {
+        if (partial) small::PartialGroupConv2D(kh, kw, s, G, t, b, l, r, C, H, W, F(in), F(filt), F(out));
+        else small::GroupConv2D(kh, kw, s, G, t, b, l, r, C, H, W, F(in), F(filt), F(out));
+    });
+}
 int sref_dwconv2d_f32(int kh, int kw, int s, int t, int b, int l, int r,
                       int C, int H, int W, void *in, void *filt, void *out)
 {
@@ -214,7 +223,8 @@ int sref_dense_f32(int No, int Ni, void *in, void *filt, void *out)
 }
 
 // ---- 1-D functions, include/small/interface_abstract_1D.hpp (rows = their batch_size argument) -----------------
-// kind 0 Conv1D, 1 PartialConv1D, 2 MaxPool1D, 3 AveragePool1D, 4 ReLUActivation1D, 5 UpSample1D (k = scale)
+// kind 0 Conv1D, 1 PartialConv1D, 2 MaxPool1D, 3 AveragePool1D, 4 ReLUActivation1D, 5 UpSample1D (k = scale),
+// 6 GroupConv1D, 7 PartialGroupConv1D (Co = groups, Ci = channels per group)
 int sref_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows, int W, void *in, void *filt, void *out)
 {
     return guarded([&] {
@@ -225,6 +235,8 @@ int sref_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows, 
         case 2: small::MaxPool1D(k, s, l, r, Ci, rows, W, F(in), F(out)); break;
         case 3: small::AveragePool1D(k, s, l, r, Ci, rows, W, F(in), F(out)); break;
         case 4: small::ReLUActivation1D(Ci, rows, W, F(in), F(out)); break;
+        case 6: small::GroupConv1D(k, s, Co, l, r, Ci, rows, W, F(in), F(filt), F(out)); break;        // Co = groups
+        case 7: small::PartialGroupConv1D(k, s, Co, l, r, Ci, rows, W, F(in), F(filt), F(out)); break;
         default: small::UpSample1D(k, Ci, rows, W, F(in), F(out)); break;
         }
     });
@@ -307,6 +319,11 @@ int sref_conv2d_u8(int kh, int kw, int s, int t, int b, int l, int r,
 {
     return guarded([&] { small::Conv2D(kh, kw, s, t, b, l, r, Co, Ci, H, W,
                                        Q(in), Q(filt), Q(out)); });
+}
+int sref_group_conv2d_u8(int kh, int kw, int s, int G, int t, int b, int l, int r,
+                         int C, int H, int W, void *in, void *filt, void *out)
+{
+    return guarded([&] { small::GroupConv2D(kh, kw, s, G, t, b, l, r, C, H, W, Q(in), Q(filt), Q(out)); });
 }
 int sref_dwconv2d_u8(int kh, int kw, int s, int t, int b, int l, int r,
                      int C, int H, int W, void *in, void *filt, void *out)

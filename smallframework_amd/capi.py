@@ -74,6 +74,8 @@ SIGNATURES = {
     "small_hip_upsample1d_f32": (_i, [_i] * 5 + [_p, _p, _p]),
     "small_hip_yolo_decode_f32": (_i, [_i] * 5 + [_p, _i, _i, _p, _p, _p]),
     "small_hip_concat": (_i, [_i, _u32, _u32, _u32, _u32, _p, _p, _p, _sz, _p]),
+    "small_hip_group_conv2d_f32": (_i, [_i] * 12 + [_p, _p, _i, _p, _p]),
+    "small_hip_group_conv2d_u8": (_i, [_i] * 12 + [_p, _q, _p, _q, _p, _q, _p]),
     "small_hip_dense_f32": (_i, [_i] * 3 + [_p, _p, _p, _p]),
     "small_hip_dense_literal_f32": (_i, [_i] * 2 + [_p, _p, _p, _p]),
     "small_hip_conv2d_u8": (_i, _conv + [_p, _q, _p, _q, _p, _q, _p]),

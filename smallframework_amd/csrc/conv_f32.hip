@@ -1198,6 +1198,37 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kh, int kw, int strid
                          pool_kw, pool_stride, ppt, ppb, ppl, ppr, Co, Ci, H, W, in, filt, bias, act, slope, out, stream);
 }
 
+// One convolution of `channels` -> `channels` per slab of `channels` channels; slab g of image n starts
+// (n * groups + g) * channels * H * W elements into the input (the same with Ho * Wo into the output) and
+// uses filter block g.  One launch per slab: the kernels index images densely, and slabs of one group are
+// `groups` slabs apart.
+int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
+                               int channels, int H, int W, const float *in, const float *filt, int accumulate,
+                               float *out, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_group_conv2d_f32";
+    if (channels <= 0 || channels % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || groups <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out) { set_error("%s: null pointer", op); return SMALL_HIP_EINVAL; }
+    const size_t in_slab = (size_t)channels * H * W;
+    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    const size_t filt_slab = (size_t)channels * channels * kh * kw;
+    const size_t slabs = (size_t)batch * groups;
+    // the slabs written must not overlap the slabs read (one slab's launch would read another's output)
+    if (in + slabs * in_slab > out && out + slabs * out_slab > in)
+    { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    for (size_t i = 0; i < slabs; ++i)
+    {
+        const int rc = conv_f32(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab,
+                                filt + (i % groups) * filt_slab, nullptr, SMALL_HIP_ACT_NONE, 0.f, accumulate ? 1 : 0,
+                                out + i * out_slab, stream);
+        if (rc != SMALL_HIP_OK) return rc;
+    }
+    return SMALL_HIP_OK;
+}
+
 int small_hip_dense_f32(int batch, int No, int Ni, const float *in, const float *filt, float *out,
                         small_hip_stream_t stream)
 {

@@ -621,6 +621,33 @@ int small_hip_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, i
                    out, oq, Fuse{}, stream);
 }
 
+// The quantised form of the grouped convolution: one launch per slab of `channels` channels.
+int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
+                              int channels, int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                              const uint8_t *filt, const small_hip_quant *fq, uint8_t *out,
+                              const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_group_conv2d_u8";
+    if (channels <= 0 || channels % CB != 0) return SMALL_HIP_ECHANNELS;
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (batch <= 0 || groups <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
+    { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !out) { set_error("%s: null pointer", op); return SMALL_HIP_EINVAL; }
+    const size_t in_slab = (size_t)channels * H * W;
+    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    const size_t filt_slab = (size_t)channels * channels * kh * kw;
+    const size_t slabs = (size_t)batch * groups;
+    if (in + slabs * in_slab > out && out + slabs * out_slab > in)
+    { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
+    for (size_t i = 0; i < slabs; ++i)
+    {
+        const int rc = conv_u8(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, iq,
+                               filt + (i % groups) * filt_slab, fq, out + i * out_slab, oq, Fuse{}, stream);
+        if (rc != SMALL_HIP_OK) return rc;
+    }
+    return SMALL_HIP_OK;
+}
+
 int small_hip_dense_u8(int batch, int No, int Ni, const uint8_t *in, const small_hip_quant *iq,
                        const uint8_t *filt, const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq,
                        small_hip_stream_t stream)

@@ -375,13 +375,14 @@ int stest_fused_two_layers_f32(int second, int variant, int ck, int cs, int ct, 
 
 // The 1-D functions of small/interface_1D.hpp on PACKED arrays (batch-1 signatures of the reference; rows = its
 // batch_size).  kind 0 Conv1D, 1 PartialConv1D (out is in/out), 2 MaxPool1D, 3 AveragePool1D, 4 ReLUActivation1D,
-// 5 UpSample1D (k = scale), 6 Conv1D_ReLU, 7 Conv1D_Bias_ReLU (bias = 4th array)
+// 5 UpSample1D (k = scale), 6 Conv1D_ReLU, 7 Conv1D_Bias_ReLU (bias = 4th array), 8 GroupConv1D, 9 PartialGroupConv1D
+// (Co = groups, Ci = channels per group)
 int stest_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows, int W, const float *in, size_t n_in,
                  const float *filt, size_t n_filt, const float *bias, float *out, size_t n_out)
 {
     using FB = small::FloatBuffer;
     return guarded([&] {
-        FB x = from_host<FB>(in, n_in), f = from_host<FB>(filt, n_filt), b = from_host<FB>(bias, bias ? Co : 0);
+        FB x = from_host<FB>(in, n_in), f = from_host<FB>(filt, n_filt), b = from_host<FB>(bias, bias && kind == 7 ? Co : 0);
         FB o = from_host<FB>(out, n_out);
         switch (kind)
         {
@@ -392,6 +393,8 @@ int stest_1d_f32(int kind, int k, int s, int l, int r, int Co, int Ci, int rows,
         case 4: small::ReLUActivation1D(Ci, rows, W, x, o); break;
         case 5: small::UpSample1D(k, Ci, rows, W, x, o); break;
         case 6: small::Conv1D_ReLU(k, s, l, r, Co, Ci, rows, W, x, f, o); break;
+        case 8: small::GroupConv1D(k, s, Co, l, r, Ci, rows, W, x, f, o); break;          // Co = groups
+        case 9: small::PartialGroupConv1D(k, s, Co, l, r, Ci, rows, W, x, f, o); break;
         default: small::Conv1D_Bias_ReLU(k, s, l, r, Co, Ci, rows, W, x, f, b, o); break;
         }
         std::memcpy(out, o.data(), n_out * sizeof(float));

@@ -194,7 +194,11 @@ static void test_exceptions()
     expect([&] { small::DepthwiseConv2D(3, 3, 1, 0, 0, 0, 0, 24, 8, 8, a, f, o); }, "DepthwiseConv2D<float> ERROR: in_channels unsupported.");
     expect([&] { small::ReLUActivation(5, 4, 4, a, o); }, "ReLUActivation<float> ERROR: in_channels unsupported.");
     expect([&] { small::UpSample2D(3, 16, 4, 4, a, o); }, "Upsample<float> ERROR: scale factor unsupported (only 1 or 2).");
+    expect([&] { small::GroupConv2D(3, 3, 3, 1, 0, 0, 0, 0, 16, 6, 6, a, f, o); }, "GroupConv2D<float> ERROR: stride unsupported.");
+    expect([&] { small::GroupConv2D(3, 3, 1, 2, 0, 0, 0, 0, 8, 6, 6, a, f, o); }, "GroupConv2D<float> ERROR: in_channels unsupported.");
+    expect([&] { small::PartialGroupConv2D(3, 3, 3, 1, 0, 0, 0, 0, 16, 6, 6, a, f, o); }, "PartialGroupConv2D<float> ERROR: stride unsupported.");
     QUInt8Buffer qa(16 * 64), qf(16 * 16 * 9), qo(16 * 64);
+    expect([&] { small::GroupConv2D(3, 3, 3, 1, 0, 0, 0, 0, 16, 6, 6, qa, qf, qo); }, "GroupConv2D<quint8> ERROR: stride unsupported.");
     expect([&] { small::Conv2D(3, 3, 3, 0, 0, 0, 0, 16, 16, 8, 8, qa, qf, qo); }, "Conv2D<quint8> ERROR: stride unsupported.");
     expect([&] { small::ReLUActivation(5, 4, 4, qa, qo); }, "ReLUActivation<quint8> ERROR: in_channels unsupported.");
 }
@@ -390,6 +394,32 @@ static void test_fused_conv_pool_dropout_softmax()
     CHECK(almost_equal(sm[5] / sm[6], std::exp(x[5] - x[6]), 1e-4f));
 }
 
+static void test_group_conv()
+{
+    std::printf("grouped convolution\n");
+    // GroupConv2D over G slabs of C channels == Conv2D(C -> C) on each slab with its own filter block;
+    // PartialGroupConv2D adds the same into the output
+    const int G = 3, Cg = 16, H = 7, W = 9, nf = Cg * Cg * 9, nx = Cg * H * W;
+    FloatBuffer x(G * nx), f(G * nf), got(G * nx), twice(G * nx);
+    small::init(x, x.size());
+    small::init(f, f.size());
+    small::GroupConv2D(3, 3, 1, G, 1, 1, 1, 1, Cg, H, W, x, f, got);
+    for (size_t i = 0; i < twice.size(); ++i) twice[i] = got[i];
+    small::PartialGroupConv2D(3, 3, 1, G, 1, 1, 1, 1, Cg, H, W, x, f, twice);
+    for (int g = 0; g < G; ++g)
+    {
+        FloatBuffer xs(nx), fs(nf), want(nx);
+        for (int i = 0; i < nx; ++i) xs[i] = x[g * nx + i];
+        for (int i = 0; i < nf; ++i) fs[i] = f[g * nf + i];
+        small::Conv2D(3, 3, 1, 1, 1, 1, 1, Cg, Cg, H, W, xs, fs, want);
+        for (int i = 0; i < nx; ++i)
+        {
+            CHECK(got[g * nx + i] == want[i]);
+            CHECK(almost_equal(twice[g * nx + i], want[i] + want[i], 1e-4f));
+        }
+    }
+}
+
 int main(int argc, char **argv)
 {
     const std::string dir = argc > 1 ? argv[1] : "tests/golden/ref_regression";
@@ -402,6 +432,7 @@ int main(int argc, char **argv)
     test_window_fixtures(dir);
     test_quint8_and_batched();
     test_fused_conv_pool_dropout_softmax();
+    test_group_conv();
     std::printf(g_fail ? "FAILED: %d checks\n" : "ALL PASSED\n", g_fail);
     return g_fail ? 1 : 0;
 }

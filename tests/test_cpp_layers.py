@@ -208,6 +208,25 @@ def test_one_d_functions(hip, oracle, case, kind):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("partial", [0, 1])
+@pytest.mark.parametrize("case", [(3, 1, 1, 1, 2, 16, 1, 13), (3, 1, 1, 1, 3, 16, 3, 11), (3, 2, 0, 1, 2, 32, 1, 12),
+                                  (1, 1, 0, 0, 4, 16, 2, 9)], ids=str)
+def test_group_conv1d(hip, oracle, case, partial):
+    """small::GroupConv1D / PartialGroupConv1D on packed arrays against the oracle (pinned on the reference's scalar
+    build in test_oracle_1d_vs_ref.py)."""
+    k, s, l, r, G, Cg, rows, W = case
+    Wo = 1 + (W + l + r - k) // s
+    x = oracle.pack(synth.normal(1, G * Cg * rows * W), 0, 1, G * Cg, rows, W, 16, 16)
+    fl = synth.he_normal(2, G * Cg * Cg * k, Cg * k)
+    nf = Cg * Cg * k
+    f = np.concatenate([oracle.pack(fl[g * nf:(g + 1) * nf], 3, Cg, Cg, 1, k, 16, 16) for g in range(G)])
+    init = synth.normal(3, G * Cg * rows * Wo) if partial else None
+    got = hip.one_d_f32(8 + partial, k, s, l, r, G, Cg, rows, W, x, f, None, init, G * Cg * rows * Wo)
+    want = ol.one_d_f32(oracle, 6 + partial, 16, k, s, l, r, G, Cg, rows, W, x, f, init)
+    assert_close_f32(got, want, what="group conv1d %s" % (case,))
+
+
+@pytest.mark.gpu
 def test_one_d_errors(hip, oracle):
     """Same exception texts as the reference's 1-D functions (interface_abstract_1D.hpp:100-103, 160-163, 1650-1653)."""
     x = np.zeros(16 * 12, np.float32)
@@ -217,6 +236,10 @@ def test_one_d_errors(hip, oracle):
     with pytest.raises(ValueError, match=r"Conv1D<float> ERROR: in_channels unsupported\."):
         hip.one_d_f32(0, 3, 1, 1, 1, 16, 5, 1, 12, np.zeros(5 * 12, np.float32), np.zeros(16 * 5 * 3, np.float32), None,
                       None, 16 * 12)
+    with pytest.raises(ValueError, match=r"GroupConv1D<float> ERROR: stride unsupported\."):
+        hip.one_d_f32(8, 3, 3, 0, 0, 1, 16, 1, 12, x, f, None, None, 16 * 4)
+    with pytest.raises(ValueError, match=r"PartialGroupConv1D<float> ERROR: in_channels unsupported\."):
+        hip.one_d_f32(9, 3, 1, 1, 1, 2, 8, 1, 12, x, f, None, None, 16 * 12)
     with pytest.raises(ValueError, match=r"MaxPool1D<float> ERROR: stride unsupported\."):
         hip.one_d_f32(2, 3, 3, 0, 0, 16, 16, 1, 12, x, None, None, None, 16 * 4)
     with pytest.raises(ValueError, match=r"Upsample<float> ERROR: scale factor unsupported \(only 1 or 2\)\."):

@@ -47,3 +47,29 @@ def test_one_d_functions(oracle, ref_REF, case, kind):
     assert ref.lib.sref_1d_f32(kind, kk, s, l, r, Co, Ci, rows, W, bi.h, bf.h, bo.h) == 0, ref.err()
     want = ol.one_d_f32(oracle, kind, cb, kk, s, l, r, Co, Ci, rows, W, x, f, init)
     assert_equal_exact(want, bo.a, "%s %s" % (KINDS[kind], case))
+
+
+# (k, stride, l_pad, r_pad, groups, channels per group, rows, W)
+GROUP_1D_CASES = [(3, 1, 1, 1, 2, 16, 1, 13), (3, 1, 1, 1, 3, 16, 3, 11), (3, 2, 0, 1, 2, 32, 1, 12), (1, 1, 0, 0, 4, 16, 2, 9)]
+
+
+@pytest.mark.parametrize("partial", [0, 1])
+@pytest.mark.parametrize("case", GROUP_1D_CASES, ids=str)
+def test_group_conv1d(oracle, ref_REF, case, partial):
+    """GroupConv1D / PartialGroupConv1D (interface_abstract_1D.hpp:1255, 1388) on the scalar build, where the
+    tensors are [groups][channels][rows][W] and the filter [groups][channels][channels][k]: every group is a
+    Conv1D on its own slab."""
+    ref = ref_REF
+    k, s, l, r, G, Cg, rows, W = case
+    Wo = 1 + (W + l + r - k) // s
+    x = synth.normal(1, G * Cg * rows * W)
+    f = synth.he_normal(2, G * Cg * Cg * k, Cg * k)
+    init = synth.normal(3, G * Cg * rows * Wo) if partial else None
+    bi, bf = ref.fbuf(x.size, x), ref.fbuf(f.size, f)
+    bo = ref.fbuf(G * Cg * rows * Wo, init if partial else np.full(G * Cg * rows * Wo, 9.0, np.float32))
+    assert ref.lib.sref_1d_f32(6 + partial, k, s, l, r, G, Cg, rows, W, bi.h, bf.h, bo.h) == 0, ref.err()
+    want = ol.one_d_f32(oracle, 6 + partial, 1, k, s, l, r, G, Cg, rows, W, x, f, init)
+    assert_equal_exact(want, bo.a, "group conv1d %s" % (case,))
+    # every group differs: a dropped or repeated group cannot pass
+    per = want.reshape(G, -1)
+    assert all(not np.array_equal(per[a], per[b]) for a in range(G) for b in range(a))
