@@ -13,6 +13,7 @@ Prints ONE JSON line on stdout; progress goes to stderr.
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -68,7 +69,7 @@ def time_forward(ex, steps, warmup):
 
 
 def time_ops(ex, steps):
-    """Per-op device time (ms) from HIP events on the launch stream, averaged over `steps`.  Float32 models are
+    """Per-op device time (ms) from HIP events on the launch stream, the median over `steps` passes.  Float32 models are
     timed launch by launch as the forward pass issues them: a convolution that carries its 2x2 max-pool has the
     time of the fused launch, and the pool's own row reads 0.  (uint8 models are timed op by op, unfused.)"""
     import torch
@@ -77,7 +78,7 @@ def time_ops(ex, steps):
     if ex.model.dtype == "f32" and ex.fused:
         entries = ex.plan
         index = {op.name: i for i, op in enumerate(ops)}
-        tot = [0.0] * len(ops)
+        seen = [[] for _ in ops]
         for _ in range(steps):
             evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(entries) + 1)]
             evs[0].record()
@@ -86,9 +87,9 @@ def time_ops(ex, steps):
                 evs[i + 1].record()
             torch.cuda.synchronize()
             for i, e in enumerate(entries):
-                tot[index[e[0].name]] += evs[i].elapsed_time(evs[i + 1])
-        return [t / steps for t in tot]
-    tot = [0.0] * len(ops)
+                seen[index[e[0].name]].append(evs[i].elapsed_time(evs[i + 1]))
+        return [statistics.median(t) if t else 0.0 for t in seen]
+    seen = [[] for _ in ops]
     for _ in range(steps):
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)]
         evs[0].record()
@@ -97,8 +98,8 @@ def time_ops(ex, steps):
             evs[i + 1].record()
         torch.cuda.synchronize()
         for i in range(len(ops)):
-            tot[i] += evs[i].elapsed_time(evs[i + 1])
-    return [t / steps for t in tot]
+            seen[i].append(evs[i].elapsed_time(evs[i + 1]))
+    return [statistics.median(t) for t in seen]
 
 
 def layer_table(model, batch, ms):
@@ -431,6 +432,31 @@ def main():
         sg = (time.perf_counter() - t0) / args.steps
         extras["hip_graph_ms_per_step"] = round(sg * 1e3, 4)
         log("%s: HIP graph replay %.3f ms/step (eager %.3f)" % (model.name, sg * 1e3, sec * 1e3))
+        # the same step when the caller holds host buffers: pinned input uploaded, forward pass, output downloaded
+        # (a note beside the headline, which is measured with the input resident in device memory)
+        op = model.ops[-1]
+        c, h, w = op.out_shape()
+        n_out = ex.batch * c * h * w
+        hx = torch.empty(ex.buf["in"].numel(), dtype=ex.tdtype, pin_memory=True)
+        hx.copy_(ex.buf["in"])
+        hy = torch.empty(n_out, dtype=ex.tdtype, pin_memory=True)
+
+        def host_step():
+            ex.buf["in"].copy_(hx, non_blocking=True)
+            ex.forward()
+            hy.copy_(ex.buf[ex.out_name][:n_out], non_blocking=True)
+        for _ in range(args.warmup):
+            host_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            host_step()
+        torch.cuda.synchronize()
+        sh = (time.perf_counter() - t0) / args.steps
+        extras["host_buffers_ms_per_step"] = round(sh * 1e3, 4)
+        extras["host_buffers_images_per_s"] = round(ex.batch / sh, 1)
+        extras["host_buffers_MB_per_step"] = round((hx.numel() * hx.element_size() + hy.numel() * hy.element_size()) / 1e6, 2)
+        log("%s: with host buffers (upload + forward + download) %.3f ms/step" % (model.name, sh * 1e3))
     if not args.no_extras and args.model == "mobilenet_v1":
         for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
             m2 = getattr(models, name)()
