@@ -6,6 +6,11 @@
 
 Only tests, the smoke check and the benchmark's cpu_baseline leg import this
 module; the shipped package never does.
+
+Functions composed here rather than in C: group_conv2d_f32 / group_conv2d_u8 (one
+convolution of the C restatement per group).  Pinned: bit-identical to the
+reference's scalar build and equal to a library grouped convolution
+(tests/test_oracle_group_vs_ref.py).
 """
 import ctypes as C
 import os
