@@ -197,7 +197,7 @@ def cpu_threads():
     return threads
 
 
-def cpu_reference_model(model, weights, x_one, budget_s=12.0, max_passes=64):
+def cpu_reference_model(model, weights, x_one, budget_s=10.0, max_passes=4096):
     """The reference's own ZEN2 build (AVX2 + OpenMP) on this host, batch-1 calls.
     -> (cpu_baseline object, per-layer mean milliseconds per image)."""
     from oracle.binding import have_ref
@@ -235,7 +235,8 @@ def add_cpu_column(table, cpu_ms, batch):
 
 
 def cpu_port_u8(model, batch=8):
-    """ResNet-8 uint8 on the scalar C port (1 core): the reference has no uint8 Accum/AveragePool."""
+    """A model on the scalar C port (1 core).  ResNet-8 uint8: the reference has no uint8 Accum/AveragePool;
+    DS-CNN: its AVX2 build cannot run the 10x4 first layer."""
     from smallframework_amd import models
     from oracle.model_exec import OracleExecutor
     w = models.make_weights(model)
@@ -516,6 +517,7 @@ def main():
                 cpu = cpu_port_u8(model) if model.dtype == "u8" else None
             if not args.no_extras and args.model == "mobilenet_v1":
                 extras["resnet8_u8_cpu"] = cpu_port_u8(models.resnet8_u8())
+                extras["dscnn_cpu"] = cpu_port_u8(models.dscnn())
                 # reference CPU build beside the other float32 configurations (bounded samples)
                 for m2 in [models.tiny_yolo_v2()] + models.layer_sweep():
                     w2 = models.make_weights(m2)
