@@ -484,3 +484,24 @@ def test_conv2d_accum_relu_u8_equals_sequence(lib, oracle, qp, mode):
         if use_relu:
             _, want = oracle.relu_u8(batch, CB, Co, Ho, Wo, want, _oq(oq), _oq(oq))
         assert_equal_exact(hu.host(do), want, "fused %s Ci=%d" % (mode, Ci))
+
+
+def test_oversized_launches_are_refused_before_anything_runs(lib):
+    """Sizes whose pixel or plane count does not fit the kernels' 32-bit indexing come back as EINVAL with a
+    message (nothing is launched: the buffers here are far smaller than such a call would touch)."""
+    f32 = hu.dev_empty(16 * 16 + 64, np.float32)
+    f32b = hu.dev_empty(64, np.float32)
+    u8 = hu.dev_empty(16 * 16 + 64, np.uint8)
+    u8b = hu.dev_empty(64, np.uint8)
+    big = 1 << 20                     # images of 8x8 pixels: 2^26 output pixels > 2^31 / 64
+    rc = lib.small_hip_conv2d_f32(big, 1, 1, 1, 0, 0, 0, 0, 16, 16, 8, 8, hu.ptr(f32b), hu.ptr(f32), hu.ptr(f32[64:]),
+                                  hu.stream())
+    assert rc == capi.EINVAL and b"too large" in lib.small_hip_last_error()
+    iq, fq, oq = hu.q(-128), hu.q(-128), hu.q(0, 1 << 30, 0, 8)
+    rc = lib.small_hip_conv2d_u8(big, 1, 1, 1, 0, 0, 0, 0, 16, 16, 8, 8, hu.ptr(u8b), hu.qref(iq), hu.ptr(u8),
+                                 hu.qref(fq), hu.ptr(u8[64:]), hu.qref(oq), hu.stream())
+    assert rc == capi.EINVAL and b"too large" in lib.small_hip_last_error()
+    rc = lib.small_hip_depthwise_conv2d_f32(1 << 28, 3, 3, 1, 1, 1, 1, 1, 256, 4, 4, hu.ptr(f32b), hu.ptr(f32),
+                                            hu.ptr(f32[64:]), hu.stream())
+    assert rc == capi.EINVAL and b"too large" in lib.small_hip_last_error()
+    hu.torch_mod().cuda.synchronize()
