@@ -504,4 +504,6 @@ def test_oversized_launches_are_refused_before_anything_runs(lib):
     rc = lib.small_hip_depthwise_conv2d_f32(1 << 28, 3, 3, 1, 1, 1, 1, 1, 256, 4, 4, hu.ptr(f32b), hu.ptr(f32),
                                             hu.ptr(f32[64:]), hu.stream())
     assert rc == capi.EINVAL and b"too large" in lib.small_hip_last_error()
+    rc = lib.small_hip_maxpool2d_f32(1 << 28, 2, 2, 2, 0, 0, 0, 0, 256, 4, 4, hu.ptr(f32b), hu.ptr(f32), hu.stream())
+    assert rc == capi.EINVAL and b"too large" in lib.small_hip_last_error()
     hu.torch_mod().cuda.synchronize()
