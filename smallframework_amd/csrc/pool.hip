@@ -258,7 +258,8 @@ int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, 
     { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
     if (!in || !out || !aligned16(in) || !aligned16(out)) { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
     if (in == out) { set_error("%s: in-place pooling is not supported", op); return SMALL_HIP_EINVAL; }
-    if ((long)batch * (C / CB) > 0x7fffffffL) { set_error("%s: batch * C / 16 too large", op); return SMALL_HIP_EINVAL; }
+    if ((long)batch * (C / CB) > 0x7fffffffL || (long)H * W > 0x7fffffffL)
+    { set_error("%s: batch * C / 16 or H * W too large", op); return SMALL_HIP_EINVAL; }
     g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
     g->Ho = out_dim(H, pt, pb, kh, stride);
     g->Wo = out_dim(W, pl, pr, kw, stride);
