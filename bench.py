@@ -8,7 +8,8 @@ resident in HBM.  The headline workload is MobileNetV1 1.0 (224x224x3, float32) 
 line also carries ResNet-8 uint8 at batch 64 and 256, the per-layer roofline table, the roofline
 of the dominant kernel and the reference's CPU build timed on this host.
 
-Prints ONE JSON line on stdout; progress goes to stderr.
+Prints ONE compact JSON line on stdout (headline, roofline, cpu_baseline, a per-configuration summary);
+the per-layer tables go to gpurun_out/bench_<workload>_full.json, progress and readable tables to stderr.
 """
 import argparse
 import json
@@ -34,6 +35,65 @@ MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_*"): 93.7}
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_model_name():
+    """The host CPU's model string (first "model name" of /proc/cpuinfo)."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def table_summary(entry, batch):
+    """images/s + min / median per-layer roofline fraction of one configuration's per-layer table."""
+    fr = sorted(r["roofline_frac"] for r in entry["layers"] if r.get("roofline_frac"))
+    out = {"images_per_s": entry["images_per_s"], "ms_per_step": entry["ms_per_step"]}
+    if fr:
+        out["layer_frac_min"] = round(fr[0], 3)
+        out["layer_frac_median"] = round(statistics.median(fr), 3)
+    for k in ("hip_graph_ms_per_step", "one_launch_ms_per_step", "one_launch_images_per_s"):
+        if k in entry:
+            out[k] = entry[k]
+    return out
+
+
+def emit(out, tag):
+    """The full result (per-layer tables, extras) goes to gpurun_out/bench_<tag>_full.json and to stderr; stdout gets
+    ONE compact JSON line: the headline fields, roofline, cpu_baseline and a short per-configuration summary."""
+    full = json.dumps(out)
+    path = os.path.join(ROOT, "gpurun_out", "bench_%s_full.json" % tag)
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            f.write(full + "\n")
+        log("full per-layer tables and extras: %s" % path)
+    except OSError as e:
+        log("could not write %s: %r" % (path, e))
+    extras = out.get("extras") or {}
+    summary = {}
+    for key, e in extras.items():
+        if isinstance(e, dict) and "layers" in e and "images_per_s" in e:
+            summary[key] = table_summary(e, None)
+    head_fr = sorted(r["roofline_frac"] for r in out.get("layers", []) if r.get("roofline_frac"))
+    if head_fr:
+        summary["headline_layers"] = {"n": len(head_fr), "frac_min": round(head_fr[0], 3),
+                                      "frac_median": round(statistics.median(head_fr), 3)}
+    for k in ("mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "hip_graph_ms_per_step",
+              "host_buffers_ms_per_step", "host_buffers_images_per_s"):
+        if k in extras:
+            summary[k] = extras[k]
+    for k in ("resnet8_u8_cpu", "dscnn_cpu", "tiny_yolo_v2_cpu"):
+        if extras.get(k):
+            summary[k] = {f: extras[k][f] for f in ("value", "unit", "cores", "kind")}
+    compact = {k: v for k, v in out.items() if k not in ("layers", "extras")}
+    compact["summary"] = summary
+    compact["full_result"] = os.path.relpath(path, ROOT)
+    print(json.dumps(compact), flush=True)
 
 
 def op_bytes(model, op, batch):
@@ -217,8 +277,8 @@ def cpu_reference_model(model, weights, x_one, budget_s=10.0, max_passes=4096):
         ts.append(time.perf_counter() - t1)
         n += 1
     mean = sum(ts) / len(ts)
-    base = {"value": round(1.0 / mean, 2), "unit": "images/s", "cores": threads, "kind": "reference",
-            "sample": "%d batch-1 forward passes of %s (all layers, unfused Conv2D+ReLU as the reference's "
+    base = {"value": round(1.0 / mean, 2), "unit": "images/s", "cores": threads, "cpu": cpu_model_name(),
+            "kind": "reference", "sample": "%d batch-1 forward passes of %s (all layers, unfused Conv2D+ReLU as the reference's "
                       "Layer classes issue them) on the reference's ZEN2 build, 1 warm-up; min %.2f ms mean %.2f ms"
                       % (n, model.name, 1e3 * min(ts), 1e3 * mean)}
     return base, [1e3 * t / n for t in per_op]
@@ -248,8 +308,9 @@ def cpu_port_u8(model, batch=8):
     for _ in range(reps):
         OracleExecutor(model, batch, w, x).forward()
     dt = (time.perf_counter() - t0) / reps
-    return {"value": round(batch / dt, 1), "unit": "images/s", "cores": 1, "kind": "port",
-            "sample": "%d images x %d passes of %s on the scalar C restatement" % (batch, reps, model.name)}
+    return {"value": round(batch / dt, 1), "unit": "images/s", "cores": 1, "cpu": cpu_model_name(), "kind": "port",
+            "sample": "%d images x %d passes of %s on this build's scalar C restatement, 1 core (not the reference's "
+                      "build)" % (batch, reps, model.name)}
 
 
 def layout_rows(lib, torch, steps, warmup):
@@ -322,7 +383,7 @@ def sweep_only(args, torch, models):
                         "algorithmic_per_launch": {"GFLOP": round(batch * op.flops() / 1e9, 3),
                                                    "MB": round(op_bytes(m, op, batch) / 1e6, 3)}},
            "cpu_baseline": None, "layers": rows}
-    print(json.dumps(out), flush=True)
+    emit(out, "layer_sweep_b%d" % batch)
 
 
 def main():
@@ -546,7 +607,7 @@ def main():
         "layers": table,
         "extras": extras,
     }
-    print(json.dumps(out), flush=True)
+    emit(out, "%s_b%d" % (model.name, batch))
 
 
 if __name__ == "__main__":

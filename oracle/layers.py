@@ -12,7 +12,8 @@ Pinned (CPU suite) against the reference's own classes compiled into oracle/_ref
 (sref_conv_layer_f32 / sref_simple_layer_f32 / sref_model_f32 of oracle/ref_shim.cpp).
 The quantised variants have no counterpart that runs in the reference (its Layer classes call
 small::Bias / the float-only activations): they compose the quantised functions that are pinned one by
-one, and PartialConv2DLayer / AddLayer follow this build's own definition: parity unpinned.
+one, and PartialConv2DLayer / AddLayer follow this build's definition of the uint8 Accum (pinned through
+the reference's two-channel Conv2D with a filter of ones, tests/test_oracle_pins.py).
 
 fused_two_layers_f32 / fused_single_f32 restate the reference's "fused" functions
 (include/small/fused_interface_abstract.hpp) as what they compute: the plain layer sequence.  Pinned

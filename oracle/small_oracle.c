@@ -18,8 +18,10 @@
  *        reference regression fixtures (PyTorch generated), REF and ZEN2 builds of the
  *        reference on seeded inputs, float64 brute force, 1x1 case against a plain matmul
  *   so_conv2d_f32 with >= 2 padded output rows/cols on a side (e.g. 10x4 stride 2 "same")
- *        float64 brute-force zero-padded convolution only: the reference's edge code is
- *        not usable there (abstract_layer.hpp:1269-1349), so this is the textbook result
+ *        float64 brute-force zero-padded convolution and a library float64 conv2d on every row
+ *        (tests/test_oracle_pins.py); the reference's scalar build, bit-identical, on the rows
+ *        its edge code handles (rows 2..21 of the 10x4 stem): elsewhere its edge code is not
+ *        usable (abstract_layer.hpp:1269-1349), so this is the textbook result
  *   so_maxpool2d_f32 (incl. "padding counts as 0" quirk), so_avgpool2d_f32 (count_include_pad)
  *        reference fixtures, REF/ZEN2 builds with negative inputs on padded borders
  *   so_relu_f32, so_leaky_relu_f32, so_accum_f32, so_bias_f32, so_upsample2d_f32, so_upsample1d_f32, so_concat
@@ -31,12 +33,19 @@
  *   so_requant, so_conv2d_u8, so_dwconv2d_u8, so_maxpool2d_u8, so_relu_u8, so_dense_u8
  *        REF build (bit exact) on seeded inputs with positive and negative zero points;
  *        RNDRSHIFT/VQRDMULH against brute force on small ranges
- *   so_accum_u8, so_avgpool2d_u8, so_conv2d_bias_act_f32 (bias + activation fused)
- *        PARITY UNPINNED for the u8 pair: the reference has no uint8 Accum or AveragePool2D
- *        (interface_abstract.hpp:983, 1981).  Semantics are defined here and checked only
- *        against brute force on tiny inputs.  The fused float entry equals the reference's
- *        Bias + PartialConv2D + activation sequence (Conv2DLayer.hpp:827-879), which the
- *        REF build pins.
+ *   so_avgpool2d_u8   the reference has no uint8 AveragePool2D (interface_abstract.hpp:983); the
+ *        definition here is a depthwise convolution with a filter of ones and filter zero point 0,
+ *        and is pinned as such: bit-identical to the REF build's DepthwiseConv2D<QUInt8Buffer> on
+ *        that filter, to so_dwconv2d_u8, and to int64 window sums (tests/test_oracle_pins.py)
+ *   so_accum_u8   the reference has no uint8 Accum (interface_abstract.hpp:1981); the definition
+ *        here equals a two-input-channel 1x1 Conv2D<QUInt8Buffer> with a filter of ones, and is
+ *        pinned as such against the REF build over all 256 x 256 byte pairs (zI == zO; the
+ *        reachable pairs otherwise) and against an evaluation in unbounded integers
+ *   uint8 functions at channel block 16: equal to channel block 1 (what REF pins) after unpacking
+ *   so_conv2d_bias_act_f32   equals the reference's Bias + PartialConv2D + activation sequence
+ *        (Conv2DLayer.hpp:827-879), which the REF build pins
+ *   quantised 1-D forms (the 2-D functions on a 1 x k window): PARITY UNPINNED as 1-D calls; the
+ *        reference's quantised 1-D functions write unrelated bytes on its scalar build
  */
 #include "small_oracle.h"
 
@@ -690,8 +699,9 @@ int so_maxpool2d_u8(int batch, int cb, int kh, int kw, int stride, int pt, int p
                      0, out, oq);
 }
 
-/* PARITY UNPINNED: sum of (x + zI) over the valid taps, requantised with the output
- * buffer's multiplier/shift (the caller folds 1/(kh*kw) into them). */
+/* No reference counterpart.  Sum of (x + zI) over the valid taps, requantised with the output
+ * buffer's multiplier/shift (the caller folds 1/(kh*kw) into them) == the reference's quantised
+ * depthwise convolution with a filter of ones and filter zero point 0, which pins it. */
 int so_avgpool2d_u8(int batch, int cb, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
                     int C, int H, int W, const uint8_t *in, const so_quant *iq, uint8_t *out,
                     const so_quant *oq)
@@ -714,7 +724,8 @@ int so_relu_u8(int batch, int cb, int C, int H, int W, const uint8_t *in, const 
     return SO_OK;
 }
 
-/* PARITY UNPINNED: out = requant_out((in + zI) + (out + zO)) */
+/* No reference counterpart.  out = requant_out((in + zI) + (out + zO)) == the reference's quantised
+ * Conv2D over two input channels with a 1x1 filter of ones, which pins it. */
 int so_accum_u8(int batch, int cb, int C, int H, int W, const uint8_t *in, const so_quant *iq,
                 uint8_t *out, const so_quant *oq)
 {

@@ -114,7 +114,7 @@ int so_relu_u8(int batch, int cb, int C, int H, int W, const uint8_t *in, const 
                uint8_t *out, const so_quant *oq);
 int so_dense_u8(int batch, int cb, int No, int Ni, const uint8_t *in, const so_quant *iq,
                 const uint8_t *filt, const so_quant *fq, uint8_t *out, const so_quant *oq);
-/* no reference counterpart (parity unpinned): see small_oracle.c */
+/* no reference counterpart; each equals a reference uint8 call on a filter of ones, which pins it (small_oracle.c) */
 int so_accum_u8(int batch, int cb, int C, int H, int W, const uint8_t *in, const so_quant *iq,
                 uint8_t *out, const so_quant *oq);
 int so_avgpool2d_u8(int batch, int cb, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
