@@ -77,7 +77,9 @@ def emit(out, tag):
     extras = out.get("extras") or {}
     summary = {}
     for key, e in extras.items():
-        if isinstance(e, dict) and "layers" in e and "images_per_s" in e:
+        # the batch-1 single layers are launch-latency-bound: in the full file, not in the compact line
+        single_b1 = key.endswith("_b1") and len(e.get("layers", ())) == 1 if isinstance(e, dict) else False
+        if isinstance(e, dict) and "layers" in e and "images_per_s" in e and not single_b1:
             summary[key] = table_summary(e, None)
     head_fr = sorted(r["roofline_frac"] for r in out.get("layers", []) if r.get("roofline_frac"))
     if head_fr:
@@ -187,16 +189,25 @@ def layer_table(model, batch, ms):
 
 
 def mfma_probe_tflops(steps=5):
-    """Calibration: float32 MFMA instructions on registers only (small_hip_mfma_f32_probe), 8 workgroups per CU.
-    -> sustained TFLOP/s of the matrix pipes on this machine (to set beside the published 157.3)."""
+    """Calibration: float32 MFMA instructions on registers only (libsmall_hip_probe.so, a measurement aid that is
+    not part of the product library), 8 workgroups per CU.  -> sustained TFLOP/s of the matrix pipes on this
+    machine (to set beside the published 157.3), or None when the probe library is not built."""
     import ctypes as C
     import torch
     from smallframework_amd import capi
-    lib = capi.load()
+    path = os.path.join(os.path.dirname(capi.LIB_PATH), "libsmall_hip_probe.so")
+    if not os.path.exists(path):
+        return None
+    probe = C.CDLL(path).shp_probe_mfma_f32
+    probe.restype, probe.argtypes = C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     sink = torch.zeros(4, device="cuda")
     st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     wgs, iters = 256 * 8, 20000
-    call = lambda: capi.check(lib.small_hip_mfma_f32_probe(wgs, iters, C.c_void_p(sink.data_ptr()), st))
+
+    def call():
+        rc = probe(wgs, iters, C.c_void_p(sink.data_ptr()), st)
+        if rc:
+            raise RuntimeError("shp_probe_mfma_f32: status %d" % rc)
     call()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -429,7 +440,7 @@ def main():
     ms = time_ops(ex, args.steps)
     table = layer_table(model, batch, ms)
     if args.library_gemm:
-        log("float32 MFMA on registers only: %.1f TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
+        log("float32 MFMA on registers only: %s TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
         log("device-to-device copy of 822 MB: %.0f GB/s read + write (published peak 8000)" % hbm_copy_gbs())
         lib_ms = library_gemm_ms(model, batch, args.steps, args.warmup)
         for r in table:
@@ -480,7 +491,9 @@ def main():
               "sum_of_layer_ms": round(sum(ms), 4)}
     if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
-        extras["mfma_f32_sustained_TFLOPs"] = round(mfma_probe_tflops(), 1)
+        sustained = mfma_probe_tflops()
+        if sustained is not None:
+            extras["mfma_f32_sustained_TFLOPs"] = round(sustained, 1)
         extras["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
         # the same forward pass replayed from a HIP graph (no host work between the launches)
         ex.capture()

@@ -3,6 +3,7 @@
 // re-stated, not copied).
 #pragma once
 
+#include <cassert>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>

@@ -83,10 +83,6 @@ int small_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, small_hip_str
 int small_hip_memset(void *dst, int value, size_t bytes, small_hip_stream_t stream);
 int small_hip_stream_synchronize(small_hip_stream_t stream);
 
-/* Measurement aid without a counterpart in the reference: `workgroups` x 4 waves each issue iters x 4 independent
- * v_mfma_f32_32x32x2_f32 on registers (4 * 4096 flop per wave and iteration, no memory traffic), which measures the
- * rate the float32 matrix pipes sustain.  sink: any device float; it is not written. */
-int small_hip_mfma_f32_probe(int workgroups, int iters, float *sink, small_hip_stream_t stream);
 
 /* ---- float32 layers -------------------------------------------------------------------- */
 /* small::Conv2D<FloatBuffer>          include/small/interface.hpp:49-56,

@@ -40,6 +40,11 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     for o in objs:
         os.remove(o)
+    # measurement aid for bench.py (register-only MFMA loop); not linked into the product library
+    cmd = ["hipcc"] + FLAGS + ["-shared", os.path.join(CSRC, "probe.hip"), "-o", os.path.join(LIBDIR, "libsmall_hip_probe.so")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for probe.hip:\n" + r.stderr)
     return LIB
 
 

@@ -70,7 +70,6 @@ SIGNATURES = {
     "small_hip_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_partial_bias_f32": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_upsample2d_f32": (_i, [_i] * 5 + [_p, _p, _p]),
-    "small_hip_mfma_f32_probe": (_i, [_i, _i, _p, _p]),
     "small_hip_upsample1d_f32": (_i, [_i] * 5 + [_p, _p, _p]),
     "small_hip_yolo_decode_f32": (_i, [_i] * 5 + [_p, _i, _i, _p, _p, _p]),
     "small_hip_concat": (_i, [_i, _u32, _u32, _u32, _u32, _p, _p, _p, _sz, _p]),
@@ -105,6 +104,12 @@ def load():
             raise FileNotFoundError(
                 "%s is missing: build it with `python -m smallframework_amd.build` "
                 "(there is no CPU fallback)" % LIB_PATH)
+        # torch brings its own copy of the HIP runtime; it has to be in the process first so that this library binds
+        # to the same one (two runtimes in one process do not see each other's devices or memory)
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)      # AttributeError if the symbol is not exported

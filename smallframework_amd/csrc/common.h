@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 
 #include "../../include/small_hip.h"
 
@@ -107,10 +108,16 @@ __device__ __forceinline__ size_t split_col(size_t col, int Wo, int *ow)
 }
 #endif
 
-// Library-owned device scratch for the calling thread's current device: grows on demand and is
-// re-used by later calls.  Work that uses it is ordered by the stream it is launched on, so
-// calls that share a device must not overlap on different streams.
-int get_workspace(size_t bytes, void **ptr);
+// Library-owned device scratch of (current device, stream): grows on demand and is re-used by later calls on the
+// same stream; other streams get their own block.  The lease holds the pool's lock: keep it alive until the last
+// launch that uses `ptr` has been enqueued (a regrow on another thread frees blocks only under that lock, with a
+// call that waits for the device).
+struct WorkspaceLease
+{
+    std::unique_lock<std::mutex> lock;
+    void *ptr = nullptr;
+};
+int lease_workspace(size_t bytes, hipStream_t stream, WorkspaceLease *lease);
 
 inline hipStream_t as_stream(small_hip_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

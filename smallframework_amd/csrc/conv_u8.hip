@@ -33,6 +33,8 @@
 // is one 16-byte load.  A lane ends up with 4 consecutive output channels of one pixel:
 // requantise, pack, store one dword; the wave writes 256 contiguous bytes.
 #include "common.h"
+
+#include <mutex>
 #include "quant.h"
 
 #include <cstdlib>
@@ -587,8 +589,14 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }
+    // refuse what conv_u8_run would refuse before anything is enqueued
+    const long P = (long)batch * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    if (P == 0) return SMALL_HIP_OK;
+    if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     void *ws = nullptr;
-    if (int rc = get_workspace(prepared_bytes(kh, kw, Co, Ci), &ws)) return rc;
+    WorkspaceLease lease;            // held until the launches below are enqueued
+    if (int rc = lease_workspace(prepared_bytes(kh, kw, Co, Ci), s, &lease)) return rc;
+    ws = lease.ptr;
     if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
     return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s);
 }

@@ -41,7 +41,7 @@ __device__ __forceinline__ float4 ew_apply(float4 x, float4 o, float slope)
 
 // n4 = number of float4 elements
 template <int OP>
-__global__ __launch_bounds__(TPB) void ew_f32_kernel(const float4 *__restrict__ in, float4 *out,
+__global__ __launch_bounds__(TPB) void ew_f32_kernel(const float4 *in, float4 *out,
                                                      size_t n4, float slope)
 {
     const size_t base = (size_t)blockIdx.x * (TPB * UNROLL) + threadIdx.x;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(TPB) void ew_f32_kernel(const float4 *__restrict__ 
     }
 }
 
-// in == out aliasing is allowed, so no __restrict__ on the pair above for ACCUM/RELU in place:
+// in == out is allowed (every activation of every model runs in place), so neither pointer above is __restrict__:
 // every lane reads its own elements before writing them.
 
 // bias: out[n][cb][p][16] = (accumulate ? out : 0) + bias[cb*16 + c]

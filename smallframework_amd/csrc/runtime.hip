@@ -1,5 +1,6 @@
 // Runtime helpers of the C ABI: error strings, device memory, copies.
 #include "common.h"
+#include "workspace.h"
 
 #include <cstring>
 #include <mutex>
@@ -18,81 +19,54 @@ void set_error(const char *fmt, ...)
 
 namespace
 {
-constexpr int MAX_DEV = 16;
-std::mutex g_ws_mu;
-void *g_ws_ptr[MAX_DEV] = {};
-size_t g_ws_cap[MAX_DEV] = {};
+struct HipMem
+{
+    static int alloc(void **p, size_t bytes)
+    {
+        hipError_t e = hipMalloc(p, bytes);
+        if (e == hipSuccess) return SMALL_HIP_OK;
+        (void)hipGetLastError();
+        set_error("workspace hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+        return e == hipErrorOutOfMemory ? SMALL_HIP_ENOMEM : SMALL_HIP_EHIP;
+    }
+    // hipFree waits for the device, so no queued kernel still reads the block when it returns
+    static int release(void *p)
+    {
+        hipError_t e = hipFree(p);
+        return e == hipSuccess ? SMALL_HIP_OK : fail_hip(e, "workspace hipFree");
+    }
+};
+
+WorkspacePool<HipMem> &pool()
+{
+    static WorkspacePool<HipMem> *p = [] {
+        auto *q = new WorkspacePool<HipMem>();       // never destroyed: blocks outlive static destruction order
+        q->set_full_code(SMALL_HIP_ENOMEM);
+        return q;
+    }();
+    return *p;
+}
 } // namespace
 
-int get_workspace(size_t bytes, void **ptr)
+int lease_workspace(size_t bytes, hipStream_t stream, WorkspaceLease *lease)
 {
     int dev = 0;
     SHP_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= MAX_DEV) return einval("get_workspace: device index out of range");
-    std::lock_guard<std::mutex> lk(g_ws_mu);
-    if (bytes > g_ws_cap[dev])
+    lease->lock = pool().lock();
+    int rc = pool().acquire(dev, stream, bytes, &lease->ptr);
+    if (rc != SMALL_HIP_OK)
     {
-        if (g_ws_ptr[dev])
-        {
-            // hipFree waits for the device, so no queued kernel still reads the old block
-            SHP_HIP(hipFree(g_ws_ptr[dev]));
-            g_ws_ptr[dev] = nullptr;
-            g_ws_cap[dev] = 0;
-        }
-        size_t cap = (bytes + (1u << 20) - 1) & ~(size_t)((1u << 20) - 1);
-        hipError_t e = hipMalloc(&g_ws_ptr[dev], cap);
-        if (e != hipSuccess)
-        {
-            (void)hipGetLastError();
-            set_error("workspace hipMalloc(%zu): %s", cap, hipGetErrorString(e));
-            return e == hipErrorOutOfMemory ? SMALL_HIP_ENOMEM : SMALL_HIP_EHIP;
-        }
-        g_ws_cap[dev] = cap;
+        if (rc == SMALL_HIP_ENOMEM && small_hip_last_error()[0] == 0) set_error("workspace: too many streams hold a block");
+        lease->lock.unlock();
     }
-    *ptr = g_ws_ptr[dev];
-    return SMALL_HIP_OK;
+    return rc;
 }
 
 } // namespace shp
 
 using namespace shp;
 
-namespace
-{
-typedef float probe_x16 __attribute__((ext_vector_type(16)));
-
-// Measurement aid: every wave issues `iters` rounds of four independent v_mfma_f32_32x32x2_f32 on registers (no
-// memory traffic inside the loop), i.e. what the matrix pipes sustain on this machine at its sustained clock.
-__global__ __launch_bounds__(256) void mfma_f32_probe_kernel(int iters, float *sink)
-{
-    probe_x16 acc[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
-    const float a = 1.0f + (float)(threadIdx.x & 3) * 0.25f, b = 0.5f;
-    for (int it = 0; it < iters; ++it)
-    {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
-    }
-    float t = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) t += acc[i][0] + acc[i][15];
-    if (t == 12345.678f) sink[0] = t;      // keeps the loop alive; never true
-}
-} // namespace
-
 extern "C" {
-
-int small_hip_mfma_f32_probe(int workgroups, int iters, float *sink, small_hip_stream_t stream)
-{
-    if (workgroups <= 0 || iters <= 0 || !sink) return shp::einval("small_hip_mfma_f32_probe: bad argument");
-    hipLaunchKernelGGL(mfma_f32_probe_kernel, dim3((unsigned)workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                       iters, sink);
-    SHP_LAUNCH_CHECK("small_hip_mfma_f32_probe");
-    return SMALL_HIP_OK;
-}
 
 const char *small_hip_version(void) { return "small_hip 0.1 (gfx950)"; }
 
