@@ -247,6 +247,21 @@ int small_hip_conv2d_u8(int batch, int kernel_height, int kernel_width, int stri
                         const small_hip_quant *input_q, const uint8_t *filter,
                         const small_hip_quant *filter_q, uint8_t *output,
                         const small_hip_quant *output_q, small_hip_stream_t stream);
+/* small_hip_conv2d_u8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * small_hip_conv2d_u8; the filter pre-pass writes into a static device array of
+ * SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES bytes instead of an allocated block, and the call returns SMALL_HIP_EINVAL
+ * when small_hip_conv2d_u8_prepared_filter_bytes(kh, kw, Co, Ci) exceeds that (input_channels of 1..3 need no
+ * scratch at all).  It calls no hipMalloc / hipFree.  Every call on one GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered by the stream.  Nothing in
+ * the array has to start at zero: the pre-pass writes every byte the convolution reads. */
+#define SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES (4u << 20)
+int small_hip_conv2d_u8_noalloc(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                                int b_pad, int l_pad, int r_pad, int output_channels, int input_channels,
+                                int input_height, int input_width, const uint8_t *input,
+                                const small_hip_quant *input_q, const uint8_t *filter,
+                                const small_hip_quant *filter_q, uint8_t *output,
+                                const small_hip_quant *output_q, small_hip_stream_t stream);
 /* The same convolution split in two for callers whose filters are constant (the reference's
  * Conv2DLayer packs its filter once at construction, include/small/Conv2DLayer.hpp:135-341):
  * _prepare_filter re-orders a packed uint8 filter (input_channels % 16 == 0) into the kernel's

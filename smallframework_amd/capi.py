@@ -78,6 +78,7 @@ SIGNATURES = {
     "small_hip_dense_f32": (_i, [_i] * 3 + [_p, _p, _p, _p]),
     "small_hip_dense_literal_f32": (_i, [_i] * 2 + [_p, _p, _p, _p]),
     "small_hip_conv2d_u8": (_i, _conv + [_p, _q, _p, _q, _p, _q, _p]),
+    "small_hip_conv2d_u8_noalloc": (_i, _conv + [_p, _q, _p, _q, _p, _q, _p]),
     "small_hip_conv2d_u8_prepared_filter_bytes": (_sz, [_i] * 4),
     "small_hip_conv2d_u8_prepare_filter": (_i, [_i] * 4 + [_p, _p, _p]),
     "small_hip_conv2d_u8_prepared": (_i, _conv + [_p, _q, _p, _q, _p, _q, _p]),

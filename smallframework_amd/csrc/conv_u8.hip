@@ -507,6 +507,40 @@ int conv_u8_check(const char *op, int batch, int kh, int kw, int stride, int pt,
     return SMALL_HIP_OK;
 }
 
+// ---- scratch of the entry point that allocates nothing -------------------------------------------------------
+// The filter pre-pass of small_hip_conv2d_u8_noalloc writes here instead of into an allocated block.  Every GPU the
+// library runs on holds its own copy of the array at its own address until the process ends; in host code the array's
+// name is only a handle for hipGetSymbolAddress, whose per-device result is what kernels and copies are given.
+constexpr size_t NOALLOC_SCRATCH_BYTES = size_t(SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES);
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+int static_scratch(const char *op, size_t bytes, void **ptr)
+{
+    constexpr int MAX_DEV = 64;
+    static std::mutex mu;
+    static void *addr[MAX_DEV] = {};
+    if (bytes > NOALLOC_SCRATCH_BYTES)
+    {
+        set_error("%s: the prepared filter needs %zu bytes, the static scratch holds %zu (use "
+                  "small_hip_conv2d_u8_prepare_filter + small_hip_conv2d_u8_prepared for larger filters)",
+                  op, bytes, NOALLOC_SCRATCH_BYTES);
+        return SMALL_HIP_EINVAL;
+    }
+    int dev = 0;
+    SHP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEV) { set_error("%s: device index out of range", op); return SMALL_HIP_EINVAL; }
+    std::lock_guard<std::mutex> lk(mu);
+    if (!addr[dev])
+    {
+        void *p = nullptr;
+        SHP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));      // the current device's copy
+        if (!p) { set_error("%s: hipGetSymbolAddress returned null", op); return SMALL_HIP_EHIP; }
+        addr[dev] = p;
+    }
+    *ptr = addr[dev];
+    return SMALL_HIP_OK;
+}
+
 struct Fuse
 {
     const uint8_t *accum_src = nullptr;
@@ -560,7 +594,7 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
 int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
             int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
             const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, const Fuse &fz,
-            small_hip_stream_t stream)
+            small_hip_stream_t stream, bool static_ws = false)
 {
     if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt, out, iq, fq, oq))
         return rc;
@@ -595,8 +629,15 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     void *ws = nullptr;
     WorkspaceLease lease;            // held until the launches below are enqueued
-    if (int rc = lease_workspace(prepared_bytes(kh, kw, Co, Ci), s, &lease)) return rc;
-    ws = lease.ptr;
+    if (static_ws)
+    {
+        if (int rc = static_scratch(op, prepared_bytes(kh, kw, Co, Ci), &ws)) return rc;
+    }
+    else
+    {
+        if (int rc = lease_workspace(prepared_bytes(kh, kw, Co, Ci), s, &lease)) return rc;
+        ws = lease.ptr;
+    }
     if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
     return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s);
 }
@@ -627,6 +668,15 @@ int small_hip_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, i
 {
     return conv_u8("small_hip_conv2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, filt, fq,
                    out, oq, Fuse{}, stream);
+}
+
+int small_hip_conv2d_u8_noalloc(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
+                                int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
+                                const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq,
+                                small_hip_stream_t stream)
+{
+    return conv_u8("small_hip_conv2d_u8_noalloc", batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, filt,
+                   fq, out, oq, Fuse{}, stream, true);
 }
 
 // The quantised form of the grouped convolution: one launch per slab of `channels` channels.

@@ -1,0 +1,75 @@
+"""small_hip_conv2d_u8_noalloc: the uint8 convolution for callers that cannot allocate device memory.  Its filter
+pre-pass writes into a static device array instead of an allocated block; results must equal small_hip_conv2d_u8
+bit for bit (and the oracle), on two calls in a row that share the array, the second one smaller."""
+import numpy as np
+import pytest
+
+import hip_util as hu
+from smallframework_amd import capi, synth
+from util import assert_equal_exact
+
+pytestmark = pytest.mark.gpu
+CB = 16
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return capi.load()
+
+
+def _oq(q):
+    from oracle.binding import quant
+    return quant(q.zero, q.multiplier, q.lshift, q.rshift)
+
+
+def _both(lib, oracle, case, qp, seed):
+    batch, kh, kw, s, (pt, pb, pl, pr), Co, Ci, H, W = case
+    zi, zf, mul, ls, rs = qp
+    x = synth.uniform_u8(seed, batch * Ci * H * W)
+    f = synth.uniform_u8(seed + 1, Co * Ci * kh * kw)
+    Ho, Wo = oracle.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
+    iq, fq, oq = hu.q(zi), hu.q(zf), hu.q(5, mul, ls, rs)
+    dx, df = hu.dev(x), hu.dev(f)
+    n = batch * Co * Ho * Wo
+    d_new, d_old = hu.dev_empty(n, np.uint8), hu.dev_empty(n, np.uint8)
+    args = (batch, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W)
+    print("noalloc case", case, qp, flush=True)
+    rc = lib.small_hip_conv2d_u8_noalloc(*args, hu.ptr(dx), hu.qref(iq), hu.ptr(df), hu.qref(fq), hu.ptr(d_new),
+                                         hu.qref(oq), hu.stream())
+    assert rc == 0, lib.small_hip_last_error()
+    got = hu.host(d_new)
+    rc = lib.small_hip_conv2d_u8(*args, hu.ptr(dx), hu.qref(iq), hu.ptr(df), hu.qref(fq), hu.ptr(d_old),
+                                 hu.qref(oq), hu.stream())
+    assert rc == 0, lib.small_hip_last_error()
+    assert_equal_exact(got, hu.host(d_old), "noalloc vs small_hip_conv2d_u8 %s" % (case,))
+    rco, want = oracle.conv2d_u8(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, _oq(iq), f, _oq(fq), _oq(oq))
+    assert rco == 0
+    assert_equal_exact(got, want, "noalloc vs oracle %s" % (case,))
+    return got
+
+
+def test_noalloc_two_calls_in_a_row_second_smaller(lib, oracle):
+    qp = (-128, -128, 1518500250, 0, 9)
+    big = (2, 3, 3, 1, (1, 1, 1, 1), 64, 64, 16, 16)          # prepared filter: 64*64*9 bytes + table
+    small = (3, 3, 3, 2, (0, 1, 0, 1), 32, 16, 12, 12)        # fits inside what the first call left behind
+    a = _both(lib, oracle, big, qp, 141)
+    b = _both(lib, oracle, small, qp, 151)
+    assert len(np.unique(a)) > 50 and len(np.unique(b)) > 50
+    # and once more the other way round, with other quantisation parameters and a 1x1 window
+    _both(lib, oracle, (1, 1, 1, 2, (0, 0, 0, 0), 32, 16, 8, 8), (100, 156, (1 << 31) - 1, 0, 15), 161)
+    _both(lib, oracle, big, (-3, 5, 1234567890, 1, 4), 171)
+
+
+def test_noalloc_small_channel_stem_and_limits(lib, oracle):
+    # 1..3 input channels take the stem kernel: no scratch involved
+    _both(lib, oracle, (2, 3, 3, 1, (1, 1, 1, 1), 16, 3, 16, 16), (-128, -128, 1518500250, 0, 9), 181)
+    # a filter whose prepared form exceeds the static array is refused before anything runs
+    kh = kw = 3
+    Co = Ci = 1024
+    assert lib.small_hip_conv2d_u8_prepared_filter_bytes(kh, kw, Co, Ci) > (4 << 20)
+    fake = hu.dev_empty(1024, np.uint8)
+    q = hu.q(0)
+    rc = lib.small_hip_conv2d_u8_noalloc(1, kh, kw, 1, 1, 1, 1, 1, Co, Ci, 4, 4, hu.ptr(fake), hu.qref(q), hu.ptr(fake),
+                                         hu.qref(q), hu.ptr(hu.dev_empty(1024, np.uint8)), hu.qref(q), hu.stream())
+    assert rc == capi.EINVAL
+    assert b"static scratch" in lib.small_hip_last_error()
