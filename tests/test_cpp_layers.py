@@ -13,7 +13,7 @@ import pytest
 from oracle import layers as ol
 from oracle.binding import quant
 from smallframework_amd import synth
-from util import assert_close_f32, assert_equal_exact
+from util import assert_close_f32, assert_equal_exact, strict_bar
 import layer_shims
 from test_oracle_layers_vs_ref import CONV_LAYER_CASES, SIMPLE_CASES, conv_layer_inputs, simple_inputs
 
@@ -103,6 +103,23 @@ def _model_case(name):
     raise KeyError(name)
 
 
+class _Acc64:
+    """The oracle with float64 accumulation forced on every convolution / depthwise call."""
+
+    def __init__(self, o):
+        self._o = o
+
+    def __getattr__(self, n):
+        f = getattr(self._o, n)
+        if n in ("conv2d_f32", "dwconv2d_f32"):
+            return lambda *a, **k: f(*a, **dict(k, acc64=1))
+        return f
+
+
+# (fraction of elements, worst excess) allowed outside |a-b| <= 1e-4|b| + 1e-5; models not listed: nothing outside
+STRICT_LIMITS = {"TinyYoloV2_leaky_125": (5e-3, 3e-5), "TinyYoloV2": (5e-3, 3e-5)}
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["MobileNetTiny", "MobileNetV1_224_1000", "Resnet8Tiny", "Resnet8_10", "DSCNNTiny",
                                   "DSCNN_10x4_12", "TinyYoloV2", "TinyYoloV2_leaky_125", "AutoencoderTiny",
@@ -115,6 +132,9 @@ def test_models(hip, oracle, name):
     assert got.shape == want.shape, (got.shape, want.shape)
     scale = max(1.0, float(np.abs(want).max()))
     assert_close_f32(got, want, atol=1e-5 * scale, what=name)
+    # the stated bar, unscaled, against the same model with float64 accumulation in every convolution
+    strict_bar(got, fn(_Acc64(oracle), x, filters), "model class " + name, *STRICT_LIMITS.get(name, (0.0, 0.0)),
+               reference=want)
     # the batched model equals the batch-1 model image by image (same kernels or within tolerance)
     one = hip.model_f32(which, x[1:2], filters, variant)
     assert_close_f32(one[0], got[1], atol=1e-5 * scale, what=name + " batch-1 vs batched")

@@ -43,3 +43,40 @@ def read_ref_bin(path):
     a = np.frombuffer(raw, dtype="<f4", offset=4)
     assert a.size == n, (path, a.size, n)
     return a.astype(np.float32)
+
+
+STRICT_LOG = os.path.join(os.path.dirname(os.path.dirname(GOLDEN)), "gpurun_out", "strict_f32_bar.jsonl")
+
+
+def strict_bar(got, truth, what, max_outside_frac, max_excess, reference=None):
+    """The stated float32 bar without any scaling: against `truth` (the same computation with float64
+    accumulation), count the elements outside |a - b| <= 1e-4 * |b| + 1e-5 and take the worst excess over that
+    bound.  Prints the figures, appends them to gpurun_out/strict_f32_bar.jsonl and asserts the given limits
+    (a fraction of the elements, and an absolute excess).  `reference`: the float32 sequential-order oracle's result
+    for the same inputs; its own count against the same truth is recorded beside the GPU's."""
+    import json
+    got = np.asarray(got, np.float64).ravel()
+    truth = np.asarray(truth, np.float64).ravel()
+    assert got.shape == truth.shape, (what, got.shape, truth.shape)
+    err = np.abs(got - truth)
+    excess = err - (RTOL * np.abs(truth) + ATOL)
+    outside = int((excess > 0).sum())
+    rec = {"what": what, "elements": int(got.size), "outside_strict_bar": outside,
+           "outside_frac": outside / max(1, got.size), "worst_excess": float(max(0.0, excess.max())),
+           "max_abs_err": float(err.max()), "max_abs_value": float(np.abs(truth).max())}
+    if reference is not None:
+        r = np.asarray(reference, np.float64).ravel()
+        rex = np.abs(r - truth) - (RTOL * np.abs(truth) + ATOL)
+        rec["reference_f32_outside"] = int((rex > 0).sum())
+        rec["reference_f32_worst_excess"] = float(max(0.0, rex.max()))
+    print("strict float32 bar: %(what)s: %(outside_strict_bar)d of %(elements)d outside (%(outside_frac).2e), "
+          "worst excess %(worst_excess).3g, max |err| %(max_abs_err).3g at max |y| %(max_abs_value).3g" % rec)
+    try:
+        os.makedirs(os.path.dirname(STRICT_LOG), exist_ok=True)
+        with open(STRICT_LOG, "a") as f:
+            f.write(json.dumps(rec) + "\n")
+    except OSError:
+        pass
+    assert rec["outside_frac"] <= max_outside_frac, rec
+    assert rec["worst_excess"] <= max_excess, rec
+    return rec
