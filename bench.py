@@ -548,12 +548,31 @@ def main():
                 e2.replay()
             torch.cuda.synchronize()
             s3 = (time.perf_counter() - t0) / max(args.steps, 50)
+            # the whole model in one launch (one workgroup per image, tensors and filters in LDS), HIP-event timed
+            e2.build_one_launch()
+            for _ in range(args.warmup):
+                e2.forward_one_launch()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n1 = max(args.steps, 50)
+            ev0.record()
+            for _ in range(n1):
+                e2.forward_one_launch()
+            ev1.record()
+            torch.cuda.synchronize()
+            s4 = ev0.elapsed_time(ev1) * 1e-3 / n1
+            algo = b * (m2.in_shape[0] * m2.in_shape[1] * m2.in_shape[2] + m2.ops[-1].Co) + \
+                sum(o.weight_elems() for o in m2.ops)
             extras["%s_b%d" % (name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
                                             "hip_graph_images_per_s": round(b / s3, 1),
                                             "hip_graph_ms_per_step": round(s3 * 1e3, 4),
+                                            "one_launch_ms_per_step": round(s4 * 1e3, 4),
+                                            "one_launch_images_per_s": round(b / s4, 1),
+                                            "one_launch_TOPs": round(b * m2.flops_per_image() / s4 / 1e12, 2),
+                                            "one_launch_algorithmic_MB": round(algo / 1e6, 3),
                                             "layers": layer_table(m2, b, ms2)}
-            log("%s batch %d: eager %.4f ms/step %.0f images/s | HIP graph %.4f ms/step %.0f images/s"
-                % (name, b, s2 * 1e3, b / s2, s3 * 1e3, b / s3))
+            log("%s batch %d: layer by layer %.4f ms/step %.0f images/s | HIP graph %.4f ms/step | ONE LAUNCH %.4f ms/step "
+                "%.0f images/s" % (name, b, s2 * 1e3, b / s2, s3 * 1e3, s4 * 1e3, b / s4))
+            e2.close()
             del e2
         torch.cuda.empty_cache()
         # the other float32 configurations: whole models and the single-layer sweep at C = 256, 56x56

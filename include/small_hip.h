@@ -359,6 +359,51 @@ int small_hip_unpack(int type, int batch, uint32_t dim0, uint32_t dim1, uint32_t
                      uint32_t c_ib, uint32_t c_ob, const void *packed, void *flat, size_t element_size,
                      small_hip_stream_t stream);
 
+/* ---- a whole quantised model in one launch ------------------------------------------------------
+ * No counterpart as a function in the reference; it stands for what the reference's Model classes do
+ * (include/small/Model.hpp, include/small/models/Resnet8Tiny.hpp:229-414: a fixed list of layers run one after
+ * the other on ping-pong buffers) for models small enough that every activation tensor and every filter fit in
+ * one compute unit's 160 KB of LDS (ResNet-8 on 32x32x3: 16 KB per tensor, 77 KB of filters).  One workgroup then
+ * owns one image from input to output and only those two touch device memory.  Results are bit-identical to the
+ * same layers issued one by one (small_hip_conv2d_accum_relu_u8, small_hip_avgpool2d_u8, small_hip_maxpool2d_u8).
+ *
+ * A layer is a convolution (any window up to the tensors' one-pixel ring: pads <= 1, stride 1 or 2; a fully
+ * connected layer is the 1x1 convolution on a 1x1 image; 1..3 input channels only on the model input, window up to
+ * 4x4) optionally followed by Accum of another tensor and / or the in-place ReLU, or a pooling layer whose window is
+ * the whole image.  Tensors are named by small integers 0..7 (re-usable like ping-pong buffers);
+ * SMALL_HIP_QM_INPUT is the model input (first layer only), SMALL_HIP_QM_OUTPUT the model output (last layer only).
+ * small_hip_qmodel_create() copies and re-orders the filters (it allocates device memory and returns after its
+ * work on `stream` has finished; the filters may be released afterwards) and returns SMALL_HIP_EINVAL with a
+ * message when the model does not fit; small_hip_qmodel_forward() is one launch and allocates nothing.
+ * input: batch images back to back, packed as for small_hip_conv2d_u8; output: batch x the last layer's packed
+ * output. */
+#define SMALL_HIP_QL_CONV 0
+#define SMALL_HIP_QL_GLOBAL_AVGPOOL 1
+#define SMALL_HIP_QL_GLOBAL_MAXPOOL 2
+#define SMALL_HIP_QM_INPUT (-1)
+#define SMALL_HIP_QM_OUTPUT (-2)
+#define SMALL_HIP_QM_NONE (-3)
+typedef struct small_hip_qlayer
+{
+    int kind;                      /* SMALL_HIP_QL_* */
+    int src, dst;                  /* tensor ids */
+    int accum_src;                 /* tensor added to the convolution's output (small::Accum), or SMALL_HIP_QM_NONE */
+    int relu;                      /* small::ReLUActivation in place on the output */
+    int kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad;
+    int output_channels, input_channels, input_height, input_width;
+    const uint8_t *filter;         /* device pointer, packed as for small_hip_conv2d_u8; NULL for pooling */
+    small_hip_quant input_q, filter_q, output_q, accum_q;   /* as the buffers of the layer-by-layer calls carry them */
+} small_hip_qlayer;
+typedef struct small_hip_qmodel small_hip_qmodel;
+int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_hip_qmodel **model,
+                            small_hip_stream_t stream);
+int small_hip_qmodel_forward(const small_hip_qmodel *model, int batch, const uint8_t *input, uint8_t *output,
+                             small_hip_stream_t stream);
+/* bytes of one image's output / of LDS the launch uses */
+size_t small_hip_qmodel_output_bytes(const small_hip_qmodel *model);
+size_t small_hip_qmodel_lds_bytes(const small_hip_qmodel *model);
+int small_hip_qmodel_destroy(small_hip_qmodel *model);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,20 @@ class Quant(C.Structure):
         super().__init__(int(zero), int(multiplier), int(lshift), int(rshift))
 
 
+class QLayer(C.Structure):
+    """small_hip_qlayer: one layer of a whole-model launch (small_hip_qmodel_create)."""
+    _fields_ = [("kind", C.c_int), ("src", C.c_int), ("dst", C.c_int), ("accum_src", C.c_int), ("relu", C.c_int),
+                ("kernel_height", C.c_int), ("kernel_width", C.c_int), ("stride", C.c_int),
+                ("t_pad", C.c_int), ("b_pad", C.c_int), ("l_pad", C.c_int), ("r_pad", C.c_int),
+                ("output_channels", C.c_int), ("input_channels", C.c_int), ("input_height", C.c_int),
+                ("input_width", C.c_int), ("filter", C.c_void_p),
+                ("input_q", Quant), ("filter_q", Quant), ("output_q", Quant), ("accum_q", Quant)]
+
+
+QL_CONV, QL_GLOBAL_AVGPOOL, QL_GLOBAL_MAXPOOL = 0, 1, 2
+QM_INPUT, QM_OUTPUT, QM_NONE = -1, -2, -3
+
+
 class SmallHipError(RuntimeError):
     def __init__(self, status, msg):
         super().__init__("small_hip status %d: %s" % (status, msg))
@@ -90,6 +104,11 @@ SIGNATURES = {
     "small_hip_dense_u8": (_i, [_i] * 3 + [_p, _q, _p, _q, _p, _q, _p]),
     "small_hip_accum_u8": (_i, [_i] * 4 + [_p, _q, _p, _q, _p]),
     "small_hip_avgpool2d_u8": (_i, _win + [_p, _q, _p, _q, _p]),
+    "small_hip_qmodel_create": (_i, [_i, C.POINTER(QLayer), C.POINTER(_p), _p]),
+    "small_hip_qmodel_forward": (_i, [_p, _i, _p, _p, _p]),
+    "small_hip_qmodel_output_bytes": (_sz, [_p]),
+    "small_hip_qmodel_lds_bytes": (_sz, [_p]),
+    "small_hip_qmodel_destroy": (_i, [_p]),
     "small_hip_pack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
     "small_hip_unpack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
 }

@@ -119,6 +119,13 @@ struct WorkspaceLease
 };
 int lease_workspace(size_t bytes, hipStream_t stream, WorkspaceLease *lease);
 
+// uint8 convolution filter pre-pass (conv_u8.hip): packed filter [Co/16][Ci/16][tap][16 ci][16 co] -> signed bytes in
+// MFMA operand order [Co/16][S_pad][16 co][16 ci] (S = taps * Ci/16 steps, padded to a multiple of 4 with zeros),
+// followed at prepared_table_offset_u8() by the int32 prefix table P[(kh+1)*(kw+1)][Co] of the per-tap filter sums
+size_t prepared_bytes_u8(int kh, int kw, int Co, int Ci);
+size_t prepared_table_offset_u8(int kh, int kw, int Co, int Ci);
+int prepare_filter_u8(int kh, int kw, int Co, int Ci, const uint8_t *filt, void *ws, hipStream_t s);
+
 inline hipStream_t as_stream(small_hip_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool pads_ok(int t, int b, int l, int r)

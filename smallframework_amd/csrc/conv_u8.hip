@@ -659,6 +659,21 @@ int fuse_check(const char *op, const uint8_t *accum_input, const small_hip_quant
 
 } // namespace
 
+namespace shp
+{
+// the filter pre-pass for other translation units (the whole-model kernel prepares its layers with it)
+size_t prepared_bytes_u8(int kh, int kw, int Co, int Ci) { return prepared_bytes(kh, kw, Co, Ci); }
+size_t prepared_table_offset_u8(int kh, int kw, int Co, int Ci)
+{
+    const int S = kh * kw * (Ci / CB), S_pad = (S + 3) & ~3;
+    return ws_ft_bytes(Co, S_pad);
+}
+int prepare_filter_u8(int kh, int kw, int Co, int Ci, const uint8_t *filt, void *ws, hipStream_t s)
+{
+    return prepare_filter(kh, kw, Co, Ci, filt, ws, s);
+}
+} // namespace shp
+
 extern "C" {
 
 int small_hip_conv2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,

@@ -1,4 +1,4 @@
-// Device-side requantisation int32 -> uint8, bit-for-bit the reference's
+// Requantisation int32 -> uint8 (device code; also callable on the host for tables built at set-up), bit-for-bit the reference's
 // VQRDMULH + RNDRSHIFT + clamp (include/small/platforms/reference/intrinsics_quint8.h:481-531).
 #pragma once
 
@@ -22,7 +22,7 @@ inline QOut make_qout(int32_t multiplier, int32_t lshift, int32_t rshift)
     return QOut{multiplier, lshift, rshift, (multiplier > 0 && rshift >= 0 && rshift <= 30) ? 1 : 0};
 }
 
-__device__ __forceinline__ int32_t requant_i32(int32_t acc, const QOut q)
+__host__ __device__ __forceinline__ int32_t requant_i32(int32_t acc, const QOut q)
 {
     // val * (1 << lshift) in 32-bit wrap-around arithmetic, then widened to 64 bits
     const int32_t shifted = (int32_t)((uint32_t)acc << (q.lshift & 31));
@@ -50,7 +50,7 @@ __device__ __forceinline__ int32_t requant_i32(int32_t acc, const QOut q)
 //     occur, truncation equals the arithmetic shift, v = (product + 2^30) >> 31 fits 31 bits, and
 //     the rounding term is -1 exactly when (v & mask) > (mask >> 1).
 // About 10 instructions instead of 25; these kernels are bound by this arithmetic.
-__device__ __forceinline__ uint32_t requant_u8(int32_t acc, const QOut q)
+__host__ __device__ __forceinline__ uint32_t requant_u8(int32_t acc, const QOut q)
 {
     if (q.fast)
     {

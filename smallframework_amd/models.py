@@ -544,6 +544,68 @@ class HipExecutor:
         for entry in self.plan:
             self.run_entry(entry, st)
 
+    # ---- the whole model in one launch (uint8 models whose tensors and filters fit one CU's LDS) --------------
+    def qmodel_layers(self):
+        """The fused plan as small_hip_qlayer records: Conv2D [+ Accum] [+ ReLU], whole-image pooling, dense as the
+        1x1 convolution on a 1x1 image.  Buffer names become tensor ids; raises ValueError for anything else."""
+        if self.model.dtype != "u8":
+            raise ValueError("one-launch models are uint8")
+        ids = {"in": capi.QM_INPUT}
+        n = len(self.plan)
+        layers = (capi.QLayer * n)()
+        q = self.model.quant
+        for i, (op, acc_op, relu) in enumerate(self.plan):
+            L = layers[i]
+            L.src = ids[op.src] if op.src in ids else ids.setdefault(op.src, len(ids) - 1)
+            L.dst = capi.QM_OUTPUT if i == n - 1 else (ids[op.dst] if op.dst in ids else ids.setdefault(op.dst, len(ids) - 1))
+            L.accum_src, L.relu = capi.QM_NONE, int(bool(relu))
+            L.input_channels, L.input_height, L.input_width = op.C, op.H, op.W
+            L.input_q, L.output_q = capi.Quant(*q[op.src]), capi.Quant(*q[op.dst])
+            if op.kind in ("conv", "dense"):
+                L.kind = capi.QL_CONV
+                kh, kw, s = (op.kh, op.kw, op.stride) if op.kind == "conv" else (1, 1, 1)
+                L.kernel_height, L.kernel_width, L.stride = kh, kw, s
+                L.t_pad, L.b_pad, L.l_pad, L.r_pad = op.pads
+                L.output_channels = op.Co
+                L.filter = self.w[op.weight].data_ptr()
+                L.filter_q = capi.Quant(*q[op.weight])
+                if acc_op is not None:
+                    L.accum_src = ids[acc_op.src]
+                    L.accum_q = capi.Quant(*q[acc_op.src])
+            elif op.kind in ("avgpool", "maxpool") and acc_op is None and not relu:
+                L.kind = capi.QL_GLOBAL_AVGPOOL if op.kind == "avgpool" else capi.QL_GLOBAL_MAXPOOL
+                L.kernel_height, L.kernel_width, L.stride = op.kh, op.kw, op.stride
+                L.t_pad, L.b_pad, L.l_pad, L.r_pad = op.pads
+                L.output_channels = op.C
+            else:
+                raise ValueError("no one-launch form for %s" % op.name)
+        return layers
+
+    def build_one_launch(self):
+        """small_hip_qmodel_create on this model's layers; -> handle (kept in self.qmodel)."""
+        layers = self.qmodel_layers()
+        h = C.c_void_p()
+        capi.check(self.lib.small_hip_qmodel_create(len(layers), layers, C.byref(h), self.stream()))
+        self.qmodel = h
+        op = self.model.ops[-1]
+        c, hh, ww = op.out_shape()
+        assert self.lib.small_hip_qmodel_output_bytes(h) == c * hh * ww
+        self.one_out = self.torch.zeros(self.batch * c * hh * ww, dtype=self.tdtype, device="cuda")
+        return h
+
+    def forward_one_launch(self):
+        capi.check(self.lib.small_hip_qmodel_forward(self.qmodel, self.batch, self._p(self.buf["in"]),
+                                                     self._p(self.one_out), self.stream()))
+
+    def output_one_launch(self):
+        self.torch.cuda.synchronize()
+        return self.one_out.cpu().numpy()
+
+    def close(self):
+        if getattr(self, "qmodel", None):
+            self.lib.small_hip_qmodel_destroy(self.qmodel)
+            self.qmodel = None
+
     def capture(self):
         """Record one forward pass into a HIP graph (the launches go to the capture stream through the
         same C ABI calls).  Needs the prepared-filter path for uint8 models: capture must not allocate."""
