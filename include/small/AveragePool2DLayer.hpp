@@ -3,6 +3,8 @@
 // input shape is honoured.
 #pragma once
 
+#include <type_traits>
+
 #include "Layer.hpp"
 
 namespace small
@@ -32,6 +34,24 @@ public:
                       m_window.l, m_window.r, (int)m_input_shape[CHANNEL], (int)m_input_shape[HEIGHT],
                       (int)m_input_shape[WIDTH], input[0]->buffer(), output->buffer());
         output->set_shape(this->output_shape());
+    }
+
+    virtual bool one_launch(small_hip_qlayer &d) const
+    {
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            d.kind = SMALL_HIP_QL_GLOBAL_AVGPOOL;
+            d.accum_src = SMALL_HIP_QM_NONE;
+            d.relu = 0;
+            d.kernel_height = (int)m_window.kh; d.kernel_width = (int)m_window.kw; d.stride = (int)m_window.stride;
+            d.t_pad = m_window.t; d.b_pad = m_window.b; d.l_pad = m_window.l; d.r_pad = m_window.r;
+            d.output_channels = d.input_channels = (int)m_input_shape[CHANNEL];
+            d.input_height = (int)m_input_shape[HEIGHT]; d.input_width = (int)m_input_shape[WIDTH];
+            d.filter = nullptr;
+            return true;
+        }
+        else
+            return false;
     }
 
 private:

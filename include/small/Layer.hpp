@@ -30,6 +30,12 @@ public:
     // inputs by value so that callers can write compute_output({&in}, &out)
     virtual void compute_output(std::vector<Tensor<BufferT> const *> input, Tensor<BufferT> *output) const = 0;
 
+    // This layer as one record of a whole-model launch (small_hip_qmodel_create): kind, window, channels, filter and
+    // its quantisation, ReLU flag; accum_src = ONE_LAUNCH_ACCUM_ONTO_OUTPUT when the layer accumulates onto its output
+    // tensor.  The model fills in tensor ids and the tensors' quantisation.  false: the layer has no such form.
+    static constexpr int ONE_LAUNCH_ACCUM_ONTO_OUTPUT = -100;
+    virtual bool one_launch(small_hip_qlayer &) const { return false; }
+
 protected:
     void set_output_shape(shape_type const &output_shape)
     {

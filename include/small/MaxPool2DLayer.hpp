@@ -3,6 +3,8 @@
 // input shape is honoured.
 #pragma once
 
+#include <type_traits>
+
 #include "Layer.hpp"
 
 namespace small
@@ -36,6 +38,24 @@ public:
 
     // window geometry (kernel, stride, pads from the padding type)
     detail::Window const &window() const { return m_window; }
+
+    virtual bool one_launch(small_hip_qlayer &d) const
+    {
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            d.kind = SMALL_HIP_QL_GLOBAL_MAXPOOL;
+            d.accum_src = SMALL_HIP_QM_NONE;
+            d.relu = 0;
+            d.kernel_height = (int)m_window.kh; d.kernel_width = (int)m_window.kw; d.stride = (int)m_window.stride;
+            d.t_pad = m_window.t; d.b_pad = m_window.b; d.l_pad = m_window.l; d.r_pad = m_window.r;
+            d.output_channels = d.input_channels = (int)m_input_shape[CHANNEL];
+            d.input_height = (int)m_input_shape[HEIGHT]; d.input_width = (int)m_input_shape[WIDTH];
+            d.filter = nullptr;
+            return true;
+        }
+        else
+            return false;
+    }
 
 private:
     shape_type const m_input_shape;

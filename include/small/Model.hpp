@@ -2,13 +2,28 @@
 // include/small/Model.hpp:22-94).  Output tensors stay owned by the model.
 #pragma once
 
+#include <cstdlib>
 #include <memory>
+#include <type_traits>
 #include <vector>
 
 #include "Layer.hpp"
 
 namespace small
 {
+
+namespace detail
+{
+// one compute_output() call of a model's forward pass: layer, the tensor it reads, the tensor it writes (an
+// accumulating layer adds onto the tensor it writes)
+template <typename BufferT>
+struct LaunchStep
+{
+    Layer<BufferT> const *layer;
+    Tensor<BufferT> const *src;
+    Tensor<BufferT> *dst;
+};
+} // namespace detail
 
 template <typename BufferT>
 class Model
@@ -22,7 +37,15 @@ public:
     virtual ~Model()
     {
         for (auto *layer : m_layers) delete layer;
+        if (m_qmodel) (void)small_hip_qmodel_destroy(m_qmodel);
     }
+
+    // Quantised models whose tensors and filters fit one compute unit's LDS run their whole forward pass as ONE launch
+    // (small_hip_qmodel_forward), bit-identical to the layer-by-layer calls; only the returned tensor is written.
+    // false: always layer by layer (also selected by SMALL_HIP_ONE_LAUNCH=0 in the environment).
+    void set_one_launch(bool on) { m_one_launch = on; }
+    // true once inference() has planned (and used) the one-launch form
+    bool one_launch_planned() const { return m_qmodel != nullptr; }
 
     shape_type const &get_input_shape() const { return m_input_shape; }
 
@@ -52,8 +75,81 @@ protected:
         return layer;
     }
 
+    // Runs `steps` (the forward pass as the sequence of compute_output() calls, first step reading the model input,
+    // last step writing the result) as one launch.  The launch is planned on first use and again whenever the
+    // quantisation fields of a tensor change (they travel with the buffers, so they are only known at call time).
+    // false: this model has no such form (a layer kind, padding or size the launch does not cover; float32) and
+    // nothing was computed: the caller issues the layers one by one.
+    bool forward_one_launch(std::vector<detail::LaunchStep<BufferT>> const &steps)
+    {
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            if (!m_one_launch || steps.empty()) return false;
+            if (steps.front().src->shape() != m_input_shape)
+                throw std::invalid_argument("Model::inference() ERROR: incorrect input buffer shape.");
+            // tensor ids in order of first use; the model input and the last destination have their own names
+            std::vector<Tensor<BufferT> const *> ids;
+            auto id_of = [&](Tensor<BufferT> const *t) {
+                for (size_t i = 0; i < ids.size(); ++i)
+                    if (ids[i] == t) return (int)i;
+                ids.push_back(t);
+                return (int)ids.size() - 1;
+            };
+            std::vector<small_hip_qlayer> recs(steps.size());
+            std::vector<int32_t> sig;
+            for (size_t i = 0; i < steps.size(); ++i)
+            {
+                small_hip_qlayer &d = recs[i];
+                if (!steps[i].layer->one_launch(d)) return false;
+                d.src = i == 0 ? SMALL_HIP_QM_INPUT : id_of(steps[i].src);
+                const int dst = id_of(steps[i].dst);
+                d.dst = i + 1 == steps.size() ? SMALL_HIP_QM_OUTPUT : dst;
+                d.input_q = steps[i].src->buffer().quant();
+                d.output_q = steps[i].dst->buffer().quant();
+                d.accum_q = d.output_q;
+                if (d.accum_src == Layer<BufferT>::ONE_LAUNCH_ACCUM_ONTO_OUTPUT) d.accum_src = dst;
+                for (small_hip_quant const &q : {d.input_q, d.output_q})
+                    sig.insert(sig.end(), {q.zero, q.multiplier, (int32_t)q.lshift, (int32_t)q.rshift});
+            }
+            if (!m_qmodel || sig != m_qsig)
+            {
+                if (m_qmodel) (void)small_hip_qmodel_destroy(m_qmodel);
+                m_qmodel = nullptr;
+                m_qsig = sig;
+                if (m_qrefused == sig) return false;
+                const int rc = small_hip_qmodel_create((int)recs.size(), recs.data(), &m_qmodel, detail::current_stream());
+                if (rc == SMALL_HIP_EINVAL || rc == SMALL_HIP_ECHANNELS || rc == SMALL_HIP_ESTRIDE)
+                {
+                    m_qrefused = sig;         // does not fit: not an error, and not worth asking again
+                    return false;
+                }
+                detail::hip_check(rc, "small_hip_qmodel_create");
+            }
+            Tensor<BufferT> *out = steps.back().dst;
+            if (out->capacity() < steps.back().layer->output_size())
+                throw std::invalid_argument("Model::forward_one_launch() ERROR: insufficient output buffer space.");
+            detail::hip_check(small_hip_qmodel_forward(m_qmodel, (int)m_input_shape[BATCH], steps.front().src->buffer().device_in(),
+                                                       out->buffer().device_out(), detail::current_stream()),
+                              "small_hip_qmodel_forward");
+            out->set_shape(steps.back().layer->output_shape());
+            return true;
+        }
+        else
+            return false;
+    }
+
     shape_type m_input_shape;
     std::vector<Layer<BufferT> *> m_layers;
+
+private:
+    static bool one_launch_default()
+    {
+        char const *e = std::getenv("SMALL_HIP_ONE_LAUNCH");
+        return !(e && e[0] == '0');
+    }
+    bool m_one_launch = one_launch_default();
+    small_hip_qmodel *m_qmodel = nullptr;
+    std::vector<int32_t> m_qsig, m_qrefused;
 };
 
 } // namespace small

@@ -94,6 +94,27 @@ public:
     BufferT const &get_packed_filters() const { return m_packed_filters; }
     BufferT const &get_packed_bias() const { return m_packed_bias; }
 
+    virtual bool one_launch(small_hip_qlayer &d) const
+    {
+        if constexpr (std::is_same<BufferT, QUInt8Buffer>::value)
+        {
+            if (m_activation_type != NONE && m_activation_type != RELU) return false;
+            auto const &os = this->output_shape();
+            d.kind = SMALL_HIP_QL_CONV;
+            d.accum_src = Layer<BufferT>::ONE_LAUNCH_ACCUM_ONTO_OUTPUT;
+            d.relu = m_activation_type == RELU;
+            d.kernel_height = (int)m_window.kh; d.kernel_width = (int)m_window.kw; d.stride = (int)m_window.stride;
+            d.t_pad = m_window.t; d.b_pad = m_window.b; d.l_pad = m_window.l; d.r_pad = m_window.r;
+            d.output_channels = (int)os[CHANNEL]; d.input_channels = (int)m_input_shape[CHANNEL];
+            d.input_height = (int)m_input_shape[HEIGHT]; d.input_width = (int)m_input_shape[WIDTH];
+            d.filter = m_packed_filters.device_in();
+            d.filter_q = m_packed_filters.quant();
+            return true;
+        }
+        else
+            return false;
+    }
+
     virtual void compute_output(std::vector<Tensor<BufferT> const *> input, Tensor<BufferT> *output) const
     {
         this->check_single_input("PartialConv2DLayer", input, m_input_shape, output);

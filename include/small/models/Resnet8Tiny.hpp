@@ -66,19 +66,24 @@ public:
     virtual std::vector<Tensor<BufferT> *> inference(Tensor<BufferT> const *input_tensor)
     {
         Tensor<BufferT> *b0 = m_buffers[0].get(), *b1 = m_buffers[1].get(), *b2 = m_buffers[2].get();
+        std::vector<detail::LaunchStep<BufferT>> steps;
         size_t l = 0;
-        this->m_layers[l++]->compute_output({input_tensor}, b0);   // stem
-        this->m_layers[l++]->compute_output({b0}, b1);
-        this->m_layers[l++]->compute_output({b1}, b0);             // b0 += conv(b1), ReLU
+        auto step = [&](Tensor<BufferT> const *src, Tensor<BufferT> *dst) { steps.push_back({this->m_layers[l++], src, dst}); };
+        step(input_tensor, b0);                                    // stem
+        step(b0, b1);
+        step(b1, b0);                                              // b0 += conv(b1), ReLU
         for (int blk = 0; blk < 2; ++blk)
         {
-            this->m_layers[l++]->compute_output({b0}, b1);         // 3x3 stride 2 + ReLU
-            this->m_layers[l++]->compute_output({b0}, b2);         // 1x1 stride 2 shortcut
-            this->m_layers[l++]->compute_output({b1}, b2);         // b2 += conv(b1), ReLU
+            step(b0, b1);                                          // 3x3 stride 2 + ReLU
+            step(b0, b2);                                          // 1x1 stride 2 shortcut
+            step(b1, b2);                                          // b2 += conv(b1), ReLU
             std::swap(b0, b2);
         }
-        this->m_layers[l++]->compute_output({b0}, b1);             // pooling
-        this->m_layers[l++]->compute_output({b1}, b0);             // classifier
+        step(b0, b1);                                              // pooling
+        step(b1, b0);                                              // classifier
+        // quantised: the whole pass in one launch when it fits (only b0 is written then); else layer by layer
+        if (!this->forward_one_launch(steps))
+            for (auto const &s : steps) s.layer->compute_output({s.src}, s.dst);
         return {b0};
     }
 

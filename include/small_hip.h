@@ -387,7 +387,8 @@ typedef struct small_hip_qlayer
 {
     int kind;                      /* SMALL_HIP_QL_* */
     int src, dst;                  /* tensor ids */
-    int accum_src;                 /* tensor added to the convolution's output (small::Accum), or SMALL_HIP_QM_NONE */
+    int accum_src;                 /* tensor added to the convolution's output (small::Accum), or SMALL_HIP_QM_NONE;
+                                      may be dst itself (a residual sum accumulated in place), never src */
     int relu;                      /* small::ReLUActivation in place on the output */
     int kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad;
     int output_channels, input_channels, input_height, input_width;

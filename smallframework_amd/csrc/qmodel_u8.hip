@@ -663,7 +663,9 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
             scratch = need > scratch ? need : scratch;
             if (l.accum_src != SMALL_HIP_QM_NONE)
             {
-                if (l.accum_src < 0 || l.accum_src >= MAX_TENSORS || !written[l.accum_src] || l.accum_src == l.dst ||
+                // the Accum source may be the destination itself (a residual sum accumulated in place, as the reference's
+                // PartialConv2DLayer does): a lane reads its four bytes of it before it writes them
+                if (l.accum_src < 0 || l.accum_src >= MAX_TENSORS || !written[l.accum_src] || l.accum_src == l.src ||
                     l.dst == SMALL_HIP_QM_OUTPUT)
                 { set_error("%s: layer %d: bad Accum source", op, i); return fail(SMALL_HIP_EINVAL); }
                 posts[(size_t)i].has_accum = 1;

@@ -320,7 +320,7 @@ int stest_model_time_f32(int which, int variant, int batch, int C, int H, int W,
 // Resnet8Tiny<QUInt8Buffer>: every tensor of the model shares one set of quantisation fields per role
 // (input, filters, activations), enough to exercise the quantised layer classes end to end.
 int stest_resnet8_u8(int batch, const uint8_t *const *filters, const size_t *sizes, int nfilters, const uint8_t *in,
-                     const int32_t *in_q, const int32_t *filter_q, uint8_t *out, int *out_shape)
+                     const int32_t *in_q, const int32_t *filter_q, int one_launch, uint8_t *out, int *out_shape)
 {
     return guarded([&] {
         const small::shape_type is{(size_t)batch, 3, 32, 32};
@@ -333,9 +333,13 @@ int stest_resnet8_u8(int batch, const uint8_t *const *filters, const size_t *siz
             fl.push_back(own.back().get());
         }
         small::Resnet8Tiny<QB> m(is, fl, false, 10);
+        m.set_one_launch(one_launch != 0);
         auto x = packed_tensor<QB>(in, is);
         set_quant(x.buffer(), in_q);
         auto outs = m.inference(&x);
+        outs = m.inference(&x);          // a second pass re-uses the planned launch
+        if (m.one_launch_planned() != (one_launch != 0))
+            throw std::runtime_error("Resnet8Tiny<QUInt8Buffer>: one-launch form requested and not used (or the reverse)");
         unpack_tensor<QB>(*outs[0], out, out_shape);
     });
 }

@@ -171,7 +171,7 @@ class HipLayers(_Shim):
         s = tuple(shape)
         return out[:int(np.prod(s))].reshape(s)
 
-    def resnet8_u8(self, x, iq, filters, fq):
+    def resnet8_u8(self, x, iq, filters, fq, one_launch=True):
         n = x.shape[0]
         x = np.ascontiguousarray(x, np.uint8)
         fl = [np.ascontiguousarray(f, np.uint8).ravel() for f in filters]
@@ -180,8 +180,8 @@ class HipLayers(_Shim):
         out = np.zeros(n * 16, np.uint8)
         shape = (C.c_int * 4)()
         q = lambda t: (C.c_int32 * 4)(*t)
-        rc = self.lib.stest_resnet8_u8(C.c_int(n), ptrs, sizes, C.c_int(len(fl)), _f32p(x), q(iq), q(fq), _f32p(out),
-                                       shape)
+        rc = self.lib.stest_resnet8_u8(C.c_int(n), ptrs, sizes, C.c_int(len(fl)), _f32p(x), q(iq), q(fq),
+                                       C.c_int(int(one_launch)), _f32p(out), shape)
         self._check(rc)
         s = tuple(shape)
         return out[:int(np.prod(s))].reshape(s)

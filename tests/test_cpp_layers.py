@@ -300,12 +300,15 @@ def test_quantised_layers(hip, oracle, case, batch):
 
 
 @pytest.mark.gpu
-def test_resnet8_quantised_model(hip, oracle):
+@pytest.mark.parametrize("one_launch", [False, True], ids=["layer_by_layer", "one_launch"])
+def test_resnet8_quantised_model(hip, oracle, one_launch):
+    """Resnet8Tiny<QUInt8Buffer>::inference(): the layer-by-layer calls and the whole pass as one launch
+    (Model::forward_one_launch, which the class uses when the model fits one compute unit's LDS)."""
     batch = 4
     iq, fq = (-128, 1 << 30, 0, 0), (-128, 1 << 30, 0, 0)
     x = synth.uniform_u8(41, batch * 3 * 32 * 32).reshape(batch, 3, 32, 32)
     filters = ol.make_filters(synth, ol.resnet8_specs(), 10, dtype=np.uint8)
-    got = hip.resnet8_u8(x, iq, filters, fq)
+    got = hip.resnet8_u8(x, iq, filters, fq, one_launch=one_launch)
     want = ol.resnet8_tiny_u8(oracle, quant, x, iq, filters, fq, DEFAULT_Q)
     assert got.shape == want.shape == (batch, 16, 1, 1)
     assert_equal_exact(got, want, "Resnet8Tiny<QUInt8Buffer>")
