@@ -130,6 +130,20 @@ def time_forward(ex, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def time_forward_one_launch(ex, steps, warmup):
+    """Seconds per small_hip_qmodel_forward launch, HIP events on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        ex.forward_one_launch()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(steps):
+        ex.forward_one_launch()
+    ev1.record()
+    torch.cuda.synchronize()
+    return ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
 def time_ops(ex, steps):
     """Per-op device time (ms) from HIP events on the launch stream, the median over `steps` passes.  Float32 models are
     timed launch by launch as the forward pass issues them: a convolution that carries its 2x2 max-pool has the
@@ -433,6 +447,15 @@ def main():
     ex = models.HipExecutor(model, batch, weights, x, fused=not args.unfused)
 
     sec = time_forward(ex, args.steps, args.warmup)
+    one_launch = None
+    if model.dtype == "u8":
+        # quantised models run as ONE launch (small_hip_qmodel_forward: a workgroup per image, tensors and filters in
+        # LDS); that is the step that is reported, the layer-by-layer time stays beside it
+        ex.build_one_launch()
+        sec_layers, sec = sec, time_forward_one_launch(ex, args.steps, args.warmup)
+        one_launch = {"layer_by_layer_ms_per_step": round(sec_layers * 1e3, 4), "ms_per_step": round(sec * 1e3, 4),
+                      "TOPs": round(batch * model.flops_per_image() / sec / 1e12, 2)}
+        log("%s: layer by layer %.4f ms/step, one launch %.4f ms/step" % (model.name, sec_layers * 1e3, sec * 1e3))
     ips = batch / sec
     log("%s: %.3f ms/step, %.1f images/s" % (model.name, sec * 1e3, ips))
 
@@ -489,6 +512,20 @@ def main():
 
     extras = {"per_kernel_ms": {k: round(v["ms"], 4) for k, v in per_kernel.items()},
               "sum_of_layer_ms": round(sum(ms), 4)}
+    if one_launch:
+        # the step IS one kernel: its roofline is the whole model's arithmetic over the launch time (int8 MFMA peak);
+        # algorithmic bytes = the images in, the logits out, every filter once
+        extras["one_launch"] = one_launch
+        extras["layer_by_layer_roofline"] = roof
+        algo = batch * (model.in_shape[0] * model.in_shape[1] * model.in_shape[2] + model.ops[-1].Co) + \
+            sum(o.weight_elems() for o in model.ops)
+        ach = batch * model.flops_per_image() / sec / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 2), "peak": round(PEAK_MFMA_I8 / 1e12, 1), "unit": "TOP/s",
+                "frac": round(ach / (PEAK_MFMA_I8 / 1e12), 4), "traffic": None, "kernel": "qmodel_u8_kernel",
+                "launches_per_step": 1, "avg_launch_ms": round(sec * 1e3, 5),
+                "algorithmic_per_launch": {"GOP": round(batch * model.flops_per_image() / 1e9, 3),
+                                           "MB": round(algo / 1e6, 3)},
+                "note": "instruction- and latency-bound: one workgroup per image, 16 waves per compute unit"}
     if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         sustained = mfma_probe_tflops()
@@ -550,16 +587,7 @@ def main():
             s3 = (time.perf_counter() - t0) / max(args.steps, 50)
             # the whole model in one launch (one workgroup per image, tensors and filters in LDS), HIP-event timed
             e2.build_one_launch()
-            for _ in range(args.warmup):
-                e2.forward_one_launch()
-            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            n1 = max(args.steps, 50)
-            ev0.record()
-            for _ in range(n1):
-                e2.forward_one_launch()
-            ev1.record()
-            torch.cuda.synchronize()
-            s4 = ev0.elapsed_time(ev1) * 1e-3 / n1
+            s4 = time_forward_one_launch(e2, max(args.steps, 50), args.warmup)
             algo = b * (m2.in_shape[0] * m2.in_shape[1] * m2.in_shape[2] + m2.ops[-1].Co) + \
                 sum(o.weight_elems() for o in m2.ops)
             extras["%s_b%d" % (name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
@@ -632,6 +660,7 @@ def main():
         "dtype": "f32" if model.dtype == "f32" else "u8", "data": "synthetic",
         "config": {"workload": "%s forward, batch %d, %dx%dx%d input, %s" % (
             model.name, batch, model.in_shape[1], model.in_shape[2], model.in_shape[0],
+            "whole model in one launch" if one_launch else
             "Conv2D+bias+activation fused" if not args.unfused else "unfused layer calls"),
             "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4)},
         "roofline": roof,
