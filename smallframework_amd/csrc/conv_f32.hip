@@ -51,7 +51,24 @@ struct ConvArgs
     int n_blocks;        // n_co_groups * n_px_blocks
     int per_xcd;         // ceil(n_blocks / 8)
     int n_main;          // hybrid kernel: workgroups that run whole tiles (multiple of the CU count)
+    // grouped convolution: blockIdx.y walks `slabs` (image, group) slabs of Ci channels that lie in_slab / out_slab
+    // floats apart; slab y uses filter block (slab0 + y) % groups.  slabs == 0: an ordinary convolution.
+    int slabs, groups, slab0;
+    long long in_slab, out_slab, filt_slab;
 };
+
+// the arguments of this workgroup's slab (uniform per workgroup: three scalar pointer additions)
+__device__ __forceinline__ ConvArgs slab_args(ConvArgs a)
+{
+    if (a.slabs > 0)
+    {
+        const int y = blockIdx.y;
+        a.in += (long long)y * a.in_slab;
+        a.out += (long long)y * a.out_slab;
+        a.filt += (long long)((a.slab0 + y) % a.groups) * a.filt_slab;
+    }
+    return a;
+}
 
 // 64 bytes of zeros.  A masked tap (padding, a pixel past the end, a step past the last) loads from
 // here instead of being zeroed after the load: a select on the loaded value sits in the step that
@@ -379,8 +396,9 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
 // wave) makes the compiler keep the accumulators in the unified register file and pack tighter
 // (2x1: 108 -> 76 registers, 2x2: 184 -> 131, no spills); measured 1-3% faster, tighter bounds spill.
 template <int COT, int PXT, bool POOL = false>
-__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a0)
 {
+    const ConvArgs a = slab_args(a0);
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
@@ -539,8 +557,9 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
 }
 
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a0)
 {
+    const ConvArgs a = slab_args(a0);
     __shared__ float red[3][COT * PXT][16][64];
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
@@ -557,8 +576,9 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
 // 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
 // The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
 template <int COT, int PXT>
-__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a0)
 {
+    const ConvArgs a = slab_args(a0);
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
     __shared__ float red[3][1][16][64];
     const int bid = blockIdx.x;
@@ -931,7 +951,7 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT - 1) / (32 * PXT);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
 }
 
 template <int COT, int PXT>
@@ -946,16 +966,23 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     if (use_tail && rest > 0 && a.kh * a.kw * (a.Ci / CB) >= 8)
     {
         a.n_main = n_main;
-        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT), dim3(256),
-                           0, s, a);
+        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT, a.slabs > 0 ? a.slabs : 1),
+                           dim3(256), 0, s, a);
     }
     else
-        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
 }
+
+// slabs > 0: a grouped convolution, `slabs` (image, group) slabs of one launch (batch must be 1: a slab is one image
+// of Ci channels); slab y takes filter block (slab0 + y) % groups
+struct GroupSlabs
+{
+    int slabs = 0, groups = 1, slab0 = 0;
+};
 
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
              int Ci, int H, int W, const float *in, const float *filt, const float *bias, int act, float slope,
-             int accumulate, float *out, small_hip_stream_t stream)
+             int accumulate, float *out, small_hip_stream_t stream, const GroupSlabs grp = GroupSlabs{})
 {
     // interface_abstract.hpp:70-220: pick the channel branch first, the stride inside it
     const bool blocked = Ci > 0 && Ci % CB == 0;
@@ -978,6 +1005,14 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     a.Ho = out_dim(H, pt, pb, kh, stride);
     a.Wo = out_dim(W, pl, pr, kw, stride);
     a.act = act; a.slope = slope; a.accumulate = accumulate;
+    if (grp.slabs > 0)
+    {
+        if (batch != 1 || !blocked || grp.slabs > 65535) { set_error("%s: bad slab launch", op); return SMALL_HIP_EINVAL; }
+        a.slabs = grp.slabs; a.groups = grp.groups; a.slab0 = grp.slab0;
+        a.in_slab = (long long)Ci * H * W;
+        a.out_slab = (long long)Co * a.Ho * a.Wo;
+        a.filt_slab = (long long)Co * Ci * kh * kw;
+    }
     const long P = (long)batch * a.Ho * a.Wo;
     if (P == 0) return SMALL_HIP_OK;
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
@@ -1041,7 +1076,7 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     // the balanced tail in place: 2x2 only pays with many tiles per SIMD and a long reduction (big
     // 3x3 layers), 2x1 from 4 tiles per SIMD (from 2 when the reduction has at least 72 steps: 128->256 3x3 @26x26 b16, 2.6 tiles per SIMD, 74 -> 69 us; 1024->1024 1x1 @7x7 b64 with 64 steps stays 1x1: 69 against 73 us), 1x1 below (few tiles: balance matters more than
     // operand re-use).
-    const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32);
+    const long tiles32 = (long)((Co + 31) / 32) * ((P + 31) / 32) * (grp.slabs > 0 ? grp.slabs : 1);
     const long simds = 4L * NUM_CU;
     const int nsteps = kh * kw * (Ci / CB);
     int cot = 1, pxt = 1;
@@ -1200,8 +1235,8 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kh, int kw, int strid
 
 // One convolution of `channels` -> `channels` per slab of `channels` channels; slab g of image n starts
 // (n * groups + g) * channels * H * W elements into the input (the same with Ho * Wo into the output) and
-// uses filter block g.  One launch per slab: the kernels index images densely, and slabs of one group are
-// `groups` slabs apart.
+// uses filter block g.  ONE launch: the (image, group) slab is the grid's second dimension, every slab is a
+// batch-1 convolution of `channels` channels at its own offsets with its group's filter block.
 int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
                                int channels, int H, int W, const float *in, const float *filt, int accumulate,
                                float *out, small_hip_stream_t stream)
@@ -1219,11 +1254,16 @@ int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups
     // the slabs written must not overlap the slabs read (one slab's launch would read another's output)
     if (in + slabs * in_slab > out && out + slabs * out_slab > in)
     { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
-    for (size_t i = 0; i < slabs; ++i)
+    (void)filt_slab;
+    // one launch for up to 65535 slabs: the slab is the grid's second dimension
+    for (size_t i = 0; i < slabs; i += 65535)
     {
-        const int rc = conv_f32(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab,
-                                filt + (i % groups) * filt_slab, nullptr, SMALL_HIP_ACT_NONE, 0.f, accumulate ? 1 : 0,
-                                out + i * out_slab, stream);
+        GroupSlabs g;
+        g.slabs = (int)(slabs - i < 65535 ? slabs - i : 65535);
+        g.groups = groups;
+        g.slab0 = (int)(i % (size_t)groups);
+        const int rc = conv_f32(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, filt,
+                                nullptr, SMALL_HIP_ACT_NONE, 0.f, accumulate ? 1 : 0, out + i * out_slab, stream, g);
         if (rc != SMALL_HIP_OK) return rc;
     }
     return SMALL_HIP_OK;

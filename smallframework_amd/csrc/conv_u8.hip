@@ -73,7 +73,30 @@ struct QConvArgs
     QOut q;
     int P, S, S_pad, n_co_groups, n_px_blocks, n_blocks, per_xcd;
     double r_howo, r_wo, r_cib, r_kw;   // reciprocals of Ho*Wo, Wo, Ci/16, kw for udiv_rcp
+    // grouped convolution: blockIdx.y walks `slabs` (image, group) slabs that lie in_slab / out_slab bytes apart; slab y
+    // uses the prepared filter (slab0 + y) % groups, prep_slab bytes apart.  slabs == 0: an ordinary convolution.
+    int slabs, groups, slab0;
+    long long in_slab, out_slab, prep_slab;
 };
+
+struct GroupSlabs
+{
+    int slabs = 0, groups = 1, slab0 = 0;
+};
+
+__device__ __forceinline__ QConvArgs slab_args(QConvArgs a)
+{
+    if (a.slabs > 0)
+    {
+        const int y = blockIdx.y;
+        a.in += (long long)y * a.in_slab;
+        a.out += (long long)y * a.out_slab;
+        const long long f = (long long)((a.slab0 + y) % a.groups) * a.prep_slab;
+        a.ft += f;
+        a.wpre = reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(a.wpre) + f);
+    }
+    return a;
+}
 
 // ---- filter pre-pass ---------------------------------------------------------------------------
 // one lane per (co, step): reads 16 ci bytes at stride 16, writes 16 contiguous signed bytes
@@ -160,8 +183,9 @@ __device__ __align__(16) uint8_t g_bias_block[16] = {0x80, 0x80, 0x80, 0x80, 0x8
                                                     0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80, 0x80};
 
 template <int COT, int PXT>
-__global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a)
+__global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a0)
 {
+    const QConvArgs a = slab_args(a0);
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;
@@ -484,7 +508,7 @@ void launch_q(QConvArgs &a, hipStream_t s)
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
     a.use_table = a.n_blocks >= table_min_wg();
-    hipLaunchKernelGGL((conv_mfma_u8_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((conv_mfma_u8_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
 }
 
 int conv_u8_check(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
@@ -551,7 +575,7 @@ struct Fuse
 int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
                 int Ci, int H, int W, const uint8_t *in, const small_hip_quant *iq, const void *prepared,
                 const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, const Fuse &fz,
-                hipStream_t s)
+                hipStream_t s, const GroupSlabs grp = GroupSlabs{})
 {
     QConvArgs a{};
     const int CiB = Ci / CB, taps = kh * kw;
@@ -577,12 +601,21 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     if (P == 0) return SMALL_HIP_OK;
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     a.P = (int)P;
+    const long n_slabs = grp.slabs > 0 ? grp.slabs : 1;
+    if (grp.slabs > 0)
+    {
+        if (batch != 1 || grp.slabs > 65535) { set_error("%s: bad slab launch", op); return SMALL_HIP_EINVAL; }
+        a.slabs = grp.slabs; a.groups = grp.groups; a.slab0 = grp.slab0;
+        a.in_slab = (long long)Ci * H * W;
+        a.out_slab = (long long)Co * a.Ho * a.Wo;
+        a.prep_slab = (long long)prepared_bytes(kh, kw, Co, Ci);
+    }
     const int CoB = Co / CB;
     // The largest wave tile (COT channel blocks x PXT pixel groups of 16) that still leaves at least
     // `want` workgroups: these layers are small and latency-bound, so filling the chip with waves
     // comes before operand re-use.
     static const long want = [] { const char *e = std::getenv("SMALL_HIP_CONVQ_MIN_WG"); return e ? std::atol(e) : 512L; }();
-    auto nwg = [&](int cot, int pxt) { return (long)((CoB + cot - 1) / cot) * ((P + 64 * pxt - 1) / (64 * pxt)); };
+    auto nwg = [&](int cot, int pxt) { return (long)((CoB + cot - 1) / cot) * ((P + 64 * pxt - 1) / (64 * pxt)) * n_slabs; };
     if (CoB % 4 == 0 && nwg(4, 2) >= want) launch_q<4, 2>(a, s);
     else if (CoB % 2 == 0 && nwg(2, 2) >= want) launch_q<2, 2>(a, s);
     else if (nwg(1, 2) >= want) launch_q<1, 2>(a, s);
@@ -694,7 +727,8 @@ int small_hip_conv2d_u8_noalloc(int batch, int kh, int kw, int stride, int pt, i
                    fq, out, oq, Fuse{}, stream, true);
 }
 
-// The quantised form of the grouped convolution: one launch per slab of `channels` channels.
+// The quantised form of the grouped convolution: the filters of all groups prepared once, then one launch over the
+// (image, group) slabs of `channels` channels.
 int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
                               int channels, int H, int W, const uint8_t *in, const small_hip_quant *iq,
                               const uint8_t *filt, const small_hip_quant *fq, uint8_t *out,
@@ -712,10 +746,28 @@ int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups,
     const size_t slabs = (size_t)batch * groups;
     if (in + slabs * in_slab > out && out + slabs * out_slab > in)
     { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
-    for (size_t i = 0; i < slabs; ++i)
+    if (int rc = conv_u8_check(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in, filt, out, iq, fq, oq))
+        return rc;
+    if (out_slab == 0) return SMALL_HIP_OK;
+    if (out_slab / channels > (size_t)(0x7fffffffL / 64)) { set_error("%s: Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
+    // every group's filter is prepared once into the leased block, then the (image, group) slabs are the second grid
+    // dimension of ONE convolution launch (65535 slabs at most per launch)
+    hipStream_t s = as_stream(stream);
+    const size_t prep = prepared_bytes(kh, kw, channels, channels);
+    WorkspaceLease lease;
+    if (int rc = lease_workspace(prep * (size_t)groups, s, &lease)) return rc;
+    for (int g = 0; g < groups; ++g)
+        if (int rc = prepare_filter(kh, kw, channels, channels, filt + (size_t)g * filt_slab,
+                                    static_cast<uint8_t *>(lease.ptr) + (size_t)g * prep, s))
+            return rc;
+    for (size_t i = 0; i < slabs; i += 65535)
     {
-        const int rc = conv_u8(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, iq,
-                               filt + (i % groups) * filt_slab, fq, out + i * out_slab, oq, Fuse{}, stream);
+        GroupSlabs g;
+        g.slabs = (int)(slabs - i < 65535 ? slabs - i : 65535);
+        g.groups = groups;
+        g.slab0 = (int)(i % (size_t)groups);
+        const int rc = conv_u8_run(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, iq,
+                                   lease.ptr, fq, out + i * out_slab, oq, Fuse{}, s, g);
         if (rc != SMALL_HIP_OK) return rc;
     }
     return SMALL_HIP_OK;
