@@ -405,6 +405,45 @@ size_t small_hip_qmodel_output_bytes(const small_hip_qmodel *model);
 size_t small_hip_qmodel_lds_bytes(const small_hip_qmodel *model);
 int small_hip_qmodel_destroy(small_hip_qmodel *model);
 
+/* ---- a whole small float32 model in one launch ---------------------------------------------------------------
+ * No counterpart in the reference (it runs a model as its layer calls, include/small/models/DSCNNTiny.hpp:170-262
+ * being the case this is built for): one workgroup per image keeps the activation tensors in LDS and streams each
+ * layer's weights through LDS a layer ahead, so a model such as the keyword-spotting DS-CNN is one kernel instead of
+ * eleven launches.  Layers: a convolution (input channels a multiple of 16, or 1..3 on the model input; any window,
+ * stride 1 or 2, any padding) or a depthwise convolution, each with optional bias and ReLU / LeakyReLU as
+ * small_hip_conv2d_bias_act_f32 / small_hip_depthwise_conv2d_bias_act_f32 apply them, or a pooling layer whose
+ * window is the whole image; a fully connected layer is the 1x1 convolution on a 1x1 image.  Tensor ids and
+ * SMALL_HIP_QM_INPUT / SMALL_HIP_QM_OUTPUT as for small_hip_qlayer.  Limits: all activation tensors that are alive
+ * plus the weights of two consecutive layers within 160 KB, at most 48 KB of weights per layer; a model beyond
+ * them is refused with SMALL_HIP_EINVAL and a message.  small_hip_fmodel_create() copies and re-orders filters and
+ * biases (it allocates device memory and returns after its work on `stream` has finished);
+ * small_hip_fmodel_forward() is one launch and allocates nothing.  Results are within the float32 tolerance of the
+ * layer-by-layer calls (another summation order), not bit-identical to them. */
+#define SMALL_HIP_FL_CONV 0
+#define SMALL_HIP_FL_DWCONV 1
+#define SMALL_HIP_FL_GLOBAL_AVGPOOL 2
+#define SMALL_HIP_FL_GLOBAL_MAXPOOL 3
+typedef struct small_hip_flayer
+{
+    int kind;                      /* SMALL_HIP_FL_* */
+    int src, dst;                  /* tensor ids */
+    int act;                       /* SMALL_HIP_ACT_* (convolutions) */
+    float slope;                   /* LeakyReLU */
+    int kernel_height, kernel_width, stride, t_pad, b_pad, l_pad, r_pad;
+    int output_channels, input_channels, input_height, input_width;   /* depthwise: output_channels is ignored */
+    const float *filter;           /* device pointer, packed as for the layer-by-layer call; NULL for pooling */
+    const float *bias;             /* device pointer or NULL */
+} small_hip_flayer;
+typedef struct small_hip_fmodel small_hip_fmodel;
+int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_hip_fmodel **model,
+                            small_hip_stream_t stream);
+int small_hip_fmodel_forward(const small_hip_fmodel *model, int batch, const float *input, float *output,
+                             small_hip_stream_t stream);
+/* floats of one image's output / bytes of LDS the launch uses */
+size_t small_hip_fmodel_output_elems(const small_hip_fmodel *model);
+size_t small_hip_fmodel_lds_bytes(const small_hip_fmodel *model);
+int small_hip_fmodel_destroy(small_hip_fmodel *model);
+
 #ifdef __cplusplus
 }
 #endif

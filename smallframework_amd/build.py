@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libsmall_hip.so")
-SOURCES = ["runtime.hip", "layout.hip", "elementwise.hip", "pool.hip", "dwconv.hip", "conv_f32.hip", "conv_u8.hip", "qmodel_u8.hip"]
+SOURCES = ["runtime.hip", "layout.hip", "elementwise.hip", "pool.hip", "dwconv.hip", "conv_f32.hip", "conv_u8.hip", "qmodel_u8.hip", "fmodel_f32.hip"]
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from float code
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature",
          "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",

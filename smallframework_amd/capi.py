@@ -35,6 +35,16 @@ class QLayer(C.Structure):
                 ("input_q", Quant), ("filter_q", Quant), ("output_q", Quant), ("accum_q", Quant)]
 
 
+class FLayer(C.Structure):
+    """small_hip_flayer: one layer of a float32 whole-model launch (small_hip_fmodel_create)."""
+    _fields_ = [("kind", C.c_int), ("src", C.c_int), ("dst", C.c_int), ("act", C.c_int), ("slope", C.c_float),
+                ("kernel_height", C.c_int), ("kernel_width", C.c_int), ("stride", C.c_int),
+                ("t_pad", C.c_int), ("b_pad", C.c_int), ("l_pad", C.c_int), ("r_pad", C.c_int),
+                ("output_channels", C.c_int), ("input_channels", C.c_int), ("input_height", C.c_int),
+                ("input_width", C.c_int), ("filter", C.c_void_p), ("bias", C.c_void_p)]
+
+
+FL_CONV, FL_DWCONV, FL_GLOBAL_AVGPOOL, FL_GLOBAL_MAXPOOL = 0, 1, 2, 3
 QL_CONV, QL_GLOBAL_AVGPOOL, QL_GLOBAL_MAXPOOL = 0, 1, 2
 QM_INPUT, QM_OUTPUT, QM_NONE = -1, -2, -3
 
@@ -109,6 +119,11 @@ SIGNATURES = {
     "small_hip_qmodel_output_bytes": (_sz, [_p]),
     "small_hip_qmodel_lds_bytes": (_sz, [_p]),
     "small_hip_qmodel_destroy": (_i, [_p]),
+    "small_hip_fmodel_create": (_i, [_i, C.POINTER(FLayer), C.POINTER(_p), _p]),
+    "small_hip_fmodel_forward": (_i, [_p, _i, _p, _p, _p]),
+    "small_hip_fmodel_output_elems": (_sz, [_p]),
+    "small_hip_fmodel_lds_bytes": (_sz, [_p]),
+    "small_hip_fmodel_destroy": (_i, [_p]),
     "small_hip_pack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
     "small_hip_unpack": (_i, [_i, _i] + [_u32] * 6 + [_p, _p, _sz, _p]),
 }

@@ -581,21 +581,64 @@ class HipExecutor:
                 raise ValueError("no one-launch form for %s" % op.name)
         return layers
 
+    def fmodel_layers(self):
+        """The float32 model as small_hip_flayer records: convolution / depthwise convolution with their fused
+        activation, whole-image pooling, dense as the 1x1 convolution on a 1x1 image."""
+        if self.model.dtype != "f32":
+            raise ValueError("float32 models only")
+        ops = self.model.ops
+        ids = {"in": capi.QM_INPUT}
+        layers = (capi.FLayer * len(ops))()
+        act = {None: capi.ACT_NONE, "relu": capi.ACT_RELU, "leaky": capi.ACT_LEAKY}
+        for i, op in enumerate(ops):
+            L = layers[i]
+            L.src = ids[op.src] if op.src in ids else ids.setdefault(op.src, len(ids) - 1)
+            L.dst = capi.QM_OUTPUT if i == len(ops) - 1 else (ids[op.dst] if op.dst in ids else ids.setdefault(op.dst, len(ids) - 1))
+            L.input_channels, L.input_height, L.input_width = op.C, op.H, op.W
+            L.act, L.slope = act[op.act], op.slope
+            L.kernel_height, L.kernel_width, L.stride = op.kh, op.kw, op.stride
+            L.t_pad, L.b_pad, L.l_pad, L.r_pad = op.pads
+            if op.kind in ("conv", "dense"):
+                L.kind = capi.FL_CONV
+                if op.kind == "dense":
+                    L.kernel_height, L.kernel_width, L.stride = 1, 1, 1
+                L.output_channels = op.Co
+                L.filter = self.w[op.weight].data_ptr()
+            elif op.kind == "dw":
+                L.kind = capi.FL_DWCONV
+                L.output_channels = op.C
+                L.filter = self.w[op.weight].data_ptr()
+            elif op.kind in ("avgpool", "maxpool"):
+                L.kind = capi.FL_GLOBAL_AVGPOOL if op.kind == "avgpool" else capi.FL_GLOBAL_MAXPOOL
+                L.output_channels = op.C
+            else:
+                raise ValueError("no one-launch form for %s" % op.name)
+        return layers
+
     def build_one_launch(self):
-        """small_hip_qmodel_create on this model's layers; -> handle (kept in self.qmodel)."""
-        layers = self.qmodel_layers()
+        """small_hip_qmodel_create (uint8) / small_hip_fmodel_create (float32) on this model's layers; -> handle."""
         h = C.c_void_p()
-        capi.check(self.lib.small_hip_qmodel_create(len(layers), layers, C.byref(h), self.stream()))
-        self.qmodel = h
         op = self.model.ops[-1]
         c, hh, ww = op.out_shape()
-        assert self.lib.small_hip_qmodel_output_bytes(h) == c * hh * ww
+        if self.model.dtype == "u8":
+            layers = self.qmodel_layers()
+            capi.check(self.lib.small_hip_qmodel_create(len(layers), layers, C.byref(h), self.stream()))
+            assert self.lib.small_hip_qmodel_output_bytes(h) == c * hh * ww
+        else:
+            layers = self.fmodel_layers()
+            capi.check(self.lib.small_hip_fmodel_create(len(layers), layers, C.byref(h), self.stream()))
+            assert self.lib.small_hip_fmodel_output_elems(h) == c * hh * ww
+        self.qmodel = h
         self.one_out = self.torch.zeros(self.batch * c * hh * ww, dtype=self.tdtype, device="cuda")
         return h
 
+    def one_launch_lds_bytes(self):
+        fn = self.lib.small_hip_qmodel_lds_bytes if self.model.dtype == "u8" else self.lib.small_hip_fmodel_lds_bytes
+        return fn(self.qmodel)
+
     def forward_one_launch(self):
-        capi.check(self.lib.small_hip_qmodel_forward(self.qmodel, self.batch, self._p(self.buf["in"]),
-                                                     self._p(self.one_out), self.stream()))
+        fn = self.lib.small_hip_qmodel_forward if self.model.dtype == "u8" else self.lib.small_hip_fmodel_forward
+        capi.check(fn(self.qmodel, self.batch, self._p(self.buf["in"]), self._p(self.one_out), self.stream()))
 
     def output_one_launch(self):
         self.torch.cuda.synchronize()
@@ -603,7 +646,7 @@ class HipExecutor:
 
     def close(self):
         if getattr(self, "qmodel", None):
-            self.lib.small_hip_qmodel_destroy(self.qmodel)
+            (self.lib.small_hip_qmodel_destroy if self.model.dtype == "u8" else self.lib.small_hip_fmodel_destroy)(self.qmodel)
             self.qmodel = None
 
     def capture(self):

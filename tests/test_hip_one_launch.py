@@ -1,6 +1,6 @@
-"""The whole quantised model in one launch (small_hip_qmodel_*): one workgroup per image, every tensor and filter in
-LDS.  Bit-exact against the CPU oracle running the same layers one after the other, and against the layer-by-layer
-GPU path."""
+"""A whole small model in one launch: one workgroup per image, tensors (and for uint8 every filter) in LDS.
+uint8 (small_hip_qmodel_*): bit-exact against the CPU oracle running the same layers one after the other, and
+against the layer-by-layer GPU path.  float32 (small_hip_fmodel_*): within the float32 bar of the oracle."""
 import ctypes as C
 
 import numpy as np
@@ -8,7 +8,7 @@ import pytest
 
 from smallframework_amd import capi, models
 from oracle.model_exec import OracleExecutor
-from util import assert_equal_exact
+from util import assert_close_f32, assert_equal_exact
 
 pytestmark = pytest.mark.gpu
 
@@ -18,7 +18,7 @@ def _run(model, batch, seed=99):
     x = models.make_input(model, batch, seed=seed)
     ex = models.HipExecutor(model, batch, w, x)
     ex.build_one_launch()
-    print("one-launch", model.name, "batch", batch, "LDS bytes", ex.lib.small_hip_qmodel_lds_bytes(ex.qmodel), flush=True)
+    print("one-launch", model.name, "batch", batch, "LDS bytes", ex.one_launch_lds_bytes(), flush=True)
     ex.forward_one_launch()
     got = ex.output_one_launch().copy()
     ex.forward()
@@ -36,3 +36,24 @@ def test_resnet8_u8_one_launch(disc, batch):
     assert_equal_exact(got, layered, "one launch vs layer by layer")
     if disc:
         assert len(np.unique(want)) > 1          # 0 and 255 both occur: the logits depend on the data
+
+
+@pytest.mark.parametrize("batch", [1, 3, 64])
+def test_dscnn_f32_one_launch(batch):
+    """The keyword-spotting DS-CNN (10x4 stride-2 stem with 4 / 5 padded rows, depthwise + pointwise blocks, average
+    pool, dense) as one launch: float32 bar against the oracle, unscaled (DS-CNN outputs are of unit scale)."""
+    got, layered, want = _run(models.dscnn(), batch)
+    assert got.shape == want.shape
+    assert_close_f32(got, want, what="DS-CNN one launch vs oracle, batch %d" % batch)
+    assert_close_f32(got, layered, what="DS-CNN one launch vs layer by layer, batch %d" % batch)
+    assert np.abs(want).max() > 0.1
+
+
+def test_fmodel_refuses_what_does_not_fit():
+    """Tiny-YOLOv2's tensors do not fit LDS: creation is refused with EINVAL and a message, nothing is launched."""
+    m = models.tiny_yolo_v2()
+    ex = models.HipExecutor(m, 1)
+    with pytest.raises(capi.SmallHipError) as e:
+        ex.build_one_launch()
+    assert e.value.status == capi.EINVAL
+    ex.close()
