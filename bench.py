@@ -448,13 +448,13 @@ def main():
 
     sec = time_forward(ex, args.steps, args.warmup)
     one_launch = None
-    if model.dtype == "u8":
-        # quantised models run as ONE launch (small_hip_qmodel_forward: a workgroup per image, tensors and filters in
-        # LDS); that is the step that is reported, the layer-by-layer time stays beside it
+    if model.dtype == "u8" or model.name == "dscnn":
+        # quantised models and the DS-CNN run as ONE launch (small_hip_qmodel_forward / small_hip_fmodel_forward: a
+        # workgroup per image, tensors in LDS); that is the step that is reported, the layer-by-layer time stays beside it
         ex.build_one_launch()
         sec_layers, sec = sec, time_forward_one_launch(ex, args.steps, args.warmup)
         one_launch = {"layer_by_layer_ms_per_step": round(sec_layers * 1e3, 4), "ms_per_step": round(sec * 1e3, 4),
-                      "TOPs": round(batch * model.flops_per_image() / sec / 1e12, 2)}
+                      "TOPs": round(batch * model.flops_per_image() / sec / 1e12, 3)}
         log("%s: layer by layer %.4f ms/step, one launch %.4f ms/step" % (model.name, sec_layers * 1e3, sec * 1e3))
     ips = batch / sec
     log("%s: %.3f ms/step, %.1f images/s" % (model.name, sec * 1e3, ips))
@@ -520,12 +520,16 @@ def main():
         algo = batch * (model.in_shape[0] * model.in_shape[1] * model.in_shape[2] + model.ops[-1].Co) + \
             sum(o.weight_elems() for o in model.ops)
         ach = batch * model.flops_per_image() / sec / 1e12
-        roof = {"bound": "mfma", "achieved": round(ach, 2), "peak": round(PEAK_MFMA_I8 / 1e12, 1), "unit": "TOP/s",
-                "frac": round(ach / (PEAK_MFMA_I8 / 1e12), 4), "traffic": None, "kernel": "qmodel_u8_kernel",
+        pk = PEAK_MFMA_I8 if model.dtype == "u8" else PEAK_MFMA_F32
+        roof = {"bound": "mfma", "achieved": round(ach, 3), "peak": round(pk / 1e12, 1),
+                "unit": "TOP/s" if model.dtype == "u8" else "TFLOP/s",
+                "frac": round(ach / (pk / 1e12), 4), "traffic": None,
+                "kernel": "qmodel_u8_kernel" if model.dtype == "u8" else "fmodel_f32_kernel",
                 "launches_per_step": 1, "avg_launch_ms": round(sec * 1e3, 5),
                 "algorithmic_per_launch": {"GOP": round(batch * model.flops_per_image() / 1e9, 3),
                                            "MB": round(algo / 1e6, 3)},
-                "note": "instruction- and latency-bound: one workgroup per image, 16 waves per compute unit"}
+                "note": "instruction-, LDS- and latency-bound: one workgroup per image, 16 waves per compute unit, only "
+                        "`batch` of the 256 compute units busy"}
     if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         sustained = mfma_probe_tflops()
@@ -613,6 +617,15 @@ def main():
             tab = layer_table(m2, b, ms2)
             extras["%s_b%d" % (m2.name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
                                                "layers": tab}
+            if m2.name == "dscnn":
+                # the whole model in one launch (small_hip_fmodel_forward: a workgroup per image, activations in LDS)
+                e2.build_one_launch()
+                s4 = time_forward_one_launch(e2, max(args.steps, 50), args.warmup)
+                extras["%s_b%d" % (m2.name, b)].update({"one_launch_ms_per_step": round(s4 * 1e3, 4),
+                                                        "one_launch_images_per_s": round(b / s4, 1),
+                                                        "one_launch_TFLOPs": round(b * m2.flops_per_image() / s4 / 1e12, 3)})
+                log("%s batch %d: ONE LAUNCH %.4f ms/step %.0f images/s" % (m2.name, b, s4 * 1e3, b / s4))
+                e2.close()
             if len(m2.ops) == 1:
                 log("%-20s batch %2d: %.4f ms  %.0f images/s  %s %.1f%% of roofline" % (
                     m2.name, b, tab[0]["ms"], b / (tab[0]["ms"] * 1e-3), tab[0]["bound"],

@@ -292,6 +292,27 @@ public:
             return false;
     }
 
+
+    virtual bool one_launch(small_hip_flayer &d) const
+    {
+        if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        {
+            if (m_activation_type == SOFTMAX) return false;
+            d.kind = SMALL_HIP_FL_CONV;
+            d.act = detail::fused_act(m_activation_type);
+            d.slope = m_slope;
+            d.kernel_height = (int)m_window.kh; d.kernel_width = (int)m_window.kw; d.stride = (int)m_window.stride;
+            d.t_pad = m_window.t; d.b_pad = m_window.b; d.l_pad = m_window.l; d.r_pad = m_window.r;
+            d.output_channels = (int)this->output_shape()[CHANNEL]; d.input_channels = (int)m_input_shape[CHANNEL];
+            d.input_height = (int)m_input_shape[HEIGHT]; d.input_width = (int)m_input_shape[WIDTH];
+            d.filter = m_packed_filters.device_in();
+            d.bias = m_packed_bias.size() > 0 ? m_packed_bias.device_in() : nullptr;
+            return true;
+        }
+        else
+            return false;
+    }
+
     virtual void compute_output(std::vector<Tensor<BufferT> const *> input, Tensor<BufferT> *output) const
     {
         this->check_single_input("Conv2DLayer", input, m_input_shape, output);

@@ -35,6 +35,8 @@ public:
     // tensor.  The model fills in tensor ids and the tensors' quantisation.  false: the layer has no such form.
     static constexpr int ONE_LAUNCH_ACCUM_ONTO_OUTPUT = -100;
     virtual bool one_launch(small_hip_qlayer &) const { return false; }
+    // the float32 form (small_hip_fmodel_create): kind, window, channels, filter, bias and activation
+    virtual bool one_launch(small_hip_flayer &) const { return false; }
 
 protected:
     void set_output_shape(shape_type const &output_shape)

@@ -57,6 +57,25 @@ public:
             return false;
     }
 
+    virtual bool one_launch(small_hip_flayer &d) const
+    {
+        if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        {
+            d.kind = SMALL_HIP_FL_GLOBAL_MAXPOOL;
+            d.act = SMALL_HIP_ACT_NONE;
+            d.slope = 0.f;
+            d.kernel_height = (int)m_window.kh; d.kernel_width = (int)m_window.kw; d.stride = (int)m_window.stride;
+            d.t_pad = m_window.t; d.b_pad = m_window.b; d.l_pad = m_window.l; d.r_pad = m_window.r;
+            d.output_channels = d.input_channels = (int)m_input_shape[CHANNEL];
+            d.input_height = (int)m_input_shape[HEIGHT]; d.input_width = (int)m_input_shape[WIDTH];
+            d.filter = nullptr;
+            d.bias = nullptr;
+            return true;
+        }
+        else
+            return false;
+    }
+
 private:
     shape_type const m_input_shape;
     detail::Window const m_window;

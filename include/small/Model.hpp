@@ -38,14 +38,17 @@ public:
     {
         for (auto *layer : m_layers) delete layer;
         if (m_qmodel) (void)small_hip_qmodel_destroy(m_qmodel);
+        if (m_fmodel) (void)small_hip_fmodel_destroy(m_fmodel);
     }
 
-    // Quantised models whose tensors and filters fit one compute unit's LDS run their whole forward pass as ONE launch
-    // (small_hip_qmodel_forward), bit-identical to the layer-by-layer calls; only the returned tensor is written.
+    // Small models whose tensors (and, quantised, filters) fit one compute unit's LDS run their whole forward pass as ONE
+    // launch: small_hip_qmodel_forward for QUInt8Buffer, bit-identical to the layer-by-layer calls;
+    // small_hip_fmodel_forward for FloatBuffer, within the float32 tolerance of them (another summation order).  Only
+    // the returned tensor is written.
     // false: always layer by layer (also selected by SMALL_HIP_ONE_LAUNCH=0 in the environment).
     void set_one_launch(bool on) { m_one_launch = on; }
     // true once inference() has planned (and used) the one-launch form
-    bool one_launch_planned() const { return m_qmodel != nullptr; }
+    bool one_launch_planned() const { return m_qmodel != nullptr || m_fmodel != nullptr; }
 
     shape_type const &get_input_shape() const { return m_input_shape; }
 
@@ -135,7 +138,44 @@ protected:
             return true;
         }
         else
-            return false;
+        {
+            if (!m_one_launch || steps.empty() || m_frefused) return false;
+            if (steps.front().src->shape() != m_input_shape)
+                throw std::invalid_argument("Model::inference() ERROR: incorrect input buffer shape.");
+            if (!m_fmodel)
+            {
+                std::vector<Tensor<BufferT> const *> ids;
+                auto id_of = [&](Tensor<BufferT> const *t) {
+                    for (size_t i = 0; i < ids.size(); ++i)
+                        if (ids[i] == t) return (int)i;
+                    ids.push_back(t);
+                    return (int)ids.size() - 1;
+                };
+                std::vector<small_hip_flayer> recs(steps.size());
+                for (size_t i = 0; i < steps.size(); ++i)
+                {
+                    if (!steps[i].layer->one_launch(recs[i])) { m_frefused = true; return false; }
+                    recs[i].src = i == 0 ? SMALL_HIP_QM_INPUT : id_of(steps[i].src);
+                    const int dst = id_of(steps[i].dst);
+                    recs[i].dst = i + 1 == steps.size() ? SMALL_HIP_QM_OUTPUT : dst;
+                }
+                const int rc = small_hip_fmodel_create((int)recs.size(), recs.data(), &m_fmodel, detail::current_stream());
+                if (rc == SMALL_HIP_EINVAL || rc == SMALL_HIP_ECHANNELS || rc == SMALL_HIP_ESTRIDE)
+                {
+                    m_frefused = true;        // does not fit: not an error, and not worth asking again
+                    return false;
+                }
+                detail::hip_check(rc, "small_hip_fmodel_create");
+            }
+            Tensor<BufferT> *out = steps.back().dst;
+            if (out->capacity() < steps.back().layer->output_size())
+                throw std::invalid_argument("Model::forward_one_launch() ERROR: insufficient output buffer space.");
+            detail::hip_check(small_hip_fmodel_forward(m_fmodel, (int)m_input_shape[BATCH], steps.front().src->buffer().device_in(),
+                                                       out->buffer().device_out(), detail::current_stream()),
+                              "small_hip_fmodel_forward");
+            out->set_shape(steps.back().layer->output_shape());
+            return true;
+        }
     }
 
     shape_type m_input_shape;
@@ -150,6 +190,8 @@ private:
     bool m_one_launch = one_launch_default();
     small_hip_qmodel *m_qmodel = nullptr;
     std::vector<int32_t> m_qsig, m_qrefused;
+    small_hip_fmodel *m_fmodel = nullptr;
+    bool m_frefused = false;
 };
 
 } // namespace small

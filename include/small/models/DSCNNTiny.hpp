@@ -65,13 +65,17 @@ public:
     virtual std::vector<Tensor<BufferT> *> inference(Tensor<BufferT> const *input_tensor)
     {
         Tensor<BufferT> *a = m_buffer_0.get(), *b = m_buffer_1.get();
+        std::vector<detail::LaunchStep<BufferT>> steps;
         size_t l = 0;
-        this->m_layers[l++]->compute_output({input_tensor}, a);
+        steps.push_back({this->m_layers[l++], input_tensor, a});
         while (l < this->m_layers.size())
         {
-            this->m_layers[l++]->compute_output({a}, b);
-            this->m_layers[l++]->compute_output({b}, a);
+            steps.push_back({this->m_layers[l++], a, b});
+            steps.push_back({this->m_layers[l++], b, a});
         }
+        // the whole pass in one launch when the model fits one compute unit's LDS (only `a` is written then)
+        if (!this->forward_one_launch(steps))
+            for (auto const &s : steps) s.layer->compute_output({s.src}, s.dst);
         return {a};
     }
 

@@ -391,10 +391,11 @@ __device__ __forceinline__ void dwpw_layer(const FMLayer &L, float *lds, const f
 #pragma unroll
         for (int c = 0; c < TC; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
         const float *arow = wl + L.w2_off + ((cg * TC * CiB * 4 + kq) * 16 + col) * 4;      // + (c * CiB + cib) * 256
-        auto multiply = [&](int cib, const float4 Bq) {
-            float4 A[TC];
+        auto filter = [&](int cib, float4 (&A)[TC]) {
 #pragma unroll
             for (int c = 0; c < TC; ++c) A[c] = *reinterpret_cast<const float4 *>(arow + (c * CiB + cib) * 256);
+        };
+        auto multiply = [&](const float4 (&A)[TC], const float4 Bq) {
             const float Bv[4] = {Bq.x, Bq.y, Bq.z, Bq.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -405,13 +406,30 @@ __device__ __forceinline__ void dwpw_layer(const FMLayer &L, float *lds, const f
                     acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(Av[j], Bv[j], acc[c], 0, 0, 0);
                 }
         };
+        // Software pipeline over the input-channel blocks: while the MFMAs of block cib run, the wave reads the filter
+        // of block cib + 1 and does that block's depthwise arithmetic.  A wave issues in order, so the overlap only
+        // happens if those instructions sit BETWEEN the MFMAs: the scheduling groups below ask for one MFMA, then a
+        // couple of LDS reads and a handful of vector instructions, sixteen times (an MFMA occupies the matrix pipe for
+        // 32 cycles = 8 issue slots).
+        float4 Ac[TC], An[TC];
+        filter(0, Ac);
         float4 Bc = depthwise();
         for (int cib = 0; cib + 1 < CiB; ++cib)
         {
-            multiply(cib, Bc);                 // MFMAs of this block ...
-            Bc = depthwise();                  // ... with the next block's depthwise arithmetic between them
+            filter(cib + 1, An);
+            multiply(Ac, Bc);
+            Bc = depthwise();
+#pragma unroll
+            for (int c = 0; c < TC; ++c) Ac[c] = An[c];
+#pragma unroll
+            for (int g = 0; g < 4 * TC; ++g)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);      // LDS reads
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);      // vector ALU
+            }
         }
-        multiply(CiB - 1, Bc);
+        multiply(Ac, Bc);
         if (!pv) continue;
 #pragma unroll
         for (int c = 0; c < TC; ++c)

@@ -141,6 +141,20 @@ def test_models(hip, oracle, name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["DSCNNTiny", "DSCNN_10x4_12", "DSCNNSquareTiny"])
+def test_dscnn_classes_layer_by_layer(hip, oracle, name, monkeypatch):
+    """The DS-CNN classes run their whole pass as one launch by default (test_models covers that form); with
+    SMALL_HIP_ONE_LAUNCH=0 they issue their layers one by one, and then equal their DAG twins bit for bit."""
+    monkeypatch.setenv("SMALL_HIP_ONE_LAUNCH", "0")
+    which, variant, fn, filters, shape = _model_case(name)
+    x = synth.normal(57, int(np.prod(shape))).reshape(shape)
+    got = hip.model_f32(which, x, filters, variant)
+    assert_close_f32(got, fn(oracle, x, filters), what=name + " layer by layer")
+    if variant == 0:
+        assert_equal_exact(hip.model_f32(which + 10, x, filters, 0), got, name + "DAG vs layer by layer")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("name", ["MobileNetTiny", "Resnet8Tiny", "DSCNNTiny", "TinyYoloV2", "AutoencoderTiny",
                                   "DSCNNSquareTiny"])
 def test_dag_twins_equal_the_sequential_models(hip, name):
@@ -151,9 +165,9 @@ def test_dag_twins_equal_the_sequential_models(hip, name):
     x = synth.normal(56, int(np.prod(shape))).reshape(shape)
     seq = hip.model_f32(which, x, filters, 0)
     dag = hip.model_f32(which + 10, x, filters, 0)
-    if name == "TinyYoloV2":
-        # the sequential class runs convolution + pooling pairs as one launch, the DAG executor layer by layer:
-        # another kernel variant, another (fixed) summation order in the last tiles
+    if name in ("TinyYoloV2", "DSCNNTiny", "DSCNNSquareTiny"):
+        # the sequential class runs convolution + pooling pairs as one launch (Tiny-YOLOv2) or the whole model as one
+        # launch (the DS-CNN classes), the DAG executor layer by layer: other kernels, another (fixed) summation order
         assert_close_f32(dag, seq, atol=1e-5 * max(1.0, float(np.abs(seq).max())), what=name + "DAG")
     else:
         assert_equal_exact(dag, seq, name + "DAG")
