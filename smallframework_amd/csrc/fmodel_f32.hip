@@ -233,15 +233,13 @@ __device__ __forceinline__ void stem_layer(const FMLayer &L, float *lds, const f
         floatx4 acc[TC];
 #pragma unroll
         for (int c = 0; c < TC; ++c) acc[c] = floatx4{0.f, 0.f, 0.f, 0.f};
-        for (int ch = 0; ch < L.chunks; ++ch)
-        {
+        // the operands of chunk ch: where its four patch elements lie (table), the elements, the filter quads
+        auto gather = [&](int ch, float4 (&A)[TC], float (&bv)[4]) {
             const int4 e4 = ktab[ch * 4 + kq];               // a | b << 8 | ci << 16 per step; -1 past the end
             const int ev[4] = {e4.x, e4.y, e4.z, e4.w};
-            float4 A[TC];
 #pragma unroll
             for (int c = 0; c < TC; ++c)
                 A[c] = *reinterpret_cast<const float4 *>(wl + ((((cg * TC + c) * L.chunks + ch) * 4 + kq) * 16 + col) * 4);
-            float bv[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
@@ -250,6 +248,8 @@ __device__ __forceinline__ void stem_layer(const FMLayer &L, float *lds, const f
                 const bool ok = pv && e >= 0 && (unsigned)ih < (unsigned)L.H && (unsigned)iw < (unsigned)L.W;
                 bv[j] = *(ok ? src + (ih * L.W + iw) * L.Ci + (e >> 16) : zero);
             }
+        };
+        auto multiply = [&](const float4 (&A)[TC], const float (&bv)[4]) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -258,7 +258,28 @@ __device__ __forceinline__ void stem_layer(const FMLayer &L, float *lds, const f
                     const float Av[4] = {A[c].x, A[c].y, A[c].z, A[c].w};
                     acc[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(Av[j], bv[j], acc[c], 0, 0, 0);
                 }
+        };
+        // chunk ch + 1 is gathered between the MFMAs of chunk ch (a wave issues in order: see dwpw_layer)
+        float4 Ac[TC], An[TC];
+        float bc[4], bn[4];
+        gather(0, Ac, bc);
+        for (int ch = 0; ch + 1 < L.chunks; ++ch)
+        {
+            gather(ch + 1, An, bn);
+            multiply(Ac, bc);
+#pragma unroll
+            for (int c = 0; c < TC; ++c) Ac[c] = An[c];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bc[j] = bn[j];
+#pragma unroll
+            for (int g = 0; g < 4 * TC; ++g)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+            }
         }
+        multiply(Ac, bc);
         if (!pv) continue;
 #pragma unroll
         for (int c = 0; c < TC; ++c)
