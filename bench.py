@@ -56,6 +56,9 @@ def table_summary(entry, batch):
     if fr:
         out["layer_frac_min"] = round(fr[0], 3)
         out["layer_frac_median"] = round(statistics.median(fr), 3)
+    fl = [r["frac_of_stream_floor"] for r in entry["layers"] if r.get("frac_of_stream_floor")]
+    if len(entry["layers"]) == 1 and fl:
+        out["of_bytes_only_kernel"] = fl[0]         # single bandwidth-bound layer: against a kernel that only moves its bytes
     for k in ("hip_graph_ms_per_step", "one_launch_ms_per_step", "one_launch_images_per_s"):
         if k in entry:
             out[k] = entry[k]
@@ -85,6 +88,11 @@ def emit(out, tag):
     if head_fr:
         summary["headline_layers"] = {"n": len(head_fr), "frac_min": round(head_fr[0], 3),
                                       "frac_median": round(statistics.median(head_fr), 3)}
+        fl = sorted(r["frac_of_stream_floor"] for r in out.get("layers", []) if r.get("frac_of_stream_floor"))
+        if fl:
+            # bandwidth-bound layers against a kernel that only moves their bytes (same place in the model)
+            summary["headline_layers"].update({"bandwidth_layers": len(fl), "of_bytes_only_kernel_min": fl[0],
+                                               "of_bytes_only_kernel_median": round(statistics.median(fl), 3)})
     for k in ("mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "hip_graph_ms_per_step",
               "host_buffers_ms_per_step", "host_buffers_images_per_s"):
         if k in extras:
@@ -200,6 +208,55 @@ def layer_table(model, batch, ms):
                      "GB/s": round(nbytes / (t * 1e-3) / 1e9, 1) if t > 0 else None,
                      "TFLOP/s": round(batch * op.flops() / (t * 1e-3) / 1e12, 2) if t > 0 and op.flops() else None})
     return rows
+
+
+def stream_floors(ex, steps):
+    """For every bandwidth-bound layer of a float32 model (depthwise convolution, pooling, activation): the time of a
+    kernel that only moves the layer's bytes (reads the input tensor, writes the output tensor: shp_probe_stream of
+    libsmall_hip_probe.so, a measurement aid outside the product library), launched where the layer is launched, i.e.
+    right after the layer that produces its input, so that the caches are in the state the layer finds.
+    -> {layer name: ms}, median over `steps`."""
+    import ctypes as C
+    import torch
+    from smallframework_amd import capi
+    path = os.path.join(os.path.dirname(capi.LIB_PATH), "libsmall_hip_probe.so")
+    if not os.path.exists(path) or ex.model.dtype != "f32":
+        return {}
+    probe = C.CDLL(path).shp_probe_stream
+    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]
+    st = ex.stream()
+    out = {}
+    for j, entry in enumerate(ex.plan):
+        op = entry[0]
+        if op.kind not in ("dw", "maxpool", "avgpool", "relu", "leaky") or entry[1] is not None:
+            continue
+        n_in, n_out = (ex.batch * e for e in op.act_elems())
+        n_in16, n_out16 = n_in // 4, min(n_out, n_in) // 4
+        src, dst = ex.buf[op.src], ex.buf[op.dst]
+        if src.data_ptr() == dst.data_ptr():
+            continue
+        ts = []
+        for _ in range(steps):
+            if j > 0:
+                ex.run_entry(ex.plan[j - 1], st)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = probe(C.c_void_p(src.data_ptr()), n_in16, C.c_void_p(dst.data_ptr()), n_out16, st)
+            e1.record()
+            if rc:
+                raise RuntimeError("shp_probe_stream: status %d" % rc)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        out[op.name] = statistics.median(ts)
+    return out
+
+
+def add_floor_column(table, floors):
+    for r in table:
+        f = floors.get(r["layer"])
+        if f and r.get("ms"):
+            r["stream_floor_ms"] = round(f, 5)
+            r["frac_of_stream_floor"] = round(f / r["ms"], 3)
 
 
 def mfma_probe_tflops(steps=5):
@@ -462,6 +519,9 @@ def main():
     # per-op device times (HIP events on the launch stream) over the same number of steps
     ms = time_ops(ex, args.steps)
     table = layer_table(model, batch, ms)
+    if not args.no_extras:
+        # what a kernel that only moves each bandwidth-bound layer's bytes takes in the same place of the model
+        add_floor_column(table, stream_floors(ex, max(5, args.steps // 2)))
     if args.library_gemm:
         log("float32 MFMA on registers only: %s TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
         log("device-to-device copy of 822 MB: %.0f GB/s read + write (published peak 8000)" % hbm_copy_gbs())
@@ -470,9 +530,12 @@ def main():
             if r["layer"] in lib_ms:
                 r["library_gemm_ms"] = round(lib_ms[r["layer"]], 5)
     for r in table:
-        log("  %-28s %9.4f ms  %-4s %6.1f%%%s" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0),
-                                                  "   library GEMM %.4f ms" % r["library_gemm_ms"]
-                                                  if "library_gemm_ms" in r else ""))
+        log("  %-28s %9.4f ms  %-4s %6.1f%%%s%s" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0),
+                                                    "   library GEMM %.4f ms" % r["library_gemm_ms"]
+                                                    if "library_gemm_ms" in r else "",
+                                                    "   bytes-only kernel %.4f ms (%.0f%% of it)" % (
+                                                        r["stream_floor_ms"], 100 * r["frac_of_stream_floor"])
+                                                    if "stream_floor_ms" in r else ""))
 
     # dominant kernel = the one with the largest summed time
     def kernel_of(op):
@@ -615,6 +678,8 @@ def main():
             s2 = time_forward(e2, args.steps, args.warmup)
             ms2 = time_ops(e2, 10)
             tab = layer_table(m2, b, ms2)
+            if b > 1:
+                add_floor_column(tab, stream_floors(e2, 5))
             extras["%s_b%d" % (m2.name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
                                                "layers": tab}
             if m2.name == "dscnn":
@@ -627,14 +692,16 @@ def main():
                 log("%s batch %d: ONE LAUNCH %.4f ms/step %.0f images/s" % (m2.name, b, s4 * 1e3, b / s4))
                 e2.close()
             if len(m2.ops) == 1:
-                log("%-20s batch %2d: %.4f ms  %.0f images/s  %s %.1f%% of roofline" % (
+                log("%-20s batch %2d: %.4f ms  %.0f images/s  %s %.1f%% of roofline%s" % (
                     m2.name, b, tab[0]["ms"], b / (tab[0]["ms"] * 1e-3), tab[0]["bound"],
-                    100 * (tab[0]["roofline_frac"] or 0)))
+                    100 * (tab[0]["roofline_frac"] or 0),
+                    "   bytes-only kernel %.4f ms" % tab[0]["stream_floor_ms"] if "stream_floor_ms" in tab[0] else ""))
             else:
                 log("%s batch %d: %.4f ms/step %.0f images/s" % (m2.name, b, s2 * 1e3, b / s2))
                 for r in tab:
-                    log("  %-28s %9.4f ms  %-4s %6.1f%%" % (r["layer"], r["ms"], r["bound"],
-                                                           100 * (r["roofline_frac"] or 0)))
+                    log("  %-28s %9.4f ms  %-4s %6.1f%%%s" % (r["layer"], r["ms"], r["bound"], 100 * (r["roofline_frac"] or 0),
+                                                             "   bytes-only kernel %.4f ms" % r["stream_floor_ms"]
+                                                             if "stream_floor_ms" in r else ""))
             del e2
             torch.cuda.empty_cache()
 
