@@ -4,8 +4,8 @@
 // A 1-D tensor is the packed 2-D tensor [C/16][rows][W][16] whose rows are independent signals: the
 // reference's `batch_size` argument is that row count (its Conv1DLayer passes shape[HEIGHT],
 // Conv1DLayer.hpp:671-690).  Every function here is therefore the 2-D kernel with a 1 x kernel_width window
-// and no vertical padding.  The 2-D kernels stride both axes alike, so more than one row is accepted with
-// stride 1 only (any stride when rows == 1); other combinations raise std::invalid_argument.
+// and no vertical padding.  The 2-D entry points stride both axes alike; several rows together with a stride other
+// than 1 go through the 1-D entry points (small_hip_conv1d_* / small_hip_pool1d_*), which stride along the width only.
 // small::batched::<Fn>(batch, ...) takes `batch` such tensors back to back.
 // The QUInt8Buffer forms (Conv1D, MaxPool1D, ReLUActivation1D) are the quantised 2-D functions on the same
 // 1 x kernel_width window; the reference's own quantised 1-D functions write unrelated bytes on its scalar build
@@ -18,12 +18,43 @@ namespace small
 {
 namespace detail
 {
+// several rows AND a stride other than 1: the case the 1-D entry points exist for
+inline bool rows_need_1d(int stride, int rows) { return rows > 1 && stride != 1; }
+
 template <class BufferT>
-inline void check_rows(const char *op, int stride, int rows)
+inline void conv1d_rows(const char *op, int batch, int k, int stride, uint8_t l_pad, uint8_t r_pad, int groups, int Co,
+                        int Ci, int rows, int width, BufferT const &in, BufferT const &filt, BufferT const &bias,
+                        ActivationType act, float slope, bool accumulate, BufferT &out)
 {
-    if (rows > 1 && stride != 1)
-        throw std::invalid_argument(std::string(op) + "<" + type_tag<BufferT>::name() +
-                                    "> ERROR: more than one row needs stride 1 on this platform.");
+    int rc;
+    if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        rc = small_hip_conv1d_f32(batch, k, stride, l_pad, r_pad, groups, Co, Ci, rows, width, in.device_in(), filt.device_in(),
+                                  bias.size() > 0 ? bias.device_in() : nullptr, (int)act, slope, accumulate ? 1 : 0,
+                                  out.device_out(), st());
+    else
+    {
+        const small_hip_quant iq = in.quant(), fq = filt.quant(), oq = out.quant();
+        rc = small_hip_conv1d_u8(batch, k, stride, l_pad, r_pad, groups, Co, Ci, rows, width, in.device_in(), &iq,
+                                 filt.device_in(), &fq, out.device_out(), &oq, st());
+    }
+    raise<BufferT>(rc, op);
+}
+
+template <class BufferT>
+inline void pool1d_rows(const char *op, bool is_max, int batch, int k, int stride, uint8_t l_pad, uint8_t r_pad, int C,
+                        int rows, int width, BufferT const &in, BufferT &out)
+{
+    int rc;
+    if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        rc = small_hip_pool1d_f32(is_max ? 1 : 0, batch, k, stride, l_pad, r_pad, C, rows, width, in.device_in(),
+                                  out.device_out(), st());
+    else
+    {
+        const small_hip_quant iq = in.quant(), oq = out.quant();
+        rc = small_hip_pool1d_u8(is_max ? 1 : 0, batch, k, stride, l_pad, r_pad, C, rows, width, in.device_in(), &iq,
+                                 out.device_out(), &oq, st());
+    }
+    raise<BufferT>(rc, op);
 }
 } // namespace detail
 
@@ -35,7 +66,9 @@ void Conv1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pa
             int input_channels, int batch_size, int input_width, BufferT const &input_buf, BufferT const &filter_buf,
             BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("Conv1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::conv1d_rows("Conv1D", batch, kernel_width, stride, l_pad, r_pad, 0, output_channels, input_channels,
+                                   batch_size, input_width, input_buf, filter_buf, BufferT(), NONE, 0.f, false, output_buf);
     try
     {
         Conv2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
@@ -50,7 +83,10 @@ void PartialConv1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8
                    int input_channels, int batch_size, int input_width, BufferT const &input_buf,
                    BufferT const &filter_buf, BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("PartialConv1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::conv1d_rows("PartialConv1D", batch, kernel_width, stride, l_pad, r_pad, 0, output_channels,
+                                   input_channels, batch_size, input_width, input_buf, filter_buf, BufferT(), NONE, 0.f, true,
+                                   output_buf);
     try
     {
         PartialConv2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
@@ -69,7 +105,10 @@ void GroupConv1D(int batch, int kernel_width, int stride, int output_groups, uin
                  int input_channels, int batch_size, int input_width, BufferT const &input_buf,
                  BufferT const &filter_buf, BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("GroupConv1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::conv1d_rows("GroupConv1D", batch, kernel_width, stride, l_pad, r_pad, output_groups, input_channels,
+                                   input_channels, batch_size, input_width, input_buf, filter_buf, BufferT(), NONE, 0.f, false,
+                                   output_buf);
     try
     {
         GroupConv2D(batch, 1, kernel_width, stride, output_groups, 0, 0, l_pad, r_pad, input_channels, batch_size,
@@ -84,7 +123,10 @@ void PartialGroupConv1D(int batch, int kernel_width, int stride, int output_grou
                         int input_channels, int batch_size, int input_width, BufferT const &input_buf,
                         BufferT const &filter_buf, BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("PartialGroupConv1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::conv1d_rows("PartialGroupConv1D", batch, kernel_width, stride, l_pad, r_pad, output_groups,
+                                   input_channels, input_channels, batch_size, input_width, input_buf, filter_buf, BufferT(),
+                                   NONE, 0.f, true, output_buf);
     try
     {
         PartialGroupConv2D(batch, 1, kernel_width, stride, output_groups, 0, 0, l_pad, r_pad, input_channels,
@@ -104,7 +146,10 @@ void Conv1D_Bias_Act(int batch, int kernel_width, int stride, uint8_t l_pad, uin
                      BufferT const &filter_buf, BufferT const &bias_buf, ActivationType act, float negative_slope,
                      BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("Conv1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::conv1d_rows("Conv1D", batch, kernel_width, stride, l_pad, r_pad, 0, output_channels, input_channels,
+                                   batch_size, input_width, input_buf, filter_buf, bias_buf, act,
+                                   negative_slope, false, output_buf);
     Conv2D_Bias_Act(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, output_channels, input_channels, batch_size,
                     input_width, input_buf, filter_buf, bias_buf, act, negative_slope, output_buf);
 }
@@ -114,7 +159,9 @@ template <class BufferT>
 void MaxPool1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels,
                int batch_size, int input_width, BufferT const &input_buf, BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("MaxPool1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::pool1d_rows("MaxPool1D", true, batch, kernel_width, stride, l_pad, r_pad, input_channels, batch_size,
+                                   input_width, input_buf, output_buf);
     try
     {
         MaxPool2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, input_channels, batch_size, input_width,
@@ -128,7 +175,9 @@ template <class BufferT, detail::if_float<BufferT> = true>
 void AveragePool1D(int batch, int kernel_width, int stride, uint8_t l_pad, uint8_t r_pad, int input_channels,
                    int batch_size, int input_width, BufferT const &input_buf, BufferT &output_buf)
 {
-    detail::check_rows<BufferT>("AveragePool1D", stride, batch_size);
+    if (detail::rows_need_1d(stride, batch_size))
+        return detail::pool1d_rows("AveragePool1D", false, batch, kernel_width, stride, l_pad, r_pad, input_channels, batch_size,
+                                   input_width, input_buf, output_buf);
     try
     {
         AveragePool2D(batch, 1, kernel_width, stride, 0, 0, l_pad, r_pad, input_channels, batch_size, input_width,

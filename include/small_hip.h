@@ -405,6 +405,29 @@ size_t small_hip_qmodel_output_bytes(const small_hip_qmodel *model);
 size_t small_hip_qmodel_lds_bytes(const small_hip_qmodel *model);
 int small_hip_qmodel_destroy(small_hip_qmodel *model);
 
+/* ---- 1-D layers on several rows ---------------------------------------------------------------------------------
+ * reference: small::Conv1D / PartialConv1D / GroupConv1D / PartialGroupConv1D (interface_abstract_1D.hpp:47, 229, 415,
+ * 1255, 1320, 1388) and small::MaxPool1D / AveragePool1D (:776, 840, 906).  A 1-D tensor is [C/16][rows][width][16]:
+ * `rows` (the reference's batch_size argument) independent signals; the 1 x k window moves by `stride` along the width
+ * only.  (With one row, or with stride 1, the 2-D entry points on a 1 x k window compute the same thing.)
+ * groups == 0: convolution output_channels <- input_channels with optional bias / activation, accumulating onto `out`
+ * when accumulate != 0; groups > 0: `groups` convolutions of input_channels -> input_channels (filter: one packed
+ * Conv2D filter per group; output_channels, bias and act are not used). */
+int small_hip_conv1d_f32(int batch, int kernel_width, int stride, int l_pad, int r_pad, int groups,
+                         int output_channels, int input_channels, int rows, int width, const float *in,
+                         const float *filter, const float *bias, int act, float slope, int accumulate, float *out,
+                         small_hip_stream_t stream);
+int small_hip_conv1d_u8(int batch, int kernel_width, int stride, int l_pad, int r_pad, int groups, int output_channels,
+                        int input_channels, int rows, int width, const uint8_t *in, const small_hip_quant *input_q,
+                        const uint8_t *filter, const small_hip_quant *filter_q, uint8_t *out,
+                        const small_hip_quant *output_q, small_hip_stream_t stream);
+/* is_max != 0: MaxPool1D, else AveragePool1D */
+int small_hip_pool1d_f32(int is_max, int batch, int kernel_width, int stride, int l_pad, int r_pad, int channels,
+                         int rows, int width, const float *in, float *out, small_hip_stream_t stream);
+int small_hip_pool1d_u8(int is_max, int batch, int kernel_width, int stride, int l_pad, int r_pad, int channels,
+                        int rows, int width, const uint8_t *in, const small_hip_quant *input_q, uint8_t *out,
+                        const small_hip_quant *output_q, small_hip_stream_t stream);
+
 /* ---- a whole small float32 model in one launch ---------------------------------------------------------------
  * No counterpart in the reference (it runs a model as its layer calls, include/small/models/DSCNNTiny.hpp:170-262
  * being the case this is built for): one workgroup per image keeps the activation tensors in LDS and streams each

@@ -119,6 +119,10 @@ SIGNATURES = {
     "small_hip_qmodel_output_bytes": (_sz, [_p]),
     "small_hip_qmodel_lds_bytes": (_sz, [_p]),
     "small_hip_qmodel_destroy": (_i, [_p]),
+    "small_hip_conv1d_f32": (_i, [_i] * 10 + [_p, _p, _p, _i, _f, _i, _p, _p]),
+    "small_hip_conv1d_u8": (_i, [_i] * 10 + [_p, _q, _p, _q, _p, _q, _p]),
+    "small_hip_pool1d_f32": (_i, [_i] * 9 + [_p, _p, _p]),
+    "small_hip_pool1d_u8": (_i, [_i] * 9 + [_p, _q, _p, _q, _p]),
     "small_hip_fmodel_create": (_i, [_i, C.POINTER(FLayer), C.POINTER(_p), _p]),
     "small_hip_fmodel_forward": (_i, [_p, _i, _p, _p, _p]),
     "small_hip_fmodel_output_elems": (_sz, [_p]),

@@ -60,6 +60,7 @@ inline int out_dim(int in, int pad_front, int pad_back, int k, int stride)
 struct Geom
 {
     int H, W, Ho, Wo, kh, kw, stride, pt, pl;
+    int stride_h;      // vertical stride: `stride` for the 2-D layers, 1 for the 1-D layers (rows are independent signals)
 };
 
 // Position of a flat pixel index in [planes][Ho][Wo].  Tensors of fewer than 2^32 pixels (all that

@@ -41,6 +41,7 @@ struct ConvArgs
     const float *bias;   // may be null
     float *out;
     int batch, Co, Ci, H, W, Ho, Wo, kh, kw, stride, pt, pl;
+    int stride_h;        // vertical stride: `stride`, or 1 for the 1-D layers (the rows are independent signals)
     int act;
     float slope;
     int accumulate;
@@ -264,7 +265,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
             pool_ok[t] = false;
             out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
         }
-        ih0[t] = oh * a.stride - a.pt;
+        ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
     }
@@ -442,7 +443,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
         const int rem = pc - n * HoWo;
         const int oh = rem / a.Wo;
         const int ow = rem - oh * a.Wo;
-        ih0[t] = oh * a.stride - a.pt;
+        ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
         out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
@@ -621,7 +622,7 @@ __global__ __launch_bounds__(256) void conv_smallci_f32_kernel(const ConvArgs a)
     const int rem = p - n * HoWo;
     const int oh = rem / a.Wo;
     const int ow = rem - oh * a.Wo;
-    const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+    const int ih0 = oh * a.stride_h - a.pt, iw0 = ow * a.stride - a.pl;
     const float *img = a.in + (size_t)n * a.H * a.W * CI;
     const float *w = a.filt + (size_t)cob * a.kh * a.kw * CI * CB;
 
@@ -743,7 +744,7 @@ __global__ __launch_bounds__(256) void conv_smallci_mfma_f32_kernel(const ConvAr
         const int rem = pc - n * HoWo;
         const int oh = rem / a.Wo;
         const int ow = rem - oh * a.Wo;
-        const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+        const int ih0 = oh * a.stride_h - a.pt, iw0 = ow * a.stride - a.pl;
 #pragma unroll
         for (int r = 0; r < KH; ++r) rowok[t][r] = pvalid[t] && (unsigned)(ih0 + r) < (unsigned)a.H;
 #pragma unroll
@@ -978,6 +979,7 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
 struct GroupSlabs
 {
     int slabs = 0, groups = 1, slab0 = 0;
+    int stride_h = 0;        // > 0: another vertical stride (1 for the 1-D layers)
 };
 
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
@@ -1002,7 +1004,8 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     a.in = in; a.filt = filt; a.bias = bias; a.out = out;
     a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W;
     a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
-    a.Ho = out_dim(H, pt, pb, kh, stride);
+    a.stride_h = grp.stride_h > 0 ? grp.stride_h : stride;
+    a.Ho = out_dim(H, pt, pb, kh, a.stride_h);
     a.Wo = out_dim(W, pl, pr, kw, stride);
     a.act = act; a.slope = slope; a.accumulate = accumulate;
     if (grp.slabs > 0)
@@ -1146,6 +1149,7 @@ int conv_pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt,
     a.in = in; a.filt = filt; a.bias = bias; a.out = out;
     a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W;
     a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
+    a.stride_h = stride;
     a.Ho = out_dim(H, pt, pb, kh, stride);
     a.Wo = out_dim(W, pl, pr, kw, stride);
     a.act = act; a.slope = slope; a.accumulate = 0;
@@ -1237,24 +1241,21 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kh, int kw, int strid
 // (n * groups + g) * channels * H * W elements into the input (the same with Ho * Wo into the output) and
 // uses filter block g.  ONE launch: the (image, group) slab is the grid's second dimension, every slab is a
 // batch-1 convolution of `channels` channels at its own offsets with its group's filter block.
-int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
-                               int channels, int H, int W, const float *in, const float *filt, int accumulate,
-                               float *out, small_hip_stream_t stream)
+static int group_conv_f32(const char *op, int batch, int kh, int kw, int stride, int stride_h, int groups, int pt, int pb, int pl,
+                          int pr, int channels, int H, int W, const float *in, const float *filt, int accumulate, float *out,
+                          small_hip_stream_t stream)
 {
-    const char *op = "small_hip_group_conv2d_f32";
     if (channels <= 0 || channels % CB != 0) return SMALL_HIP_ECHANNELS;
     if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
     if (batch <= 0 || groups <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
     { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
     if (!in || !filt || !out) { set_error("%s: null pointer", op); return SMALL_HIP_EINVAL; }
     const size_t in_slab = (size_t)channels * H * W;
-    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
-    const size_t filt_slab = (size_t)channels * channels * kh * kw;
+    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride_h ? stride_h : stride) * out_dim(W, pl, pr, kw, stride);
     const size_t slabs = (size_t)batch * groups;
-    // the slabs written must not overlap the slabs read (one slab's launch would read another's output)
+    // the slabs written must not overlap the slabs read (one slab's workgroups would read another's output)
     if (in + slabs * in_slab > out && out + slabs * out_slab > in)
     { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
-    (void)filt_slab;
     // one launch for up to 65535 slabs: the slab is the grid's second dimension
     for (size_t i = 0; i < slabs; i += 65535)
     {
@@ -1262,11 +1263,37 @@ int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups
         g.slabs = (int)(slabs - i < 65535 ? slabs - i : 65535);
         g.groups = groups;
         g.slab0 = (int)(i % (size_t)groups);
+        g.stride_h = stride_h;
         const int rc = conv_f32(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, filt,
                                 nullptr, SMALL_HIP_ACT_NONE, 0.f, accumulate ? 1 : 0, out + i * out_slab, stream, g);
         if (rc != SMALL_HIP_OK) return rc;
     }
     return SMALL_HIP_OK;
+}
+
+int small_hip_group_conv2d_f32(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
+                               int channels, int H, int W, const float *in, const float *filt, int accumulate,
+                               float *out, small_hip_stream_t stream)
+{
+    return group_conv_f32("small_hip_group_conv2d_f32", batch, kh, kw, stride, 0, groups, pt, pb, pl, pr, channels, H, W, in,
+                          filt, accumulate, out, stream);
+}
+
+// The 1-D convolutions (interface_abstract_1D.hpp:47-560, 1255-1450): `rows` independent signals of `width` samples in
+// one [C/16][rows][width][16] tensor, a 1 x k window moved by `stride` along the width only.  groups == 0: Conv1D /
+// PartialConv1D (accumulate) with optional bias and activation; groups > 0: GroupConv1D / PartialGroupConv1D of
+// input_channels -> input_channels per group (output_channels, bias and activation are not used).
+int small_hip_conv1d_f32(int batch, int k, int stride, int l_pad, int r_pad, int groups, int Co, int Ci, int rows, int width,
+                         const float *in, const float *filt, const float *bias, int act, float slope, int accumulate,
+                         float *out, small_hip_stream_t stream)
+{
+    if (groups > 0)
+        return group_conv_f32("small_hip_conv1d_f32", batch, 1, k, stride, 1, groups, 0, 0, l_pad, r_pad, Ci, rows, width, in, filt,
+                              accumulate, out, stream);
+    GroupSlabs g;
+    g.stride_h = 1;
+    return conv_f32("small_hip_conv1d_f32", batch, 1, k, stride, 0, 0, l_pad, r_pad, Co, Ci, rows, width, in, filt, bias, act,
+                    slope, accumulate ? 1 : 0, out, stream, g);
 }
 
 int small_hip_dense_f32(int batch, int No, int Ni, const float *in, const float *filt, float *out,

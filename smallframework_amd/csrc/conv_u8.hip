@@ -66,6 +66,7 @@ struct QConvArgs
     const uint8_t *accum_src; // optional shortcut tensor added after the convolution (same shape as out)
     uint8_t *out;
     int batch, Co, Ci, H, W, Ho, Wo, kh, kw, stride, pt, pl;
+    int stride_h;            // vertical stride: `stride`, or 1 for the 1-D layers
     int32_t ZI, ZF;          // zero points + 128
     int32_t zS, zO;          // zero points of the shortcut and of the output buffer (fused Accum / ReLU)
     int relu;
@@ -82,6 +83,7 @@ struct QConvArgs
 struct GroupSlabs
 {
     int slabs = 0, groups = 1, slab0 = 0;
+    int stride_h = 0;        // > 0: another vertical stride (1 for the 1-D layers)
 };
 
 __device__ __forceinline__ QConvArgs slab_args(QConvArgs a)
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(256) void conv_mfma_u8_kernel(const QConvArgs a0)
         const int rem = pc - n * HoWo;
         const int oh = udiv_rcp(rem, a.Wo, a.r_wo);
         const int ow = rem - oh * a.Wo;
-        ih0[t] = oh * a.stride - a.pt;
+        ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk;
         rem_of[t] = rem;
@@ -385,6 +387,7 @@ struct QSmallArgs
     const uint8_t *filt;
     uint8_t *out;
     int batch, Co, H, W, Ho, Wo, kh, kw, stride, pt, pl, P;
+    int stride_h;
     int32_t zi, zf;
     const uint8_t *accum_src;
     int32_t zS, zO;
@@ -410,7 +413,7 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
     const int rem = p - n * HoWo;
     const int oh = rem / a.Wo;
     const int ow = rem - oh * a.Wo;
-    const int ih0 = oh * a.stride - a.pt, iw0 = ow * a.stride - a.pl;
+    const int ih0 = oh * a.stride_h - a.pt, iw0 = ow * a.stride - a.pl;
     const uint8_t *img = a.in + (size_t)n * a.H * a.W * CI;
     const uint8_t *w = a.filt + (size_t)cob * a.kh * a.kw * CI * CB;
     uint32_t acc[CB];
@@ -591,7 +594,8 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     a.relu = fz.relu;
     a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W; a.kh = kh; a.kw = kw;
     a.stride = stride; a.pt = pt; a.pl = pl;
-    a.Ho = out_dim(H, pt, pb, kh, stride);
+    a.stride_h = grp.stride_h > 0 ? grp.stride_h : stride;
+    a.Ho = out_dim(H, pt, pb, kh, a.stride_h);
     a.Wo = out_dim(W, pl, pr, kw, stride);
     a.r_howo = 1.0 / ((double)a.Ho * a.Wo); a.r_wo = 1.0 / a.Wo;
     a.ZI = (int32_t)((uint32_t)iq->zero + 128u);
@@ -627,8 +631,9 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
 int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
             int H, int W, const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt,
             const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq, const Fuse &fz,
-            small_hip_stream_t stream, bool static_ws = false)
+            small_hip_stream_t stream, bool static_ws = false, const GroupSlabs grp = GroupSlabs{})
 {
+    const int stride_h = grp.stride_h > 0 ? grp.stride_h : stride;
     if (int rc = conv_u8_check(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt, out, iq, fq, oq))
         return rc;
     hipStream_t s = as_stream(stream);
@@ -637,7 +642,8 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         QSmallArgs a{};
         a.in = in; a.filt = filt; a.out = out; a.batch = batch; a.Co = Co; a.H = H; a.W = W;
         a.kh = kh; a.kw = kw; a.stride = stride; a.pt = pt; a.pl = pl;
-        a.Ho = out_dim(H, pt, pb, kh, stride);
+        a.stride_h = stride_h;
+        a.Ho = out_dim(H, pt, pb, kh, stride_h);
         a.Wo = out_dim(W, pl, pr, kw, stride);
         a.zi = iq->zero; a.zf = fq->zero;
         a.accum_src = fz.accum_src; a.zS = fz.zS; a.zO = oq->zero; a.relu = fz.relu;
@@ -657,7 +663,7 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         return SMALL_HIP_OK;
     }
     // refuse what conv_u8_run would refuse before anything is enqueued
-    const long P = (long)batch * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    const long P = (long)batch * out_dim(H, pt, pb, kh, stride_h) * out_dim(W, pl, pr, kw, stride);
     if (P == 0) return SMALL_HIP_OK;
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     void *ws = nullptr;
@@ -672,7 +678,7 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         ws = lease.ptr;
     }
     if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
-    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s);
+    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s, grp);
 }
 
 int fuse_check(const char *op, const uint8_t *accum_input, const small_hip_quant *accum_q, const void *out, Fuse *fz,
@@ -729,19 +735,18 @@ int small_hip_conv2d_u8_noalloc(int batch, int kh, int kw, int stride, int pt, i
 
 // The quantised form of the grouped convolution: the filters of all groups prepared once, then one launch over the
 // (image, group) slabs of `channels` channels.
-int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
-                              int channels, int H, int W, const uint8_t *in, const small_hip_quant *iq,
-                              const uint8_t *filt, const small_hip_quant *fq, uint8_t *out,
-                              const small_hip_quant *oq, small_hip_stream_t stream)
+static int group_conv_u8(const char *op, int batch, int kh, int kw, int stride, int stride_h, int groups, int pt, int pb, int pl,
+                         int pr, int channels, int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                         const uint8_t *filt, const small_hip_quant *fq, uint8_t *out, const small_hip_quant *oq,
+                         small_hip_stream_t stream)
 {
-    const char *op = "small_hip_group_conv2d_u8";
     if (channels <= 0 || channels % CB != 0) return SMALL_HIP_ECHANNELS;
     if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
     if (batch <= 0 || groups <= 0 || kh <= 0 || kw <= 0 || H <= 0 || W <= 0 || !pads_ok(pt, pb, pl, pr))
     { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
     if (!in || !filt || !out) { set_error("%s: null pointer", op); return SMALL_HIP_EINVAL; }
     const size_t in_slab = (size_t)channels * H * W;
-    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    const size_t out_slab = (size_t)channels * out_dim(H, pt, pb, kh, stride_h ? stride_h : stride) * out_dim(W, pl, pr, kw, stride);
     const size_t filt_slab = (size_t)channels * channels * kh * kw;
     const size_t slabs = (size_t)batch * groups;
     if (in + slabs * in_slab > out && out + slabs * out_slab > in)
@@ -766,11 +771,36 @@ int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups,
         g.slabs = (int)(slabs - i < 65535 ? slabs - i : 65535);
         g.groups = groups;
         g.slab0 = (int)(i % (size_t)groups);
+        g.stride_h = stride_h;
         const int rc = conv_u8_run(op, 1, kh, kw, stride, pt, pb, pl, pr, channels, channels, H, W, in + i * in_slab, iq,
                                    lease.ptr, fq, out + i * out_slab, oq, Fuse{}, s, g);
         if (rc != SMALL_HIP_OK) return rc;
     }
     return SMALL_HIP_OK;
+}
+
+int small_hip_group_conv2d_u8(int batch, int kh, int kw, int stride, int groups, int pt, int pb, int pl, int pr,
+                              int channels, int H, int W, const uint8_t *in, const small_hip_quant *iq,
+                              const uint8_t *filt, const small_hip_quant *fq, uint8_t *out,
+                              const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    return group_conv_u8("small_hip_group_conv2d_u8", batch, kh, kw, stride, 0, groups, pt, pb, pl, pr, channels, H, W, in, iq,
+                         filt, fq, out, oq, stream);
+}
+
+// The quantised 1-D convolutions (interface_abstract_1D.hpp:229, 1320): `rows` independent signals of `width` samples, a
+// 1 x k window moved by `stride` along the width only; groups > 0: the grouped form (input_channels per group).
+int small_hip_conv1d_u8(int batch, int k, int stride, int l_pad, int r_pad, int groups, int Co, int Ci, int rows, int width,
+                        const uint8_t *in, const small_hip_quant *iq, const uint8_t *filt, const small_hip_quant *fq,
+                        uint8_t *out, const small_hip_quant *oq, small_hip_stream_t stream)
+{
+    if (groups > 0)
+        return group_conv_u8("small_hip_conv1d_u8", batch, 1, k, stride, 1, groups, 0, 0, l_pad, r_pad, Ci, rows, width, in, iq,
+                             filt, fq, out, oq, stream);
+    GroupSlabs g;
+    g.stride_h = 1;
+    return conv_u8("small_hip_conv1d_u8", batch, 1, k, stride, 0, 0, l_pad, r_pad, Co, Ci, rows, width, in, iq, filt, fq, out, oq,
+                   Fuse{}, stream, false, g);
 }
 
 int small_hip_dense_u8(int batch, int No, int Ni, const uint8_t *in, const small_hip_quant *iq,

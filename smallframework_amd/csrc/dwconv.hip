@@ -342,6 +342,7 @@ int dw_check(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     if (in == out) { set_error("%s: in-place convolution is not supported", op); return SMALL_HIP_EINVAL; }
     if ((long)batch * (C / CB) > 0x7fffffffL) { set_error("%s: batch * C / 16 too large", op); return SMALL_HIP_EINVAL; }
     g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
+    g->stride_h = stride;
     g->Ho = out_dim(H, pt, pb, kh, stride);
     g->Wo = out_dim(W, pl, pr, kw, stride);
     return SMALL_HIP_OK;

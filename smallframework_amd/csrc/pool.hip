@@ -29,7 +29,7 @@ __global__ __launch_bounds__(TPB) void pool_f32_kernel(const float4 *__restrict_
     const int ow = pp.ow, oh = pp.oh;
     const size_t plane = pp.plane;                        // n * cblocks + cb
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
-    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    const int ih0 = oh * g.stride_h - g.pt, iw0 = ow * g.stride - g.pl;
     const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     if (IS_MAX && full) acc = src[((size_t)ih0 * g.W + iw0) * 4];
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(TPB) void pool_win_f32_kernel(const float4 *__restr
     const int ow = pp.ow, oh = pp.oh;
     const size_t plane = pp.plane;
     const float4 *src = in + plane * (size_t)g.H * g.W * 4 + q;
-    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    const int ih0 = oh * g.stride_h - g.pt, iw0 = ow * g.stride - g.pl;
     float4 v[KH * KW];
 #pragma unroll
     for (int a = 0; a < KH; ++a)
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(TPB) void pool_u8_kernel(const uint32_t *__restrict
     const int ow = pp.ow, oh = pp.oh;
     const size_t plane = pp.plane;
     const uint32_t *src = in + plane * (size_t)g.H * g.W * 4 + q;
-    const int ih0 = oh * g.stride - g.pt, iw0 = ow * g.stride - g.pl;
+    const int ih0 = oh * g.stride_h - g.pt, iw0 = ow * g.stride - g.pl;
     const bool full = ih0 >= 0 && iw0 >= 0 && ih0 + g.kh <= g.H && iw0 + g.kw <= g.W;
     int32_t acc[4] = {0, 0, 0, 0};
     if (IS_MAX && full)
@@ -248,7 +248,7 @@ inline bool is_global(const Geom &g, int pt, int pb, int pl, int pr)
     return g.kh == g.H && g.kw == g.W && pt == 0 && pb == 0 && pl == 0 && pr == 0 && g.H * g.W >= 16;
 }
 
-int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, int pt, int pb, int pl,
+int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, int stride_h, int pt, int pb, int pl,
                int pr, int C, int H, int W, const void *in, const void *out, Geom *g)
 {
     // interface_abstract.hpp:797-833 / 929-977: channel test first, then stride
@@ -261,17 +261,18 @@ int pool_check(const char *op, bool avg, int batch, int kh, int kw, int stride, 
     if ((long)batch * (C / CB) > 0x7fffffffL || (long)H * W > 0x7fffffffL)
     { set_error("%s: batch * C / 16 or H * W too large", op); return SMALL_HIP_EINVAL; }
     g->H = H; g->W = W; g->kh = kh; g->kw = kw; g->stride = stride; g->pt = pt; g->pl = pl;
-    g->Ho = out_dim(H, pt, pb, kh, stride);
+    g->stride_h = stride_h ? stride_h : stride;
+    g->Ho = out_dim(H, pt, pb, kh, g->stride_h);
     g->Wo = out_dim(W, pl, pr, kw, stride);
     return SMALL_HIP_OK;
 }
 
 template <bool IS_MAX>
-int pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+int pool_f32(const char *op, int batch, int kh, int kw, int stride, int stride_h, int pt, int pb, int pl, int pr, int C,
              int H, int W, const float *in, float *out, small_hip_stream_t stream)
 {
     Geom g;
-    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
+    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, stride_h, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
     const size_t total4 = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total4 == 0) return SMALL_HIP_OK;
     const float norm = (float)(1.0 / (1.0 * kh * kw));
@@ -295,13 +296,13 @@ int pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
 }
 
 template <bool IS_MAX>
-int pool_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
+int pool_u8(const char *op, int batch, int kh, int kw, int stride, int stride_h, int pt, int pb, int pl, int pr, int C,
             int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
             const small_hip_quant *oq, small_hip_stream_t stream)
 {
     if (!iq || !oq) { set_error("%s: null quantisation parameters", op); return SMALL_HIP_EINVAL; }
     Geom g;
-    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
+    if (int rc = pool_check(op, !IS_MAX, batch, kh, kw, stride, stride_h, pt, pb, pl, pr, C, H, W, in, out, &g)) return rc;
     const size_t total = (size_t)batch * C * g.Ho * g.Wo / 4;
     if (total == 0) return SMALL_HIP_OK;
     const QOut q = make_qout(oq->multiplier, oq->lshift, oq->rshift);
@@ -328,27 +329,44 @@ extern "C" {
 int small_hip_maxpool2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
                             int H, int W, const float *in, float *out, small_hip_stream_t stream)
 {
-    return pool_f32<true>("small_hip_maxpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, stream);
+    return pool_f32<true>("small_hip_maxpool2d_f32", batch, kh, kw, stride, 0, pt, pb, pl, pr, C, H, W, in, out, stream);
 }
 
 int small_hip_avgpool2d_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
                             int H, int W, const float *in, float *out, small_hip_stream_t stream)
 {
-    return pool_f32<false>("small_hip_avgpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, out, stream);
+    return pool_f32<false>("small_hip_avgpool2d_f32", batch, kh, kw, stride, 0, pt, pb, pl, pr, C, H, W, in, out, stream);
 }
 
 int small_hip_maxpool2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
                            int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
                            const small_hip_quant *oq, small_hip_stream_t stream)
 {
-    return pool_u8<true>("small_hip_maxpool2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
+    return pool_u8<true>("small_hip_maxpool2d_u8", batch, kh, kw, stride, 0, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
 }
 
 int small_hip_avgpool2d_u8(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int C,
                            int H, int W, const uint8_t *in, const small_hip_quant *iq, uint8_t *out,
                            const small_hip_quant *oq, small_hip_stream_t stream)
 {
-    return pool_u8<false>("small_hip_avgpool2d_u8", batch, kh, kw, stride, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
+    return pool_u8<false>("small_hip_avgpool2d_u8", batch, kh, kw, stride, 0, pt, pb, pl, pr, C, H, W, in, iq, out, oq, stream);
+}
+
+// The 1-D pooling layers (interface_abstract_1D.hpp:776-1100): `rows` independent signals of `width` samples in one
+// [C/16][rows][width][16] tensor, a 1 x k window moved by `stride` along the width only.
+int small_hip_pool1d_f32(int is_max, int batch, int k, int stride, int l_pad, int r_pad, int C, int rows, int width,
+                         const float *in, float *out, small_hip_stream_t stream)
+{
+    return is_max ? pool_f32<true>("small_hip_pool1d_f32", batch, 1, k, stride, 1, 0, 0, l_pad, r_pad, C, rows, width, in, out, stream)
+                  : pool_f32<false>("small_hip_pool1d_f32", batch, 1, k, stride, 1, 0, 0, l_pad, r_pad, C, rows, width, in, out, stream);
+}
+
+int small_hip_pool1d_u8(int is_max, int batch, int k, int stride, int l_pad, int r_pad, int C, int rows, int width,
+                        const uint8_t *in, const small_hip_quant *iq, uint8_t *out, const small_hip_quant *oq,
+                        small_hip_stream_t stream)
+{
+    return is_max ? pool_u8<true>("small_hip_pool1d_u8", batch, 1, k, stride, 1, 0, 0, l_pad, r_pad, C, rows, width, in, iq, out, oq, stream)
+                  : pool_u8<false>("small_hip_pool1d_u8", batch, 1, k, stride, 1, 0, 0, l_pad, r_pad, C, rows, width, in, iq, out, oq, stream);
 }
 
 } // extern "C"

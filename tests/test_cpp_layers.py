@@ -224,15 +224,21 @@ def test_one_d_functions(hip, oracle, case, kind):
     x, f, init, n_out = one_d_inputs(case, okind, 16, oracle)
     kk = 2 if kind == 5 else k
     bias = synth.normal(4, Co) if kind == 7 else None
-    if rows > 1 and s != 1 and kind not in (4, 5):
-        with pytest.raises(ValueError, match="more than one row needs stride 1"):
-            hip.one_d_f32(kind, kk, s, l, r, Co, Ci, rows, W, x, f, bias, init, n_out)
-        return
+    # several rows with stride 2 go through the 1-D entry points (small_hip_conv1d_f32 / small_hip_pool1d_f32), which
+    # stride along the width only; everything else through the 2-D kernels on a 1 x k window
     got = hip.one_d_f32(kind, kk, s, l, r, Co, Ci, rows, W, x, f, bias, init, n_out)
     if kind >= 6:
         Wo = 1 + (W + l + r - k) // s
-        rc, want = oracle.conv2d_bias_act_f32(1, 16, 1, k, s, 0, 0, l, r, Co, Ci, rows, W, x, f, bias, ol.RELU, 0.0)
-        assert rc == 0 and want.size == Co * rows * Wo
+        if rows > 1 and s != 1:
+            # row by row convolution (the oracle's 1-D function), then bias and ReLU per channel of the packed tensor
+            want = ol.one_d_f32(oracle, 0, 16, k, s, l, r, Co, Ci, rows, W, x, f, None).reshape(Co // 16, rows * Wo, 16)
+            if bias is not None:
+                want = want + np.asarray(bias, np.float32).reshape(Co // 16, 1, 16)
+            want = np.maximum(want, 0).astype(np.float32).ravel()
+        else:
+            rc, want = oracle.conv2d_bias_act_f32(1, 16, 1, k, s, 0, 0, l, r, Co, Ci, rows, W, x, f, bias, ol.RELU, 0.0)
+            assert rc == 0
+        assert want.size == Co * rows * Wo
     else:
         want = ol.one_d_f32(oracle, kind, 16, kk, s, l, r, Co, Ci, rows, W, x, f, init)
     if okind in (0, 1, 3):
@@ -244,7 +250,7 @@ def test_one_d_functions(hip, oracle, case, kind):
 @pytest.mark.gpu
 @pytest.mark.parametrize("partial", [0, 1])
 @pytest.mark.parametrize("case", [(3, 1, 1, 1, 2, 16, 1, 13), (3, 1, 1, 1, 3, 16, 3, 11), (3, 2, 0, 1, 2, 32, 1, 12),
-                                  (1, 1, 0, 0, 4, 16, 2, 9)], ids=str)
+                                  (1, 1, 0, 0, 4, 16, 2, 9), (3, 2, 0, 1, 3, 16, 4, 12), (2, 2, 0, 0, 2, 32, 3, 10)], ids=str)
 def test_group_conv1d(hip, oracle, case, partial):
     """small::GroupConv1D / PartialGroupConv1D on packed arrays against the oracle (pinned on the reference's scalar
     build in test_oracle_1d_vs_ref.py)."""
