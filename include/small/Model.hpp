@@ -42,10 +42,10 @@ public:
     }
 
     // Small models whose tensors (and, quantised, filters) fit one compute unit's LDS run their whole forward pass as ONE
-    // launch: small_hip_qmodel_forward for QUInt8Buffer, bit-identical to the layer-by-layer calls;
-    // small_hip_fmodel_forward for FloatBuffer, within the float32 tolerance of them (another summation order).  Only
-    // the returned tensor is written.
-    // false: always layer by layer (also selected by SMALL_HIP_ONE_LAUNCH=0 in the environment).
+    // launch: small_hip_qmodel_forward for QUInt8Buffer, bit-identical to the layer-by-layer calls and used by default;
+    // small_hip_fmodel_forward for FloatBuffer, within the float32 tolerance of them (another summation order) and
+    // therefore only on request.  Only the returned tensor is written.
+    // true / false: use / never use that form (environment: SMALL_HIP_ONE_LAUNCH=1 / 0).
     void set_one_launch(bool on) { m_one_launch = on; }
     // true once inference() has planned (and used) the one-launch form
     bool one_launch_planned() const { return m_qmodel != nullptr || m_fmodel != nullptr; }
@@ -182,10 +182,14 @@ protected:
     std::vector<Layer<BufferT> *> m_layers;
 
 private:
+    // QUInt8Buffer: on unless SMALL_HIP_ONE_LAUNCH=0 (the launch is bit-identical to the layer calls).  FloatBuffer: off
+    // unless SMALL_HIP_ONE_LAUNCH=1 or set_one_launch(true): its sums run in another order, and callers (the reference's
+    // own model tests among them) compare a model's output with the layer functions' bit for bit.
     static bool one_launch_default()
     {
         char const *e = std::getenv("SMALL_HIP_ONE_LAUNCH");
-        return !(e && e[0] == '0');
+        if (std::is_same<BufferT, QUInt8Buffer>::value) return !(e && e[0] == '0');
+        return e && e[0] == '1';
     }
     bool m_one_launch = one_launch_default();
     small_hip_qmodel *m_qmodel = nullptr;

@@ -768,19 +768,25 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
     static const bool fuse_off = [] { const char *e = std::getenv("SMALL_HIP_FMODEL_FUSE"); return e && e[0] == '0'; }();
     int tensor_floats[MAX_TENSORS] = {};
     int dev_src[MAX_LAYERS], dev_dst[MAX_LAYERS], n_dev = 0;
+    // where a caller's tensor id lives: a fused pair must not write the tensor it reads (callers ping-pong between two
+    // ids, so the 1x1 convolution's destination usually IS the depthwise input, whose neighbouring pixels other waves
+    // still read); its result then goes to the tensor the depthwise result would have had, and the two ids trade places
+    int phys[MAX_TENSORS];
+    for (int t = 0; t < MAX_TENSORS; ++t) phys[t] = t;
     for (int i = 0; i < n_layers; ++i)
     {
         FMLayer L = tmp[(size_t)i];
-        int src = layers[i].src, dst = layers[i].dst;
+        const int lsrc = layers[i].src, ldst = layers[i].dst;
+        int src = lsrc >= 0 ? phys[lsrc] : lsrc, dst = ldst >= 0 ? phys[ldst] : ldst;
         if (!fuse_off && L.kind == K_DW && L.kh == 3 && L.kw == 3 && i + 1 < n_layers)
         {
             const FMLayer &N = tmp[(size_t)i + 1];
             bool ok = N.kind == K_CONV && N.kh == 1 && N.kw == 1 && N.stride == 1 && N.Ho == N.H && N.Wo == N.W &&
-                      layers[i + 1].src == dst && L.blob16 + N.blob16 <= NPRE * NT;
+                      layers[i + 1].src == ldst && L.blob16 + N.blob16 <= NPRE * NT;
             for (int j = i + 2; ok && j < n_layers; ++j)      // nobody else reads the depthwise result
             {
-                if (layers[j].src == dst) ok = false;
-                if (layers[j].dst == dst) break;
+                if (layers[j].src == ldst) ok = false;
+                if (layers[j].dst == ldst) break;
             }
             if (ok)
             {
@@ -790,10 +796,18 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
                 L.bias2_off = L.w2_off + N.bias_off;
                 L.nscale2 = N.nscale;
                 L.blob16 += N.blob16;
-                dst = layers[i + 1].dst;
+                const int odst = layers[i + 1].dst;
+                if (odst >= 0 && phys[odst] == src)
+                {
+                    const int free_id = phys[ldst];
+                    phys[ldst] = phys[odst];
+                    phys[odst] = free_id;
+                }
+                dst = odst >= 0 ? phys[odst] : odst;
                 ++i;
             }
         }
+        if (dst >= 0 && dst == src) { set_error("%s: layer %d writes the tensor it reads", op, i); return fail(SMALL_HIP_EINVAL); }
         h.layer[n_dev] = L;
         dev_src[n_dev] = src; dev_dst[n_dev] = dst;
         max_blob = L.blob16 * 4 > max_blob ? L.blob16 * 4 : max_blob;

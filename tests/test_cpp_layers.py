@@ -142,16 +142,18 @@ def test_models(hip, oracle, name):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["DSCNNTiny", "DSCNN_10x4_12", "DSCNNSquareTiny"])
-def test_dscnn_classes_layer_by_layer(hip, oracle, name, monkeypatch):
-    """The DS-CNN classes run their whole pass as one launch by default (test_models covers that form); with
-    SMALL_HIP_ONE_LAUNCH=0 they issue their layers one by one, and then equal their DAG twins bit for bit."""
-    monkeypatch.setenv("SMALL_HIP_ONE_LAUNCH", "0")
+def test_dscnn_classes_one_launch(hip, oracle, name, monkeypatch):
+    """With SMALL_HIP_ONE_LAUNCH=1 (or Model::set_one_launch(true)) the float32 DS-CNN classes run their whole pass as
+    one launch (small_hip_fmodel_forward): within the float32 bar of the oracle and of the layer-by-layer result, which
+    stays the default because callers compare a model with the layer functions bit for bit."""
     which, variant, fn, filters, shape = _model_case(name)
     x = synth.normal(57, int(np.prod(shape))).reshape(shape)
+    layered = hip.model_f32(which, x, filters, variant)
+    monkeypatch.setenv("SMALL_HIP_ONE_LAUNCH", "1")
     got = hip.model_f32(which, x, filters, variant)
-    assert_close_f32(got, fn(oracle, x, filters), what=name + " layer by layer")
-    if variant == 0:
-        assert_equal_exact(hip.model_f32(which + 10, x, filters, 0), got, name + "DAG vs layer by layer")
+    assert_close_f32(got, fn(oracle, x, filters), what=name + " one launch vs oracle")
+    assert_close_f32(got, layered, what=name + " one launch vs layer by layer")
+    assert not np.array_equal(got, layered), "the one-launch form was not used (results bit-identical to the layer calls)"
 
 
 @pytest.mark.gpu
@@ -165,9 +167,9 @@ def test_dag_twins_equal_the_sequential_models(hip, name):
     x = synth.normal(56, int(np.prod(shape))).reshape(shape)
     seq = hip.model_f32(which, x, filters, 0)
     dag = hip.model_f32(which + 10, x, filters, 0)
-    if name in ("TinyYoloV2", "DSCNNTiny", "DSCNNSquareTiny"):
-        # the sequential class runs convolution + pooling pairs as one launch (Tiny-YOLOv2) or the whole model as one
-        # launch (the DS-CNN classes), the DAG executor layer by layer: other kernels, another (fixed) summation order
+    if name == "TinyYoloV2":
+        # the sequential class runs convolution + pooling pairs as one launch, the DAG executor layer by layer:
+        # another kernel variant, another (fixed) summation order in the last tiles
         assert_close_f32(dag, seq, atol=1e-5 * max(1.0, float(np.abs(seq).max())), what=name + "DAG")
     else:
         assert_equal_exact(dag, seq, name + "DAG")

@@ -57,3 +57,19 @@ def test_fmodel_refuses_what_does_not_fit():
         ex.build_one_launch()
     assert e.value.status == capi.EINVAL
     ex.close()
+
+
+@pytest.mark.parametrize("name,batch", [("dscnn", 64), ("resnet8_u8", 64)])
+def test_one_launch_repeats_bit_for_bit(name, batch):
+    """Forty launches on the same input give the same bytes: no workgroup reads a tensor another wave is still writing
+    (a fused depthwise + 1x1 layer writes its result to another LDS tensor than the one its 3x3 windows read)."""
+    m = getattr(models, name)()
+    ex = models.HipExecutor(m, batch, models.make_weights(m), models.make_input(m, batch, seed=7))
+    ex.build_one_launch()
+    ex.forward_one_launch()
+    first = ex.output_one_launch().copy()
+    for i in range(40):
+        ex.forward_one_launch()
+        again = ex.output_one_launch()
+        assert np.array_equal(again.view(np.uint8), first.view(np.uint8)), "launch %d differs from the first" % (i + 2)
+    ex.close()
