@@ -56,6 +56,11 @@ struct ConvArgs
     // floats apart; slab y uses filter block (slab0 + y) % groups.  slabs == 0: an ordinary convolution.
     int slabs, groups, slab0;
     long long in_slab, out_slab, filt_slab;
+    // equal-share split of the reduction (conv_mfma_f32_streamk_kernel): the launch's K-steps, tile after tile, are cut into
+    // sk_chunks runs of sk_chunk steps; a run that does not cover a whole tile leaves raw accumulators in sk_scratch
+    // ([tile][part < sk_parts][SK_PART_FLOATS]) for conv_streamk_fixup_kernel to add up in run order
+    int sk_chunk, sk_chunks, sk_parts;
+    float *sk_scratch;
 };
 
 // the arguments of this workgroup's slab (uniform per workgroup: three scalar pointer additions)
@@ -209,9 +214,12 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
 // the MFMA register, two 16-byte loads per lane and tile.
 constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks start 16 banks apart
 
+// s_begin / s_count: only K-steps [s_begin, s_begin + s_count) of the tile (s_count < 0: all of them); raw != nullptr: the
+// accumulators go there as they are ([wave][tile of the wave][register quad][lane] float4) instead of through the epilogue
 template <int COT, int PXT, bool POOL = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
-                                              const int cg, const int pxb)
+                                              const int cg, const int pxb, const int s_begin = 0, const int s_count = -1,
+                                              float *raw = nullptr)
 {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -303,8 +311,10 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
 
-    int ta = 0, tb = 0, cib = 0;
-    const int nsteps = taps * CiB;
+    // first step: channel block fastest, then the window column, then the row
+    const int tap0 = s_begin / CiB;
+    int cib = s_begin - tap0 * CiB, ta = tap0 / a.kw, tb = tap0 - (tap0 / a.kw) * a.kw;
+    const int nsteps = s_count < 0 ? taps * CiB : s_count;
     bool live = true;
 
     // issues the global loads of the step at (ta, tb, cib) and advances the position
@@ -389,6 +399,18 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // an odd step count leaves the last step staged in buffer 0 / B0 (the loop's invariant)
     if (nsteps & 1) multiply(0, B0);
 
+    if (raw)
+    {
+        float4 *r4 = reinterpret_cast<float4 *>(raw) + (size_t)wave * (COT * PXT * 4 * WAVE) + lane;
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    r4[((c * PXT + t) * 4 + q) * WAVE] = make_float4(acc[c][t][4 * q], acc[c][t][4 * q + 1], acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
+        return;
+    }
     if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix);
     else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
@@ -599,6 +621,90 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int px32 = (lid / a.n_co_groups) * (4 * PXT) + sub / COT;
     if (co32 * 32 >= a.Co || px32 * 32 >= a.P) return;     // uniform over the workgroup
     conv_splitk_tile<1, 1>(a, red, co32, px32);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Equal shares of the reduction for launches with few tiles and a long reduction (3x3 convolutions with 512 / 1024
+// channels on a 13x13 map: 352 workgroup tiles for 256 compute units, 288 or 576 K-steps each).  Whole tiles leave a
+// second round in which a third of the machine works; cutting only the left-over tiles four ways (the hybrid kernel) leaves
+// the first round with one wave per SIMD.  Here all K-steps of the launch, tile after tile, are cut into 2 x 256 equal runs;
+// a workgroup multiplies its run (the end of one tile and the start of the next, as a rule) with the LDS-staged body, two
+// workgroups per compute unit, all finishing together.  A run that is not a whole tile leaves its raw accumulators in a
+// scratch block; conv_streamk_fixup_kernel adds the two or three runs of a tile in run order (deterministic) and applies
+// accumulate / bias / activation.
+constexpr int SK_CHUNKS = 2 * NUM_CU;
+template <int COT, int PXT>
+constexpr int sk_part_floats() { return 4 * COT * PXT * 16 * WAVE; }
+
+template <int COT, int PXT>
+__global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_streamk_kernel(const ConvArgs a)
+{
+    __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;      // consecutive runs (the same tiles) on one XCD
+    if (lid >= a.sk_chunks) return;
+    const int nsteps = a.kh * a.kw * (a.Ci / CB);
+    const long total = (long)a.n_blocks * nsteps;
+    long k0 = (long)lid * a.sk_chunk;
+    const long k1 = k0 + a.sk_chunk < total ? k0 + a.sk_chunk : total;
+    while (k0 < k1)                                                   // uniform over the workgroup
+    {
+        const int tile = (int)(k0 / nsteps);
+        const int sb = (int)(k0 - (long)tile * nsteps);
+        const int cnt = (int)(nsteps - sb < k1 - k0 ? nsteps - sb : k1 - k0);
+        float *raw = nullptr;
+        if (cnt != nsteps)
+        {
+            const int first = (int)(((long)tile * nsteps) / a.sk_chunk);          // the run that starts the tile
+            raw = a.sk_scratch + ((size_t)tile * a.sk_parts + (lid - first)) * sk_part_floats<COT, PXT>();
+        }
+        conv_lds_tile<COT, PXT>(a, lds_a, tile % a.n_co_groups, tile / a.n_co_groups, sb, cnt, raw);
+        k0 += cnt;
+        __syncthreads();                                              // the next tile stages into the same LDS buffers
+    }
+}
+
+template <int COT, int PXT>
+__global__ __launch_bounds__(256) void conv_streamk_fixup_kernel(const ConvArgs a)
+{
+    const int tile = blockIdx.x;
+    const int nsteps = a.kh * a.kw * (a.Ci / CB);
+    const int first = (int)(((long)tile * nsteps) / a.sk_chunk);
+    const int last = (int)(((long)(tile + 1) * nsteps - 1) / a.sk_chunk);
+    if (last == first) return;                  // one run covered the whole tile and wrote it through the epilogue
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+    const int cg = tile % a.n_co_groups, pxb = tile / a.n_co_groups;
+    const int HoWo = a.Ho * a.Wo, CoB = a.Co / CB;
+    bool pvalid[PXT];
+    size_t out_pix[PXT];
+#pragma unroll
+    for (int t = 0; t < PXT; ++t)
+    {
+        const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
+        pvalid[t] = p < a.P;
+        const int pc = pvalid[t] ? p : 0;
+        const int n = pc / HoWo, rem = pc - n * HoWo;
+        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+    }
+    floatx16 acc[COT][PXT];
+    const float4 *r4 = reinterpret_cast<const float4 *>(a.sk_scratch + (size_t)tile * a.sk_parts * sk_part_floats<COT, PXT>()) +
+                       (size_t)wave * (COT * PXT * 4 * WAVE) + lane;
+    for (int part = 0; part <= last - first; ++part)
+    {
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                {
+                    const float4 v = r4[((c * PXT + t) * 4 + q) * WAVE];
+                    if (part == 0) { acc[c][t][4 * q] = v.x; acc[c][t][4 * q + 1] = v.y; acc[c][t][4 * q + 2] = v.z; acc[c][t][4 * q + 3] = v.w; }
+                    else { acc[c][t][4 * q] += v.x; acc[c][t][4 * q + 1] += v.y; acc[c][t][4 * q + 2] += v.z; acc[c][t][4 * q + 3] += v.w; }
+                }
+        r4 += sk_part_floats<COT, PXT>() / 4;
+    }
+    conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1012,6 +1118,41 @@ struct GroupSlabs
     int stride_h = 0;        // > 0: another vertical stride (1 for the 1-D layers)
 };
 
+// the equal-share launch pair; false: the shape does not qualify
+template <int COT, int PXT>
+int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
+{
+    *done = false;
+    a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
+    a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
+    a.n_blocks = a.n_co_groups * a.n_px_blocks;
+    const int nsteps = a.kh * a.kw * (a.Ci / CB);
+    const long total = (long)a.n_blocks * nsteps;
+    // few tiles that do not fill whole rounds and a long reduction (measured, batch 16 on 13x13 maps: 512 -> 1024 3x3 287 -> 264 us,
+    // 1024 -> 1024 519 -> 467 us, 256 -> 512 (144 steps) 81 -> 69 us; with 72 steps or fewer the fix-up pass costs more than
+    // the balance gains).  SMALL_HIP_CONV_STREAMK=<workgroups per compute unit> (default 2), _MIN=<steps> (default 128)
+    static const int min_steps = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK_MIN"); return e ? std::atoi(e) : 128; }();
+    static const int per_cu = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK"); const int v = e ? std::atoi(e) : 2; return v > 0 ? v : 2; }();
+    if (a.n_blocks <= NUM_CU / 2 || a.n_blocks >= 3 * NUM_CU || a.n_blocks % NUM_CU == 0 || nsteps < min_steps || a.Co % (32 * COT) != 0)
+        return SMALL_HIP_OK;
+    const int chunks = per_cu * NUM_CU;
+    a.sk_chunks = chunks;
+    a.sk_chunk = (int)((total + chunks - 1) / chunks);
+    a.sk_chunks = (int)((total + a.sk_chunk - 1) / a.sk_chunk);
+    a.sk_parts = (nsteps + a.sk_chunk - 1) / a.sk_chunk + 1;
+    a.per_xcd = (a.sk_chunks + NUM_XCD - 1) / NUM_XCD;
+    WorkspaceLease lease;            // held until both launches are enqueued
+    const size_t bytes = (size_t)a.n_blocks * a.sk_parts * sk_part_floats<COT, PXT>() * sizeof(float);
+    if (int rc = lease_workspace(bytes, s, &lease)) return rc;
+    a.sk_scratch = static_cast<float *>(lease.ptr);
+    hipLaunchKernelGGL((conv_mfma_f32_streamk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    SHP_LAUNCH_CHECK(op);
+    hipLaunchKernelGGL((conv_streamk_fixup_kernel<COT, PXT>), dim3(a.n_blocks), dim3(256), 0, s, a);
+    SHP_LAUNCH_CHECK(op);
+    *done = true;
+    return SMALL_HIP_OK;
+}
+
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
              int Ci, int H, int W, const float *in, const float *filt, const float *bias, int act, float slope,
              int accumulate, float *out, small_hip_stream_t stream, const GroupSlabs grp = GroupSlabs{})
@@ -1137,6 +1278,15 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     {
         int c2 = 0, p2 = 0;
         if (std::sscanf(e, "%d,%d", &c2, &p2) == 2) { cot = c2; pxt = p2; }
+    }
+    // few tiles, long reduction: equal shares of the K-steps (tuning knob SMALL_HIP_CONV_STREAMK=0 switches it off; the
+    // first call on a stream allocates the scratch block, like the uint8 convolution's filter pre-pass)
+    static const bool streamk_off = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK"); return e && e[0] == '0'; }();
+    if (!streamk_off && grp.slabs == 0 && Co % 64 == 0)
+    {
+        bool done = false;
+        if (int rc = launch_streamk<2, 1>(op, a, s, &done)) return rc;
+        if (done) return SMALL_HIP_OK;
     }
     if (cot == 2 && pxt == 2) launch_mfma<2, 2>(a, s);
     else if (cot == 1 && pxt == 2) launch_mfma<1, 2>(a, s);

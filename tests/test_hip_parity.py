@@ -84,6 +84,52 @@ def test_conv2d_f32(lib, oracle, case, mode):
     del cib
 
 
+# few workgroup tiles and a long reduction: the equal-share split of the K-steps (two runs per compute unit, raw
+# accumulators through a scratch block, fixed-order fix-up pass).  First case: 136 tiles x 144 steps, every tile cut into
+# four or five runs; second: 600 tiles, runs of 169 steps, so some runs hold a whole tile (written through the epilogue
+# directly) next to pieces of its neighbours; third: 5x5 window, stride 2, a ragged last pixel block.
+EQUAL_SHARE_CASES = [
+    (1, 3, 3, 1, (1, 1, 1, 1), 256, 256, 65, 65),
+    (1, 3, 3, 1, (1, 1, 1, 1), 64, 256, 240, 320),
+    (3, 5, 5, 2, (2, 2, 2, 2), 128, 96, 150, 141),
+]
+
+
+@pytest.mark.parametrize("mode", ["conv", "partial", "bias_leaky"])
+@pytest.mark.parametrize("case", EQUAL_SHARE_CASES, ids=str)
+def test_conv2d_f32_equal_share_split(lib, oracle, case, mode):
+    batch, kh, kw, s, (pt, pb, pl, pr), Co, Ci, H, W = case
+    x = synth.normal(21, batch * Ci * H * W)
+    f = synth.he_normal(22, Co * Ci * kh * kw, Ci * kh * kw)
+    Ho, Wo = oracle.out_hw(kh, kw, s, pt, pb, pl, pr, H, W)
+    # the launcher's own rule: 2 x 1 wave tiles -> 64 channels x 128 pixels per workgroup tile
+    n_tiles, steps = (Co // 64) * -(-(batch * Ho * Wo) // 128), kh * kw * Ci // 16
+    assert 128 < n_tiles < 768 and n_tiles % 256 and steps >= 128, "the case would not take the equal-share launch"
+    o0 = synth.normal(23, batch * Co * Ho * Wo)
+    bias = synth.normal(24, Co)
+    dx, df, do, db = hu.dev(x), hu.dev(f), hu.dev(o0), hu.dev(bias)
+    args = (batch, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W)
+    if mode == "conv":
+        rc = lib.small_hip_conv2d_f32(*args, hu.ptr(dx), hu.ptr(df), hu.ptr(do), hu.stream())
+        rco, want = oracle.conv2d_f32(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, f)
+    elif mode == "partial":
+        rc = lib.small_hip_partial_conv2d_f32(*args, hu.ptr(dx), hu.ptr(df), hu.ptr(do), hu.stream())
+        rco, want = oracle.conv2d_f32(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, f, out=o0.copy(), accumulate=1)
+    else:
+        rc = lib.small_hip_conv2d_bias_act_f32(*args, hu.ptr(dx), hu.ptr(df), hu.ptr(db), 2, 0.1, hu.ptr(do), hu.stream())
+        rco, want = oracle.conv2d_bias_act_f32(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, f, bias, 2, 0.1)
+    assert rc == 0 and rco == 0, lib.small_hip_last_error()
+    got = hu.host(do)
+    assert_close_f32(got, want, what="equal-share %s %s" % (mode, case))
+    # a second launch gives the same bytes (fixed run order in the fix-up pass)
+    if mode != "partial":
+        do2 = hu.dev(o0)
+        fn = lib.small_hip_conv2d_f32 if mode == "conv" else None
+        if fn:
+            assert fn(*args, hu.ptr(dx), hu.ptr(df), hu.ptr(do2), hu.stream()) == 0
+            assert np.array_equal(hu.host(do2), got)
+
+
 def test_conv2d_f32_batched_slices_match_batch1_across_kernel_variants(lib, oracle):
     """A batch of 48 images of a 256->256 pointwise layer runs the LDS-staged kernel with a split-K
     tail, a single image runs the split-K kernel: image n of the batched call matches the batch-1
