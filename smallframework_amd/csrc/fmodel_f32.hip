@@ -54,12 +54,13 @@ struct FMLayer
     int Ci, Co, H, W, Ho, Wo, kh, kw, stride, pt, pl;
     int K, chunks;                       // first layer: reduction length kh*kw*Ci and its chunks of 16 (four MFMA steps)
     int blob_off, blob16;                // the layer's weights in the blob (float offset) and their size in 16-byte pieces
+    int next_blob_off, next_blob16;      // the same of the layer after this one (0 pieces after the last): read with this record
     int bias_off, ktab_off;              // float offsets inside the layer's weights
     float nscale;                        // what a negative result is multiplied by: 1 none, 0 ReLU, slope LeakyReLU
     float r_wo, r_cob, r_p, norm;        // 1 / Wo, 1 / (Co / 16), 1 / (Ho * Wo), pooling scale
     // K_DWPW: a 3x3 depthwise convolution whose result feeds the 1x1 convolution that follows without leaving registers
     int Co2, w2_off, bias2_off;          // the 1x1 convolution: output channels, weights and bias inside the layer's weights
-    float nscale2;
+    float nscale2, r_cob2;               // ... and 1 / (Co2 / 16)
 };
 
 struct FMHeader
@@ -220,11 +221,12 @@ __device__ __forceinline__ void stem_layer(const FMLayer &L, float *lds, const f
     const int col = lane & 15, kq = lane >> 4;
     const int CoB = L.Co / CB, P = L.Ho * L.Wo;
     const int n_pt = (P + 15) >> 4, n_cg = CoB / TC, n_work = n_pt * n_cg;
+    const float r_ncg = L.r_cob * (float)TC;                 // 1 / n_cg
     const float *src = lds + L.src_off;
     const int4 *ktab = reinterpret_cast<const int4 *>(wl + L.ktab_off);
     for (int work = wave; work < n_work; work += NW)
     {
-        const int pt = work / n_cg, cg = work - pt * n_cg;
+        const int pt = (int)(((float)work + 0.5f) * r_ncg), cg = work - pt * n_cg;
         const int p = pt * 16 + col;
         const bool pv = p < P;
         const int pc = pv ? p : 0;
@@ -370,10 +372,11 @@ __device__ __forceinline__ void dwpw_layer(const FMLayer &L, float *lds, const f
     const int CiB = L.Ci / CB, CoB = L.Co2 / CB;
     const int Pin = L.H * L.W, P = L.Ho * L.Wo;
     const int n_pt = (P + 15) >> 4, n_cg = CoB / TC, n_work = n_pt * n_cg;
+    const float r_ncg = L.r_cob2 * (float)TC;                // 1 / n_cg
     const float *src = lds + L.src_off;
     for (int work = wave; work < n_work; work += NW)
     {
-        const int pt = work / n_cg, cg = work - pt * n_cg;
+        const int pt = (int)(((float)work + 0.5f) * r_ncg), cg = work - pt * n_cg;
         const int p = pt * 16 + col;
         const bool pv = p < P;
         const int pc = pv ? p : 0;
@@ -608,8 +611,8 @@ __global__ __launch_bounds__(NT) void fmodel_f32_kernel(const FMHeader *__restri
         const float *wl = wbuf + (li & 1) * w_floats;
         // the next layer's weights go from global memory straight into the other LDS buffer (no registers are held
         // across the layer): in flight while this layer is computed, waited for before the barrier that ends it
-        if (li + 1 < n_layers)
-            weights_to_lds(blob + hdr->layer[li + 1].blob_off, wbuf + ((li + 1) & 1) * w_floats, hdr->layer[li + 1].blob16, tid, wave);
+        if (L.next_blob16 > 0)
+            weights_to_lds(blob + L.next_blob_off, wbuf + ((li + 1) & 1) * w_floats, L.next_blob16, tid, wave);
         if (L.kind == K_CONV)
         {
             const int n_tiles = ((L.Ho * L.Wo + 15) >> 4) * (L.Co / CB);
@@ -795,6 +798,7 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
                 L.w2_off = N.blob_off - L.blob_off;
                 L.bias2_off = L.w2_off + N.bias_off;
                 L.nscale2 = N.nscale;
+                L.r_cob2 = 1.0f / (float)(N.Co / CB);
                 L.blob16 += N.blob16;
                 const int odst = layers[i + 1].dst;
                 if (odst >= 0 && phys[odst] == src)
@@ -820,6 +824,11 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
         ++n_dev;
     }
     h.n_layers = n_dev;
+    for (int i = 0; i + 1 < n_dev; ++i)
+    {
+        h.layer[i].next_blob_off = h.layer[i + 1].blob_off;
+        h.layer[i].next_blob16 = h.layer[i + 1].blob16;
+    }
 
     // LDS plan (floats): [weights x2][pooling partials][input][tensors]
     int off = 0;
