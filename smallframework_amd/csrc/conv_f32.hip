@@ -204,6 +204,26 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
         }
 }
 
+// The pooling form's pixel order: 32-pixel tiles of 4 rows x 8 columns of one image's convolution output (a.P = number
+// of tiles * 32); lane column `col` = row * 8 + column inside the tile.  pool_ok: this lane stores the pooled pixel of its
+// 2x2 window at pool_pix (element offset of channel 0 of channel block 0 in [N][Co/16][Ho/2][Wo/2][16]).
+__device__ __forceinline__ void pool_tile_pixel(const ConvArgs &a, const int tile, const int col, int &n, int &oh, int &ow,
+                                                bool &pvalid, bool &pool_ok, size_t &pool_pix)
+{
+    const int tiles_x = (a.Wo + 7) >> 3, tiles_y = (a.Ho + 3) >> 2;
+    const int tl = tile * 32 < a.P ? tile : 0;
+    n = tl / (tiles_x * tiles_y);
+    const int tin = tl - n * (tiles_x * tiles_y);
+    const int ty = tin / tiles_x, tx = tin - ty * tiles_x;
+    oh = ty * 4 + (col >> 3);
+    ow = tx * 8 + (col & 7);
+    pvalid = tile * 32 < a.P && oh < a.Ho && ow < a.Wo;
+    if (!pvalid) { oh = 0; ow = 0; }
+    const int Hp = a.Ho >> 1, Wp = a.Wo >> 1;
+    pool_ok = pvalid && ((col & 9) == 0) && (oh >> 1) < Hp && (ow >> 1) < Wp;
+    pool_pix = ((size_t)n * (a.Co / CB) * (Hp * Wp) + (size_t)((oh >> 1) * Wp + (ow >> 1))) * CB;
+}
+
 // ---------------------------------------------------------------------------------------------
 // The main kernel body: filter operand staged through LDS.  The four waves of a workgroup
 // multiply the same output-channel group, so the step's [16 ci][16 co] filter tiles (COT*2 KiB)
@@ -244,23 +264,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     {
         int n, oh, ow, rem;
         if (POOL)
-        {
-            // tiles of 4 rows x 8 columns of one image (a.P = number of tiles * 32)
-            const int tile = (pxb * 4 + wave) * PXT + t;
-            const int tiles_x = (a.Wo + 7) >> 3, tiles_y = (a.Ho + 3) >> 2;
-            const int tl = tile * 32 < a.P ? tile : 0;
-            n = tl / (tiles_x * tiles_y);
-            const int tin = tl - n * (tiles_x * tiles_y);
-            const int ty = tin / tiles_x, tx = tin - ty * tiles_x;
-            oh = ty * 4 + (col >> 3);
-            ow = tx * 8 + (col & 7);
-            pvalid[t] = tile * 32 < a.P && oh < a.Ho && ow < a.Wo;
-            if (!pvalid[t]) { oh = 0; ow = 0; }
-            rem = oh * a.Wo + ow;
-            const int Hp = a.Ho >> 1, Wp = a.Wo >> 1;
-            pool_ok[t] = pvalid[t] && ((col & 9) == 0) && (oh >> 1) < Hp && (ow >> 1) < Wp;
-            out_pix[t] = ((size_t)n * CoB * (Hp * Wp) + (size_t)((oh >> 1) * Wp + (ow >> 1))) * CB;
-        }
+            pool_tile_pixel(a, (pxb * 4 + wave) * PXT + t, col, n, oh, ow, pvalid[t], pool_ok[t], out_pix[t]);
         else
         {
             const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
@@ -435,7 +439,8 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
 // each, then waves 1..3 hand their partial accumulators to wave 0 through LDS, which adds them in
 // the fixed order 0+1+2+3 (deterministic) and runs the epilogue.  Operands go straight from global
 // memory to the MFMA registers (nothing is shared between the waves until the reduction).
-template <int COT, int PXT>
+// POOL: the 32-pixel tiles are the pooling form's 4 x 8 patches and the epilogue pools (pool_tile_pixel)
+template <int COT, int PXT, bool POOL = false>
 __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)[3][COT * PXT][16][64],
                                                  const int cg, const int pxb)
 {
@@ -455,20 +460,28 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
+    bool pool_ok[PXT];
 #pragma unroll
     for (int t = 0; t < PXT; ++t)
     {
-        const int p = (pxb * PXT + t) * 32 + col;
-        pvalid[t] = p < a.P;
-        const int pc = pvalid[t] ? p : 0;
-        const int n = pc / HoWo;
-        const int rem = pc - n * HoWo;
-        const int oh = rem / a.Wo;
-        const int ow = rem - oh * a.Wo;
+        int n, oh, ow, rem;
+        if (POOL)
+            pool_tile_pixel(a, pxb * PXT + t, col, n, oh, ow, pvalid[t], pool_ok[t], out_pix[t]);
+        else
+        {
+            const int p = (pxb * PXT + t) * 32 + col;
+            pvalid[t] = p < a.P;
+            const int pc = pvalid[t] ? p : 0;
+            n = pc / HoWo;
+            rem = pc - n * HoWo;
+            oh = rem / a.Wo;
+            ow = rem - oh * a.Wo;
+            pool_ok[t] = false;
+            out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
+        }
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
-        out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
     }
     const float *w_row[COT];
 #pragma unroll
@@ -575,7 +588,8 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
                 for (int t = 0; t < PXT; ++t)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc[c][t][r] += red[w][c * PXT + t][r][lane];
-        conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+        if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix);
+        else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
     }
 }
 
@@ -598,7 +612,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
 // single 32x32 tiles, each multiplied by one workgroup whose four waves split the reduction, i.e.
 // 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
 // The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
-template <int COT, int PXT>
+template <int COT, int PXT, bool POOL = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -609,7 +623,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     {
         // n_main is a multiple of NUM_XCD: consecutive logical ids share an XCD
         const int lid = (bid % NUM_XCD) * (a.n_main / NUM_XCD) + bid / NUM_XCD;
-        conv_lds_tile<COT, PXT>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+        conv_lds_tile<COT, PXT, POOL>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
         return;
     }
     constexpr int SUB = 4 * COT * PXT;            // 32x32 tiles per whole workgroup tile
@@ -620,7 +634,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int co32 = (lid % a.n_co_groups) * COT + sub % COT;
     const int px32 = (lid / a.n_co_groups) * (4 * PXT) + sub / COT;
     if (co32 * 32 >= a.Co || px32 * 32 >= a.P) return;     // uniform over the workgroup
-    conv_splitk_tile<1, 1>(a, red, co32, px32);
+    conv_splitk_tile<1, 1, POOL>(a, red, co32, px32);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1091,6 +1105,18 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
     hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
 }
 
+// Whole rounds + cut tail (conv_mfma_f32_hybrid_kernel) or whole tiles only?  A split-K piece multiplies about half as
+// fast as a whole tile (operands straight from global memory, one MFMA chain per wave), so the cut tail wins while the
+// left-over tiles fill less than half a round and loses beyond.  Batch sweeps of 256->256 @28x28, 512->512 @14x14 and
+// 3x3 64->128 @52x52: 28..128 left-over tiles of 256: 1..6 us faster; 164..252: 2..7 us slower.  With one whole round
+// of two-tile waves the round itself slows down more than the tail gains (338 tiles: 73 against 68 us).
+template <int COT, int PXT>
+bool tail_pays(int n_main, int rest, int nsteps)
+{
+    static const bool use_tail = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return !(e && e[0] == '0'); }();
+    return use_tail && rest > 0 && rest <= NUM_CU / 2 && nsteps >= 8 && (COT * PXT == 1 || n_main >= 2 * NUM_CU);
+}
+
 template <int COT, int PXT>
 void launch_mfma(ConvArgs &a, hipStream_t s)
 {
@@ -1098,9 +1124,8 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    static const bool use_tail = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return !(e && e[0] == '0'); }();
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
-    if (use_tail && rest > 0 && a.kh * a.kw * (a.Ci / CB) >= 8)
+    if (tail_pays<COT, PXT>(n_main, rest, a.kh * a.kw * (a.Ci / CB)))
     {
         a.n_main = n_main;
         hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT, a.slabs > 0 ? a.slabs : 1),
@@ -1303,7 +1328,14 @@ void launch_mfma_pool(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
+    if (tail_pays<COT, PXT>(n_main, rest, a.kh * a.kw * (a.Ci / CB)))
+    {
+        a.n_main = n_main;
+        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, true>), dim3(n_main + rest * 4 * COT * PXT), dim3(256), 0, s, a);
+    }
+    else
+        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
 }
 
 // Conv2D + bias + activation + MaxPool2D 2x2 stride 2 (no pool padding) in one launch

@@ -30,7 +30,10 @@ CASES = [
     (2, 3, 1, (1, 1, 1, 1), 32, 16, 16, 16, True, capi.ACT_LEAKY),        # main kernel, 1x1 wave tile
     (1, 3, 1, (1, 1, 1, 1), 64, 32, 13, 13, False, capi.ACT_RELU),        # odd extents, ragged 4x8 tiles
     (5, 3, 1, (1, 1, 1, 1), 128, 64, 12, 20, True, capi.ACT_LEAKY),
-    (16, 3, 1, (1, 1, 1, 1), 64, 32, 52, 52, True, capi.ACT_LEAKY),       # 2x1 wave tile (many tiles)
+    (16, 3, 1, (1, 1, 1, 1), 64, 32, 52, 52, True, capi.ACT_LEAKY),       # 728 workgroup tiles of whole rounds only
+    (16, 3, 1, (1, 1, 1, 1), 64, 16, 60, 68, True, capi.ACT_RELU),        # 2x1 wave tile, 270 workgroup tiles, ragged patches
+    (3, 3, 1, (1, 1, 1, 1), 32, 16, 120, 136, True, capi.ACT_LEAKY),      # 383 workgroup tiles: one whole round + a cut tail
+    (11, 3, 1, (1, 1, 1, 1), 64, 16, 40, 160, False, capi.ACT_RELU),      # 2x1 wave tile, 550 = two rounds + a cut tail
     (2, 1, 1, (0, 0, 0, 0), 48, 32, 10, 10, True, capi.ACT_RELU),         # 1x1 convolution
     (2, 3, 2, (0, 1, 0, 1), 32, 16, 18, 18, False, capi.ACT_NONE),        # stride-2 convolution
     (1, 5, 1, (2, 2, 2, 2), 16, 16, 8, 8, True, capi.ACT_RELU),
