@@ -165,10 +165,10 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
     else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix);
 }
 
-// Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 4 rows x 8
-// columns of the convolution's output (lane col = row * 8 + column), so a pooling window is this lane, lane
-// ^ 1 (next column) and lanes ^ 8 (next row): bias and activation, two shuffles and maxima per value, and
-// the lanes at even row and even column store the pooled pixel into [N][Co/16][Ho/2][Wo/2][16].
+// Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 8 pooling windows of
+// four pixels (pool_tile_pixel), so a window is this lane, lane ^ 1 (next column) and lanes ^ 2 (next row): bias
+// and activation, two shuffles and maxima per value, and the first lane of each window stores the pooled pixel
+// into [N][Co/16][Ho/2][Wo/2][16].
 template <int COT, int PXT>
 __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
                                                    const bool (&pool_ok)[PXT], const size_t (&pool_pix)[PXT])
@@ -194,7 +194,7 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
                     float v = act_bf(acc[c][t][4 * q + e] + b4[e], nscale);
                     const float u = __shfl_xor(v, 1, WAVE);
                     v = v > u ? v : u;
-                    const float w = __shfl_xor(v, 8, WAVE);
+                    const float w = __shfl_xor(v, 2, WAVE);
                     m[e] = v > w ? v : w;
                 }
                 if (pool_ok[t] && co4 < a.Co)
@@ -204,24 +204,26 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
         }
 }
 
-// The pooling form's pixel order: 32-pixel tiles of 4 rows x 8 columns of one image's convolution output (a.P = number
-// of tiles * 32); lane column `col` = row * 8 + column inside the tile.  pool_ok: this lane stores the pooled pixel of its
-// 2x2 window at pool_pix (element offset of channel 0 of channel block 0 in [N][Co/16][Ho/2][Wo/2][16]).
+// The pooling form's pixel order: pooling windows (image, pooled row, pooled column) counted straight through, four
+// pixels each; lane column `col` = (window of the tile) * 4 + (row in the window) * 2 + (column in the window), a.P = 4 x
+// the number of windows.  No slot is lost to ragged patches (a 26x26 map cut into 4 x 8 patches computed 32% more pixels
+// than it has), and convolution rows / columns that no window covers (odd extents) are not computed at all.  pool_ok:
+// this lane stores the pooled pixel of its window at pool_pix (element offset of channel 0 of channel block 0 in
+// [N][Co/16][Ho/2][Wo/2][16]).
 __device__ __forceinline__ void pool_tile_pixel(const ConvArgs &a, const int tile, const int col, int &n, int &oh, int &ow,
                                                 bool &pvalid, bool &pool_ok, size_t &pool_pix)
 {
-    const int tiles_x = (a.Wo + 7) >> 3, tiles_y = (a.Ho + 3) >> 2;
-    const int tl = tile * 32 < a.P ? tile : 0;
-    n = tl / (tiles_x * tiles_y);
-    const int tin = tl - n * (tiles_x * tiles_y);
-    const int ty = tin / tiles_x, tx = tin - ty * tiles_x;
-    oh = ty * 4 + (col >> 3);
-    ow = tx * 8 + (col & 7);
-    pvalid = tile * 32 < a.P && oh < a.Ho && ow < a.Wo;
-    if (!pvalid) { oh = 0; ow = 0; }
-    const int Hp = a.Ho >> 1, Wp = a.Wo >> 1;
-    pool_ok = pvalid && ((col & 9) == 0) && (oh >> 1) < Hp && (ow >> 1) < Wp;
-    pool_pix = ((size_t)n * (a.Co / CB) * (Hp * Wp) + (size_t)((oh >> 1) * Wp + (ow >> 1))) * CB;
+    const int Wp = a.Wo >> 1, HpWp = (a.Ho >> 1) * Wp;
+    const int p = tile * 32 + col;
+    pvalid = p < a.P;
+    const int w = pvalid ? p >> 2 : 0;
+    n = w / HpWp;
+    const int r = w - n * HpWp;
+    const int ph = r / Wp, pw = r - ph * Wp;
+    oh = 2 * ph + ((col >> 1) & 1);
+    ow = 2 * pw + (col & 1);
+    pool_ok = pvalid && (col & 3) == 0;
+    pool_pix = ((size_t)n * (a.Co / CB) * HpWp + r) * CB;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -439,7 +441,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
 // each, then waves 1..3 hand their partial accumulators to wave 0 through LDS, which adds them in
 // the fixed order 0+1+2+3 (deterministic) and runs the epilogue.  Operands go straight from global
 // memory to the MFMA registers (nothing is shared between the waves until the reduction).
-// POOL: the 32-pixel tiles are the pooling form's 4 x 8 patches and the epilogue pools (pool_tile_pixel)
+// POOL: the 32-pixel tiles are the pooling form's groups of 8 windows and the epilogue pools (pool_tile_pixel)
 template <int COT, int PXT, bool POOL = false>
 __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)[3][COT * PXT][16][64],
                                                  const int cg, const int pxb)
@@ -1398,10 +1400,11 @@ int conv_pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt,
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }
-    // pixel tiles of 4 rows x 8 columns; P counts tile slots
-    const long ntiles = (long)batch * ((a.Ho + 3) / 4) * ((a.Wo + 7) / 8);
-    if (ntiles > 0x7fffffffL / 64) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
-    a.P = (int)(ntiles * 32);
+    // pixel tiles of 8 pooling windows; P = 4 x the number of windows
+    const long nwin = (long)batch * (a.Ho / 2) * (a.Wo / 2);
+    if (nwin > 0x7fffffffL / 16) { set_error("%s: too many pixels for one launch", op); return SMALL_HIP_EINVAL; }
+    a.P = (int)(nwin * 4);
+    const long ntiles = (nwin + 7) / 8;
     const long tiles32 = (long)((Co + 31) / 32) * ntiles;
     const long simds = 4L * NUM_CU;
     const int nsteps = kh * kw * (Ci / CB);
