@@ -73,7 +73,7 @@ public:
                 m_order[step + 1] == m_pool_after[cur])
             {
                 // convolution whose only consumer is a max-pooling layer: both in one call (one launch for a 2x2
-                // stride-2 pool on a map the kernel's tiles fill); the convolution's own output is never cached
+                // stride-2 pool); the convolution's own output is never cached
                 const size_t pl = m_pool_after[cur];
                 auto *conv = static_cast<Conv2DLayer<BufferT> *>(this->m_layers[cur]);
                 auto *pool = static_cast<MaxPool2DLayer<BufferT> *>(this->m_layers[pl]);

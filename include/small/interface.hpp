@@ -239,8 +239,8 @@ void Conv2D_Accum_ReLU(int batch, int kernel_height, int kernel_width, int strid
 }
 
 // out = MaxPool2D(act(Conv2D(in, filter) + bias)) in one launch when the pooling window is 2x2 stride 2 without
-// padding (the pooling runs on the accumulators) when the kernel's pixel tiles fill the map well; any other
-// window or a ragged map runs the two layers through inter_output_buf.  bias_buf may be empty.
+// padding (the pooling runs on the accumulators; first layers only when the kernel's pixel tiles fill the map well); any
+// other window runs the two layers through inter_output_buf.  bias_buf may be empty.
 template <class BufferT, detail::if_float<BufferT> = true>
 void Conv2D_Bias_Act_Maxpool2D(int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride,
                                uint8_t conv_t_pad, uint8_t conv_b_pad, uint8_t conv_l_pad, uint8_t conv_r_pad,
@@ -256,14 +256,14 @@ void Conv2D_Bias_Act_Maxpool2D(int batch, int conv_kernel_height, int conv_kerne
                    !(act == LEAKY && negative_slope < 0.f);
     if (fusable)
     {
-        // the fused kernel works on 4 x 8 pixel tiles of one image (16 x 16 for first layers): on small maps the
-        // ragged tiles cost more than the saved pooling pass (measured: 26x26 loses, 52x52 wins): fuse from 90% fill
+        // first layers (1-3 input channels) are fused on 16 x 16 pixel tiles of one image: on small maps the ragged
+        // tiles cost more than the saved pooling pass, so fuse from 90% fill; the main kernel counts pooling windows
+        // straight through and loses nothing on any map
         const long Hc = (long)output_dim(input_height + conv_t_pad + conv_b_pad, conv_stride, conv_kernel_height);
         const long Wc = (long)output_dim(input_width + conv_l_pad + conv_r_pad, conv_stride, conv_kernel_width);
         const bool first = input_channels % (int)BufferT::C_ib != 0;
-        const long th = first ? 16 : 4, tw = first ? 16 : 8;
-        const long slots = ((Hc + th - 1) / th * th) * ((Wc + tw - 1) / tw * tw);
-        fusable = Hc > 0 && Wc > 0 && 10 * Hc * Wc >= 9 * slots;
+        const long slots = ((Hc + 15) / 16 * 16) * ((Wc + 15) / 16 * 16);
+        fusable = Hc > 0 && Wc > 0 && (!first || 10 * Hc * Wc >= 9 * slots);
     }
     if (fusable)
     {

@@ -418,12 +418,13 @@ class HipExecutor:
 
     @staticmethod
     def _pool_tiles_fill(op):
-        """The fused convolution + pooling kernel works on 4 x 8 pixel tiles (16 x 16 for first layers) of one
-        image; on small maps the ragged tiles cost more than the saved pooling pass (measured: 26x26 loses, 52x52
-        wins), so fuse from 90% tile utilisation."""
-        th, tw = (4, 8) if op.C % CB == 0 else (16, 16)
+        """First layers (1-3 input channels) are fused on 16 x 16 pixel tiles of one image: on small maps the ragged
+        tiles cost more than the saved pooling pass, so fuse from 90% tile utilisation.  The main kernel counts
+        pooling windows straight through and loses nothing on any map."""
+        if op.C % CB == 0:
+            return True
         ho, wo = op.Ho, op.Wo
-        return ho * wo >= 0.9 * (-(-ho // th) * th) * (-(-wo // tw) * tw)
+        return ho * wo >= 0.9 * (-(-ho // 16) * 16) * (-(-wo // 16) * 16)
 
     @staticmethod
     def _p(t):
