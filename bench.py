@@ -126,6 +126,29 @@ def op_bound(model, op, batch):
     return (t_mfma, "mfma") if t_mfma > t_hbm else (t_hbm, "hbm")
 
 
+# (timed steps, warm-up steps) per headline model when the command line gives none: ~200 ms timed after ~100 ms of load
+DEFAULT_COUNTS = {"mobilenet_v1": (200, 100), "tiny_yolo_v2": (200, 100), "layer_sweep": (200, 100),
+                  "resnet8_u8": (6000, 3000), "dscnn": (6000, 3000)}
+
+
+def counts_for(step_fn, args, at_least=0):
+    """(timed steps, warm-up steps) for a side measurement.  With counts on the command line: those.  Otherwise from
+    the duration of `step_fn` (3 + 10 probe calls), so that the warm-up is about 100 ms of load and the timed region
+    about 200 ms whatever the model's size."""
+    if not args.auto_counts:
+        return max(args.steps, at_least), args.warmup
+    import torch
+    for _ in range(3):
+        step_fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        step_fn()
+    torch.cuda.synchronize()
+    est = max((time.perf_counter() - t0) / 10, 1e-6)
+    return min(8000, max(200, int(0.2 / est) + 1)), min(4000, max(100, int(0.1 / est) + 1))
+
+
 def time_forward(ex, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -159,30 +182,34 @@ def time_ops(ex, steps):
     import torch
     ops = ex.model.ops
     st = ex.stream()
+    # Events for all passes are made first and the passes are issued back to back with one synchronisation at the end:
+    # the GPU stays loaded (a pause between passes lets its clock drop), and the host never waits inside a pass.
     if ex.model.dtype == "f32" and ex.fused:
         entries = ex.plan
         index = {op.name: i for i, op in enumerate(ops)}
-        seen = [[] for _ in ops]
-        for _ in range(steps):
-            evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(entries) + 1)]
-            evs[0].record()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(entries) + 1)] for _ in range(steps)]
+        for ev in evs:
+            ev[0].record()
             for i, e in enumerate(entries):
                 ex.run_entry(e, st)
-                evs[i + 1].record()
-            torch.cuda.synchronize()
+                ev[i + 1].record()
+        torch.cuda.synchronize()
+        seen = [[] for _ in ops]
+        for ev in evs:
             for i, e in enumerate(entries):
-                seen[index[e[0].name]].append(evs[i].elapsed_time(evs[i + 1]))
+                seen[index[e[0].name]].append(ev[i].elapsed_time(ev[i + 1]))
         return [statistics.median(t) if t else 0.0 for t in seen]
-    seen = [[] for _ in ops]
-    for _ in range(steps):
-        evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)]
-        evs[0].record()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)] for _ in range(steps)]
+    for ev in evs:
+        ev[0].record()
         for i, op in enumerate(ops):
             ex.run_op(op, st)
-            evs[i + 1].record()
-        torch.cuda.synchronize()
+            ev[i + 1].record()
+    torch.cuda.synchronize()
+    seen = [[] for _ in ops]
+    for ev in evs:
         for i in range(len(ops)):
-            seen[i].append(evs[i].elapsed_time(evs[i + 1]))
+            seen[i].append(ev[i].elapsed_time(ev[i + 1]))
     return [statistics.median(t) for t in seen]
 
 
@@ -437,8 +464,9 @@ def sweep_only(args, torch, models):
     rows, head = [], None
     for m in models.layer_sweep():
         ex = models.HipExecutor(m, batch)
-        sec = time_forward(ex, args.steps, args.warmup)
-        ms = time_ops(ex, args.steps)
+        k, w = counts_for(ex.forward, args)
+        sec = time_forward(ex, k, w)
+        ms = time_ops(ex, min(k, 200))
         r = layer_table(m, batch, ms)[0]
         r["layer"] = m.name
         r["images_per_s"] = round(batch / (r["ms"] * 1e-3), 1)
@@ -471,8 +499,11 @@ def sweep_only(args, torch, models):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # defaults (DEFAULT_COUNTS): the GPU reaches its sustained clock only after some tens of milliseconds of load
+    # (MobileNetV1 batch 64: 1.05 ms/step over steps 4..23 of a fresh process, 1.00 ms/step from step 50 on), so the
+    # default warm-up is about 100 ms of forward passes and the timed region about 200 ms
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--model", default="mobilenet_v1",
                     choices=["mobilenet_v1", "resnet8_u8", "tiny_yolo_v2", "dscnn", "layer_sweep"])
     ap.add_argument("--batch", type=int, default=0)
@@ -493,6 +524,11 @@ def main():
         log("bench.py: no GPU visible")
         sys.exit(1)
     capi.load()
+    args.auto_counts = args.steps is None and args.warmup is None
+    if args.steps is None:
+        args.steps = DEFAULT_COUNTS[args.model][0]
+    if args.warmup is None:
+        args.warmup = DEFAULT_COUNTS[args.model][1]
     if args.model == "layer_sweep":
         return sweep_only(args, torch, models)
     default_batch = {"mobilenet_v1": 64, "resnet8_u8": 64, "tiny_yolo_v2": 16, "dscnn": 64}
@@ -517,11 +553,11 @@ def main():
     log("%s: %.3f ms/step, %.1f images/s" % (model.name, sec * 1e3, ips))
 
     # per-op device times (HIP events on the launch stream) over the same number of steps
-    ms = time_ops(ex, args.steps)
+    ms = time_ops(ex, min(args.steps, 200))
     table = layer_table(model, batch, ms)
     if not args.no_extras:
         # what a kernel that only moves each bandwidth-bound layer's bytes takes in the same place of the model
-        add_floor_column(table, stream_floors(ex, max(5, args.steps // 2)))
+        add_floor_column(table, stream_floors(ex, max(5, min(args.steps, 200) // 2)))
     if args.library_gemm:
         log("float32 MFMA on registers only: %s TFLOP/s sustained (published peak 157.3)" % mfma_probe_tflops())
         log("device-to-device copy of 822 MB: %.0f GB/s read + write (published peak 8000)" % hbm_copy_gbs())
@@ -640,21 +676,23 @@ def main():
         for name, b in (("resnet8_u8", 64), ("resnet8_u8", 256)):
             m2 = getattr(models, name)()
             e2 = models.HipExecutor(m2, b)
-            s2 = time_forward(e2, max(args.steps, 50), args.warmup)
+            k2, w2 = counts_for(e2.forward, args, 50)
+            s2 = time_forward(e2, k2, w2)
             ms2 = time_ops(e2, 10)
             # the same forward pass replayed from a HIP graph (21 launches, no host work in between)
             e2.capture()
-            for _ in range(args.warmup):
+            for _ in range(w2):
                 e2.replay()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            for _ in range(max(args.steps, 50)):
+            for _ in range(k2):
                 e2.replay()
             torch.cuda.synchronize()
-            s3 = (time.perf_counter() - t0) / max(args.steps, 50)
+            s3 = (time.perf_counter() - t0) / k2
             # the whole model in one launch (one workgroup per image, tensors and filters in LDS), HIP-event timed
             e2.build_one_launch()
-            s4 = time_forward_one_launch(e2, max(args.steps, 50), args.warmup)
+            k4, w4 = counts_for(e2.forward_one_launch, args, 50)
+            s4 = time_forward_one_launch(e2, k4, w4)
             algo = b * (m2.in_shape[0] * m2.in_shape[1] * m2.in_shape[2] + m2.ops[-1].Co) + \
                 sum(o.weight_elems() for o in m2.ops)
             extras["%s_b%d" % (name, b)] = {"images_per_s": round(b / s2, 1), "ms_per_step": round(s2 * 1e3, 4),
@@ -675,7 +713,8 @@ def main():
         others += [(m, b) for b in (1, 64) for m in models.layer_sweep()]
         for m2, b in others:
             e2 = models.HipExecutor(m2, b)
-            s2 = time_forward(e2, args.steps, args.warmup)
+            k2, w2 = counts_for(e2.forward, args)
+            s2 = time_forward(e2, k2, w2)
             ms2 = time_ops(e2, 10)
             tab = layer_table(m2, b, ms2)
             if b > 1:
@@ -685,7 +724,8 @@ def main():
             if m2.name == "dscnn":
                 # the whole model in one launch (small_hip_fmodel_forward: a workgroup per image, activations in LDS)
                 e2.build_one_launch()
-                s4 = time_forward_one_launch(e2, max(args.steps, 50), args.warmup)
+                k4, w4 = counts_for(e2.forward_one_launch, args, 50)
+                s4 = time_forward_one_launch(e2, k4, w4)
                 extras["%s_b%d" % (m2.name, b)].update({"one_launch_ms_per_step": round(s4 * 1e3, 4),
                                                         "one_launch_images_per_s": round(b / s4, 1),
                                                         "one_launch_TFLOPs": round(b * m2.flops_per_image() / s4 / 1e12, 3)})

@@ -1109,14 +1109,19 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
 
 // Whole rounds + cut tail (conv_mfma_f32_hybrid_kernel) or whole tiles only?  A split-K piece multiplies about half as
 // fast as a whole tile (operands straight from global memory, one MFMA chain per wave), so the cut tail wins while the
-// left-over tiles fill less than half a round and loses beyond.  Batch sweeps of 256->256 @28x28, 512->512 @14x14 and
-// 3x3 64->128 @52x52: 28..128 left-over tiles of 256: 1..6 us faster; 164..252: 2..7 us slower.  With one whole round
-// of two-tile waves the round itself slows down more than the tail gains (338 tiles: 73 against 68 us).
+// left-over tiles fill at most half a round and loses beyond, whatever the wave tile and the number of whole rounds.
+// Batch sweeps, left-over tiles of 256 -> gain (+) or loss (-) in us: 1x1 256->256 @28x28 (16 K-steps) 32: +3, 128: +1,
+// 224: -3; 512->512 @14x14 (32) 80: +2..6, 176: -2, 224: -6; 3x3 64->128 @52x52 (36) 84: +1, 168: -3, 252: -7;
+// 3x3 128->256 @26x26 (72) 20: +25, 84: +10, 128: +4, 168: -3, 216: -10; 3x3 256->512 @13x13 (144) 40: +42, 128: +13,
+// 168: -12, 216: -27.
 template <int COT, int PXT>
 bool tail_pays(int n_main, int rest, int nsteps)
 {
-    static const bool use_tail = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return !(e && e[0] == '0'); }();
-    return use_tail && rest > 0 && rest <= NUM_CU / 2 && nsteps >= 8 && (COT * PXT == 1 || n_main >= 2 * NUM_CU);
+    // tuning knob SMALL_HIP_CONV_TAIL: 0 = never, 2 = whenever tiles are left over
+    static const int knob = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return e ? e[0] - '0' : 1; }();
+    (void)n_main;
+    if (knob == 0 || rest == 0 || nsteps < 8) return false;
+    return knob == 2 || rest <= NUM_CU / 2;
 }
 
 template <int COT, int PXT>
