@@ -171,26 +171,34 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_strip_kernel(const float4 *__re
 
 // 3x3 depthwise through LDS.  A workgroup owns a TW x TH tile of output pixels of one (image,
 // channel block) plane.  The input pixels under it (64 bytes each) are fetched from memory exactly
-// once, in row-contiguous 16-byte pieces with every load in flight together, and parked in LDS with
-// zeros where the tile hangs over the image; the nine filter taps of the block go to LDS too.  A
-// lane then owns one output column, four channels and R consecutive rows.  At stride 1 it slides a
-// three-row register window down the staged tile (three 16-byte LDS reads per output); at stride 2
-// it reads its nine taps per output.  The strip kernel issued 4.5 (stride 1) to 7 (stride 2)
-// vector-cache loads per output plus nine tap loads per lane, and that cache, not HBM, was its limit.
+// once, in row-contiguous 16-byte pieces, and parked in LDS with zeros where the tile hangs over
+// the image; the nine filter taps of the block go to LDS too.  The staging is done by the memory
+// pipeline (global_load_lds_dwordx4: a wave's 64 lanes write one KiB of consecutive LDS, each lane
+// gives its own global address; pieces outside the image come from a block of zeros): no lane holds
+// the pieces in registers or waits for them before it can issue an LDS store (against staging
+// through registers, batch 64: 512 channels on 14x14 13.0 -> 10.0 us, 256 on 28x28 21.1 -> 17.4,
+// 128 on 56x56 32.7 -> 30.3).  A lane then owns one output column, four channels and R consecutive
+// rows.  At stride 1 it slides a three-row register window down the staged tile (three 16-byte LDS
+// reads per output); at stride 2 it reads its nine taps per output.  The strip kernel issued 4.5
+// (stride 1) to 7 (stride 2) vector-cache loads per output plus nine tap loads per lane, and that
+// cache, not HBM, was its limit.
+__device__ __align__(16) const float g_dw_zero[4] = {0.f, 0.f, 0.f, 0.f};
+
 template <int S, int TW, int R, bool ACC, int SRU = 0>
 __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__restrict__ in,
                                                              const float4 *__restrict__ filt, float4 *out,
                                                              int cblocks, int tiles_x, int tiles_y,
                                                              int nblocks, int per_xcd, Geom g, Epi e)
 {
-    constexpr int SR = SRU ? SRU : 64 / TW;                  // rows of lane slots in use (SRU < 64/TW leaves slots idle for a smaller tile)
-    constexpr int TH = SR * R;                               // output rows per tile
-    constexpr int IW = (TW - 1) * S + 3, IH = (TH - 1) * S + 3;  // staged input tile, in pixels
-    constexpr int ROW4 = IW * 4;                             // float4 per staged row
+    constexpr int SR = SRU ? SRU : 64 / TW;
+    constexpr int TH = SR * R;
+    constexpr int IW = (TW - 1) * S + 3, IH = (TH - 1) * S + 3;
+    constexpr int ROW4 = IW * 4;
     constexpr int E = IH * ROW4;
     constexpr int NLD = (E + TPB - 1) / TPB;
-    __shared__ float4 sX[E];
-    __shared__ float4 sW[36];
+    constexpr int EP = NLD * TPB;                            // every lane writes a piece in every round
+    __shared__ float4 sX[EP];
+    __shared__ float4 sW[64];
 
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * per_xcd + bid / NUM_XCD;
@@ -203,9 +211,10 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     const int ih0 = oh0 * S - g.pt, iw0 = ow0 * S - g.pl;
     const float4 *src = in + (size_t)plane * g.H * g.W * 4;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 *gzero = reinterpret_cast<const float4 *>(g_dw_zero);
     const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    float4 v[NLD];
 #pragma unroll
     for (int k = 0; k < NLD; ++k)
     {
@@ -213,26 +222,22 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
         const int r = el / ROW4, c4 = el - r * ROW4;
         const int ih = ih0 + r, iw = iw0 + (c4 >> 2);
         const bool ok = el < E && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-        v[k] = src[ok ? ((size_t)ih * g.W + iw) * 4 + (c4 & 3) : 0];
-        if (!ok) v[k] = zero;
+        const float4 *gp = ok ? src + ((size_t)ih * g.W + iw) * 4 + (c4 & 3) : gzero;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                         (__attribute__((address_space(3))) void *)&sX[k * TPB + wave * 64], 16, 0, 0);
     }
-    if (tid < 36) sW[tid] = filt[(size_t)cbk * 36 + tid];
-#pragma unroll
-    for (int k = 0; k < NLD; ++k)
+    if (wave == 0)
     {
-        const int el = tid + k * TPB;
-        if (el < E) sX[el] = v[k];
+        const float4 *gp = filt + (size_t)cbk * 36 + (tid < 36 ? tid : 35);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                         (__attribute__((address_space(3))) void *)&sW[0], 16, 0, 0);
     }
-    __syncthreads();
 
     const int q = tid & 3, slot = tid >> 2;
     const int tx = slot % TW, sy_raw = slot / TW;
     const bool slot_on = sy_raw < SR;
     const int sy = slot_on ? sy_raw : 0;      // idle slots read in bounds and store nothing
     const int ow = ow0 + tx;
-    float4 w[9];
-#pragma unroll
-    for (int t = 0; t < 9; ++t) w[t] = sW[t * 4 + q];
     float4 bias = zero;
     if (e.bias) bias = e.bias[cbk * 4 + q];
     const float nscale = act_scale(e.act, e.slope);
@@ -240,6 +245,12 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     float4 *dst = out + (size_t)plane * g.Ho * g.Wo * 4 + (size_t)ow * 4 + q;
     const bool col_ok = slot_on && ow < g.Wo;
 
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this lane's pieces have landed
+    __syncthreads();                         // everyone's have
+
+    float4 w[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w[t] = sW[t * 4 + q];
     float4 win[3][3];
     if (S == 1)
     {
@@ -253,7 +264,6 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
     {
         if (S == 1)
         {
-            // rows o, o+1, o+2 of the lane's window live in win[o%3], win[(o+1)%3], win[(o+2)%3]
 #pragma unroll
             for (int c = 0; c < 3; ++c) win[(o + 2) % 3][c] = xs[((o + 2) * IW + c) * 4];
         }
@@ -278,7 +288,7 @@ __global__ __launch_bounds__(TPB) void dw3x3_f32_tile_kernel(const float4 *__res
                 acc.x = fmaf(x.x, k.x, acc.x); acc.y = fmaf(x.y, k.y, acc.y);
                 acc.z = fmaf(x.z, k.z, acc.z); acc.w = fmaf(x.w, k.w, acc.w);
             }
-        if (ACC) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }   // bias is zero without one
+        if (ACC) { acc.x += bias.x; acc.y += bias.y; acc.z += bias.z; acc.w += bias.w; }
         acc.x = act_bf(acc.x, nscale); acc.y = act_bf(acc.y, nscale);
         acc.z = act_bf(acc.z, nscale); acc.w = act_bf(acc.w, nscale);
         if (ok) dst[(size_t)oh * g.Wo * 4] = acc;
@@ -396,7 +406,8 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 const int tiles_y = (g.Ho + shapes[best].th - 1) / shapes[best].th;
                 const size_t nb = (size_t)batch * (C / CB) * tiles_x * tiles_y;
                 if (nb > 0x7fffffff / 2) { set_error("%s: too many blocks for one launch", op); return SMALL_HIP_EINVAL; }
-                const int nblocks = (int)nb, per_xcd = (nblocks + NUM_XCD - 1) / NUM_XCD;
+                const int nblocks = (int)nb;
+                const int per_xcd = (nblocks + NUM_XCD - 1) / NUM_XCD;
                 decltype(&dw3x3_f32_tile_kernel<1, 16, 4, false>) tk;
 #define SHP_DW_TILE(S_, TW_, R_) (accumulate ? dw3x3_f32_tile_kernel<S_, TW_, R_, true> : dw3x3_f32_tile_kernel<S_, TW_, R_, false>)
                 if (stride == 1)
