@@ -373,8 +373,9 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
     {
         constexpr int R1 = 4, R2 = 3;      // output rows per lane at stride 1 / stride 2
         static const bool tile_off = [] { const char *v = std::getenv("SMALL_HIP_DW_TILE"); return v && v[0] == '0'; }();
-        // measured: the strip kernel wins below 7x7 outputs at stride 1 and below 28x28 at stride 2
-        const int min_side = stride == 1 ? 7 : 28;
+        // measured: the strip kernel wins below 7x7 outputs at stride 1 and below 14x14 at stride 2 (256 channels 28x28 -> 14x14,
+        // batch 64: tile kernel 11.4 us, strip kernel 14.0 us; 512 channels 14x14 -> 7x7: 7.0 us either way)
+        const int min_side = stride == 1 ? 7 : 14;
         if (g.Ho >= min_side && g.Wo >= min_side && !tile_off)
         {
             // the tile shape that wastes the fewest lanes on this image; ties go to the first
