@@ -938,12 +938,21 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
     typedef float floatx4v __attribute__((ext_vector_type(4)));
     constexpr int T = 16;                                    // tile side in output pixels
     constexpr int PH = (T - 1) * S + 3, PW = PH;             // input patch in pixels
-    constexpr int PITCH = VEC ? (PW * CI + 3 + 3) / 4 * 4 : PW * CI;   // floats per staged patch row
-    constexpr int NEL = PH * PITCH;
+    // The patch is staged by the memory pipeline (global_load_lds: a wave's 64 lanes write consecutive LDS, each lane gives
+    // its own global address, positions outside the image read a block of zeros): no registers, no LDS store instructions.
+    // VEC: 16-byte pieces, J lanes per patch row, the row pitch is 4 J floats so that a wave's pieces are consecutive.
+    constexpr int P4 = (PW * CI + 3 + 3) / 4;                // 16-byte pieces per staged row (VEC)
+    constexpr int J = P4 <= 8 ? 8 : P4 <= 16 ? 16 : P4 <= 32 ? 32 : 64;   // lanes per row (power of two)
+    static_assert(!VEC || P4 <= 64, "patch row too long");
+    constexpr int PITCH = VEC ? 4 * J : PW * CI;             // floats per staged patch row
+    constexpr int VROWS = 256 / J, VPASS = (PH + VROWS - 1) / VROWS;
+    constexpr int SPASS = (PH * PITCH + 255) / 256;          // rounds of 256 floats (not VEC)
+    constexpr int NEL = VEC ? VPASS * VROWS * PITCH : SPASS * 256;   // every lane writes in every round
     constexpr int K = 9 * CI, NS = (K + 3) / 4;
     __shared__ __align__(16) float patch[NEL];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, kq = lane >> 4;
     const int CoB = a.Co / CB;
     const int HoWo = a.Ho * a.Wo;
@@ -960,48 +969,37 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
     int lead = 0;
     if (VEC)
     {
-        constexpr int P4 = PITCH / 4;                        // 16-byte pieces per staged row
-        constexpr int J = P4 <= 8 ? 8 : P4 <= 16 ? 16 : P4 <= 32 ? 32 : 64;   // threads per row (power of two)
-        constexpr int R = 256 / J, NPASS = (PH + R - 1) / R;
-        static_assert(P4 <= 64, "patch row too long");
         const int x0 = iw_base * CI;
         lead = x0 & 3;                                       // two's complement: also right for x0 = -CI
         const int xa = x0 - lead;                            // multiple of 4
         const int j = tid & (J - 1), r0 = tid / J;
-        float4 pv[NPASS];
 #pragma unroll
-        for (int ps = 0; ps < NPASS; ++ps)
+        for (int ps = 0; ps < VPASS; ++ps)
         {
-            const int py = r0 + ps * R, ih = ih_base + py, xe = xa + 4 * j;
+            const int py = r0 + ps * VROWS, ih = ih_base + py, xe = xa + 4 * j;
             const bool ok = j < P4 && py < PH && (unsigned)ih < (unsigned)a.H && xe >= 0 && xe < row_el;
-            pv[ps] = *reinterpret_cast<const float4 *>(ok ? img + ih * row_el + xe : g_zero_block);
-        }
-#pragma unroll
-        for (int ps = 0; ps < NPASS; ++ps)
-        {
-            const int py = r0 + ps * R;
-            if (j < P4 && py < PH) *reinterpret_cast<float4 *>(&patch[py * PITCH + 4 * j]) = pv[ps];
+            const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
+            // lane (row r0, piece j) of round ps writes patch[(ps * VROWS + r0) * PITCH + 4 j] = 16 bytes at 16 (ps * 256 + tid)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                             (__attribute__((address_space(3))) void *)&patch[(ps * 256 + wave * 64) * 4], 16, 0, 0);
         }
     }
     else
     {
         // element e = (patch row, position inside the row segment)
-        constexpr int PER_THREAD = (NEL + 255) / 256;
-        float pv[PER_THREAD];
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j)
+        for (int j = 0; j < SPASS; ++j)
         {
             const int e = tid + j * 256;
             const int py = e / PITCH, x = e - py * PITCH;
             const int ih = ih_base + py, xe = iw_base * CI + x;
-            const bool ok = e < NEL && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
-            const float *src = ok ? img + ih * row_el + xe : g_zero_block;
-            pv[j] = *src;
+            const bool ok = py < PH && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
+            const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                             (__attribute__((address_space(3))) void *)&patch[j * 256 + wave * 64], 4, 0, 0);
         }
-#pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j)
-            if (tid + j * 256 < NEL) patch[tid + j * 256] = pv[j];
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0): this lane's pieces have landed
     __syncthreads();
 
     // patch position of reduction element k = tap * CI + ci = 4 s + kq, relative to the lane's pixel: window row k / (3 CI),
