@@ -238,7 +238,11 @@ constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks
 
 // s_begin / s_count: only K-steps [s_begin, s_begin + s_count) of the tile (s_count < 0: all of them); raw != nullptr: the
 // accumulators go there as they are ([wave][tile of the wave][register quad][lane] float4) instead of through the epilogue
-template <int COT, int PXT, bool POOL = false>
+// PW: a pointwise convolution (1x1 window, stride 1, no padding): the activation operand of a lane is its own pixel's
+// channel vector, channel block after channel block, so a K-step needs one address instruction per pixel tile where the
+// general form needs about ten (window position, bounds, select).  Every vector instruction between the MFMAs takes an
+// issue slot of the SIMD away from them (measured on a loop of this shape: 12 vector instructions per 16 MFMAs = 4%).
+template <int COT, int PXT, bool POOL = false, bool PW = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
                                               const int cg, const int pxb, const int s_begin = 0, const int s_count = -1,
                                               float *raw = nullptr)
@@ -282,6 +286,8 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        // PW: the pixel's own position (a pixel past the end reads pixel 0 of image 0 and stores nothing)
+        if (PW) in_img[t] += (size_t)(oh * a.W + ow) * CB;
     }
 
     // ---- cooperative filter fetch: COT*2 tiles of 64 float4 each -----------------------------
@@ -329,6 +335,22 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // address arithmetic between the MFMAs instead of running it after them.
     const int in_blk32 = a.H * a.W * CB;
     auto fetch = [&](float4 (&Areg)[A_PER_THREAD], float4 (&B)[PXT][2]) {
+        if (PW)
+        {
+            const int woff = cib * (CB * CB);
+#pragma unroll
+            for (int j = 0; j < A_PER_THREAD; ++j) Areg[j] = *reinterpret_cast<const float4 *>(a_src[j] + woff);
+            const int cib_off = cib * in_blk32;              // wave-uniform
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                const float4 *p = reinterpret_cast<const float4 *>(in_img[t] + cib_off);
+                B[t][0] = p[0];
+                B[t][1] = p[1];
+            }
+            cib = cib + 1 < CiB ? cib + 1 : cib;             // the two fetches past the last step repeat it
+            return;
+        }
         const int tap = ta * a.kw + tb;
         // filter first: its staging store is the first consumer, so it can wait for these loads
         // alone and leave the activation loads of the same step in flight
@@ -424,7 +446,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
 // The second launch bound (minimum waves per SIMD: 6 / 5 / 2 for one / two / four MFMA tiles per
 // wave) makes the compiler keep the accumulators in the unified register file and pack tighter
 // (2x1: 108 -> 76 registers, 2x2: 184 -> 131, no spills); measured 1-3% faster, tighter bounds spill.
-template <int COT, int PXT, bool POOL = false>
+template <int COT, int PXT, bool POOL = false, bool PW = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -432,7 +454,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
-    conv_lds_tile<COT, PXT, POOL>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+    conv_lds_tile<COT, PXT, POOL, PW>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -614,7 +636,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
 // single 32x32 tiles, each multiplied by one workgroup whose four waves split the reduction, i.e.
 // 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
 // The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
-template <int COT, int PXT, bool POOL = false>
+template <int COT, int PXT, bool POOL = false, bool PW = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -625,7 +647,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     {
         // n_main is a multiple of NUM_XCD: consecutive logical ids share an XCD
         const int lid = (bid % NUM_XCD) * (a.n_main / NUM_XCD) + bid / NUM_XCD;
-        conv_lds_tile<COT, PXT, POOL>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+        conv_lds_tile<COT, PXT, POOL, PW>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
         return;
     }
     constexpr int SUB = 4 * COT * PXT;            // 32x32 tiles per whole workgroup tile
@@ -1130,14 +1152,24 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
+    // pointwise form of the main loop (tuning knob SMALL_HIP_CONV_PW=0 switches it off)
+    static const bool pw_off = [] { const char *e = std::getenv("SMALL_HIP_CONV_PW"); return e && e[0] == '0'; }();
+    const bool pw = !pw_off && a.kh == 1 && a.kw == 1 && a.stride == 1 && a.stride_h == 1 && a.pt == 0 && a.pl == 0 &&
+                    a.Ho == a.H && a.Wo == a.W;
+    const unsigned slabs_y = a.slabs > 0 ? a.slabs : 1;
     if (tail_pays<COT, PXT>(n_main, rest, a.kh * a.kw * (a.Ci / CB)))
     {
         a.n_main = n_main;
-        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), dim3(n_main + rest * 4 * COT * PXT, a.slabs > 0 ? a.slabs : 1),
-                           dim3(256), 0, s, a);
+        const dim3 grid(n_main + rest * 4 * COT * PXT, slabs_y);
+        if (pw) hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, false, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), grid, dim3(256), 0, s, a);
     }
     else
-        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
+    {
+        const dim3 grid(a.per_xcd * NUM_XCD, slabs_y);
+        if (pw) hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, false, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), grid, dim3(256), 0, s, a);
+    }
 }
 
 // slabs > 0: a grouped convolution, `slabs` (image, group) slabs of one launch (batch must be 1: a slab is one image
