@@ -288,8 +288,10 @@ def add_floor_column(table, floors):
 
 def mfma_probe_tflops(steps=5):
     """Calibration: float32 MFMA instructions on registers only (libsmall_hip_probe.so, a measurement aid that is
-    not part of the product library), 8 workgroups per CU.  -> sustained TFLOP/s of the matrix pipes on this
-    machine (to set beside the published 157.3), or None when the probe library is not built."""
+    not part of the product library), 4 workgroups per CU (one wave per SIMD and workgroup; with 8 the same loop reads
+    138 instead of 155 TFLOP/s: past five or so waves per SIMD the matrix pipe loses issue slots to the switching between
+    them).  -> sustained TFLOP/s of the matrix pipes on this machine (to set beside the published 157.3), or None when
+    the probe library is not built."""
     import ctypes as C
     import torch
     from smallframework_amd import capi
@@ -300,7 +302,7 @@ def mfma_probe_tflops(steps=5):
     probe.restype, probe.argtypes = C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     sink = torch.zeros(4, device="cuda")
     st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    wgs, iters = 256 * 8, 20000
+    wgs, iters = 256 * 4, 20000
 
     def call():
         rc = probe(wgs, iters, C.c_void_p(sink.data_ptr()), st)

@@ -5,8 +5,9 @@ namespace
 {
 typedef float probe_x16 __attribute__((ext_vector_type(16)));
 
-// Measurement aid: every wave issues `iters` rounds of four independent v_mfma_f32_32x32x2_f32 on registers (no
-// memory traffic inside the loop), i.e. what the matrix pipes sustain on this machine at its sustained clock.
+// Measurement aid: every wave issues `iters` rounds of four v_mfma_f32_32x32x2_f32 on registers (no memory traffic
+// inside the loop), four rounds per loop iteration (a loop of four MFMAs spends a measurable part of its time in the
+// loop's own branch: 138 TFLOP/s instead of 155), i.e. what the matrix pipes sustain on this machine.
 __global__ __launch_bounds__(256) void mfma_f32_probe_kernel(int iters, float *sink)
 {
     probe_x16 acc[4];
@@ -15,10 +16,12 @@ __global__ __launch_bounds__(256) void mfma_f32_probe_kernel(int iters, float *s
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
     const float a = 1.0f + (float)(threadIdx.x & 3) * 0.25f, b = 0.5f;
-    for (int it = 0; it < iters; ++it)
+    for (int it = 0; it < iters; it += 4)
     {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
     }
     float t = 0.f;
 #pragma unroll
@@ -58,10 +61,11 @@ int shp_probe_stream(const void *in, size_t n_in16, void *out, size_t n_out16, v
     return (int)hipGetLastError();
 }
 
-// Launches `workgroups` workgroups of 4 waves, each issuing 4 * iters MFMAs; returns 0 or the HIP error code.
+// Launches `workgroups` workgroups of 4 waves, each issuing 4 * iters MFMAs (iters: a multiple of 4); returns 0 or the
+// HIP error code.
 int shp_probe_mfma_f32(int workgroups, int iters, float *sink, void *stream)
 {
-    if (workgroups <= 0 || iters <= 0 || !sink) return -1;
+    if (workgroups <= 0 || iters <= 0 || iters % 4 != 0 || !sink) return -1;
     hipLaunchKernelGGL(mfma_f32_probe_kernel, dim3((unsigned)workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                        iters, sink);
     return (int)hipGetLastError();
