@@ -288,10 +288,11 @@ def add_floor_column(table, floors):
 
 def mfma_probe_tflops(steps=5):
     """Calibration: float32 MFMA instructions on registers only (libsmall_hip_probe.so, a measurement aid that is
-    not part of the product library), 4 workgroups per CU (one wave per SIMD and workgroup; with 8 the same loop reads
-    138 instead of 155 TFLOP/s: past five or so waves per SIMD the matrix pipe loses issue slots to the switching between
-    them).  -> sustained TFLOP/s of the matrix pipes on this machine (to set beside the published 157.3), or None when
-    the probe library is not built."""
+    not part of the product library), 4 workgroups per CU (one wave per SIMD and workgroup).  With 8 workgroups per CU
+    this four-accumulator loop reads 138 instead of 155 TFLOP/s; a one-accumulator loop sustains 155 with eight waves per
+    SIMD as well, so that figure says something about the probe at that occupancy, not about the machine.
+    -> sustained TFLOP/s of the matrix pipes on this machine (to set beside the published 157.3), or None when the probe
+    library is not built."""
     import ctypes as C
     import torch
     from smallframework_amd import capi
