@@ -214,20 +214,22 @@ def time_ops(ex, steps):
 
 
 def layer_table(model, batch, ms):
-    """Per-op rows.  A convolution that carried the following 2x2 max-pool in its launch is priced on the fused
-    launch's own algorithmic bytes (its input + the pooled output + the filter); the pool's row is empty."""
+    """Per-op rows.  A convolution that carried the following 2x2 max-pool (or, a first layer, the following depthwise
+    layer) in its launch is priced on the fused launch's own algorithmic bytes (its input + the second layer's output +
+    the filters); the second layer's row is empty."""
     rows = []
     ops = model.ops
     es = model.esize()
     for i, (op, t) in enumerate(zip(ops, ms)):
         tb, kind = op_bound(model, op, batch)
         nbytes = op_bytes(model, op, batch)
-        if t == 0.0 and op.kind == "maxpool":
+        if t == 0.0 and op.kind in ("maxpool", "dw"):
             rows.append({"layer": op.name, "ms": 0.0, "bound": kind, "roofline_frac": None, "GB/s": None,
                          "TFLOP/s": None, "fused_into": "previous convolution"})
             continue
-        if op.kind == "conv" and i + 1 < len(ops) and ops[i + 1].kind == "maxpool" and ms[i + 1] == 0.0:
-            nbytes = batch * (op.act_elems()[0] + ops[i + 1].act_elems()[1]) * es + op.weight_elems() * es
+        if op.kind == "conv" and i + 1 < len(ops) and ops[i + 1].kind in ("maxpool", "dw") and ms[i + 1] == 0.0:
+            nbytes = batch * (op.act_elems()[0] + ops[i + 1].act_elems()[1]) * es + \
+                (op.weight_elems() + ops[i + 1].weight_elems()) * es
             if kind == "hbm" or nbytes / PEAK_HBM > tb:
                 tb, kind = nbytes / PEAK_HBM, "hbm"
         rows.append({"layer": op.name, "ms": round(t, 5), "bound": kind,

@@ -81,6 +81,7 @@ SIGNATURES = {
     "small_hip_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_partial_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_conv2d_bias_act_maxpool2d_f32": (_i, [_i] * 19 + [_p, _p, _p, _i, _f, _p, _p]),
+    "small_hip_conv2d_bias_act_dwconv2d_bias_act_f32": (_i, [_i] * 19 + [_p, _p, _p, _p, _p, _i, _f, _p, _p]),
     "small_hip_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_partial_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_depthwise_conv2d_bias_act_f32": (_i, _win + [_p, _p, _p, _i, _f, _p, _p]),

@@ -1117,6 +1117,166 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
     }
 }
 
+// First layer (3x3 window, 1-3 input channels) + bias + activation followed by a 3x3 stride-1 depthwise convolution with
+// one pixel of padding all round + bias + activation, in one launch (the reference's Conv2D_ReLU_DepthwiseConv2D_ReLU
+// pairing, fused_interface_abstract.hpp:1840; MobileNetV1's first two layers).  A workgroup produces a 14 x 14 tile of
+// the depthwise output: it stages the input patch and multiplies exactly like conv_stem3x3_lds_f32_kernel, but on the
+// 16 x 16 tile of first-layer pixels that the 14 x 14 depthwise outputs need (one pixel of halo all round; positions
+// outside the first layer's output are the depthwise layer's zero padding), parks the activated result of one channel
+// block in LDS as [pixel][16 channels] and runs the depthwise window on it like dw3x3_f32_tile_kernel (a lane = one
+// column, four channels, four rows, a three-row register window; the same order of operations, so the result equals
+// the two launches bit for bit).  The first layer's output (the largest tensor of the model) is never written or read.
+struct StemDwArgs
+{
+    const float *dw_filt;   // [Co/16][3][3][16]
+    const float *dw_bias;   // [Co] or nullptr
+};
+
+template <int CI, int S, int NCOB>
+__global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const ConvArgs a, const StemDwArgs d, int tiles_x, int tiles_y)
+{
+    typedef float floatx4v __attribute__((ext_vector_type(4)));
+    constexpr int T = 16, TO = 14;                           // first-layer tile side, depthwise tile side
+    constexpr int PH = (T - 1) * S + 3, PW = PH;             // input patch in pixels
+    constexpr int PITCH = PW * CI;
+    constexpr int SPASS = (PH * PITCH + 255) / 256;
+    constexpr int NEL = SPASS * 256;
+    constexpr int K = 9 * CI, NS = (K + 3) / 4;
+    __shared__ __align__(16) float patch[NEL];
+    __shared__ float4 mid[T * T * 4];                        // [row][column][channel quad] of one channel block
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, kq = lane >> 4;
+    const int CoB = a.Co / CB;
+    const int HoWo = a.Ho * a.Wo;
+    int tile = blockIdx.x;
+    const int n = tile / (tiles_x * tiles_y);
+    tile -= n * (tiles_x * tiles_y);
+    const int ty = tile / tiles_x, tx = tile - ty * tiles_x;
+    const int oh0 = ty * TO - 1, ow0 = tx * TO - 1;          // first-layer pixel of tile position (0, 0)
+    const int ih_base = oh0 * S - a.pt, iw_base = ow0 * S - a.pl;
+
+    // ---- stage the input patch (memory pipeline straight to LDS, zeros outside the image) -----------------
+    const float *img = a.in + (size_t)n * a.H * a.W * CI;
+    const int row_el = a.W * CI;
+#pragma unroll
+    for (int j = 0; j < SPASS; ++j)
+    {
+        const int e = tid + j * 256;
+        const int py = e / PITCH, x = e - py * PITCH;
+        const int ih = ih_base + py, xe = iw_base * CI + x;
+        const bool ok = py < PH && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
+        const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                         (__attribute__((address_space(3))) void *)&patch[j * 256 + wave * 64], 4, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+
+    const int lane_base = 4 * wave * S * PITCH + col * S * CI;
+    int off[NS];
+    bool kvalid[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        const int k = 4 * s + kq;
+        kvalid[s] = 4 * s + 3 < K || k < K;
+        const int kc = kvalid[s] ? k : 0;
+        const int wr = (kc >= 3 * CI ? 1 : 0) + (kc >= 6 * CI ? 1 : 0);
+        off[s] = lane_base + wr * PITCH + (kc - wr * 3 * CI);
+    }
+    const float nscale = act_scale(a.act, a.slope);
+    const int ow1 = ow0 + col;                               // first-layer column of this lane
+    const bool col_in = (unsigned)ow1 < (unsigned)a.Wo;
+
+    // depthwise phase: lane = (channel quad q, column dx, row group sy), rows sy*4 .. sy*4+3 of the 14 x 14 tile
+    const int q = tid & 3, slot = tid >> 2;
+    const int dx = slot & 15, sy = slot >> 4;
+    const int dwo = tx * TO + dx;                            // depthwise output column
+    const bool dcol_ok = dx < TO && dwo < a.Wo;
+
+#pragma unroll 1
+    for (int cb_i = 0; cb_i < NCOB; ++cb_i)
+    {
+        const int cob = blockIdx.y * NCOB + cb_i;
+        // ---- first layer on the 16 x 16 tile ---------------------------------------------------------------
+        const float *w_blk = a.filt + (size_t)cob * (K * CB) + col;
+        float av[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            const int k = 4 * s + kq;
+            const float *wp = k < K ? w_blk + k * CB : g_zero_block;
+            av[s] = *wp;
+        }
+        floatx4v acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t] = floatx4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+            {
+                const float b = patch[off[s] + t * (S * PITCH)];
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], kvalid[s] ? b : 0.f, acc[t], 0, 0, 0);
+            }
+        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
+        if (cb_i > 0) __syncthreads();                       // the previous block's depthwise reads are done
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+        {
+            const int row = 4 * wave + t, oh1 = oh0 + row;
+            float4 v = make_float4(acc[t][0] + bb.x, acc[t][1] + bb.y, acc[t][2] + bb.z, acc[t][3] + bb.w);
+            v.x = act_bf(v.x, nscale); v.y = act_bf(v.y, nscale); v.z = act_bf(v.z, nscale); v.w = act_bf(v.w, nscale);
+            // outside the first layer's output: the depthwise layer's padding
+            if (!(col_in && (unsigned)oh1 < (unsigned)a.Ho)) v = make_float4(0.f, 0.f, 0.f, 0.f);
+            mid[(row * T + col) * 4 + kq] = v;
+        }
+        __syncthreads();
+
+        // ---- depthwise 3x3 on the parked tile ----------------------------------------------------------------
+        const float4 *wq = reinterpret_cast<const float4 *>(d.dw_filt) + (size_t)cob * 36 + q;
+        float4 w[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) w[t] = wq[t * 4];
+        float4 dbias = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (d.dw_bias) dbias = *reinterpret_cast<const float4 *>(d.dw_bias + cob * CB + 4 * q);
+        const float4 *xs = mid + ((sy * 4) * T + (dx < TO ? dx : 0)) * 4 + q;     // idle columns read in bounds
+        float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)(n * CoB + cob) * HoWo + dwo) * 4 + q;
+        float4 win[3][3];
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[r][c] = xs[(r * T + c) * 4];
+#pragma unroll
+        for (int o = 0; o < 4; ++o)
+        {
+            const int lr = sy * 4 + o;                       // row inside the 14 x 14 tile
+            const int rr = lr + 2 < T ? o + 2 : o;           // rows 14, 15 of the tile have no third window row: not stored
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[(o + 2) % 3][c] = xs[(rr * T + c) * 4];
+            const int oh = ty * TO + lr;
+            const bool ok = dcol_ok && lr < TO && oh < a.Ho;
+            float4 acc2 = dbias;
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int c = 0; c < 3; ++c)
+                {
+                    const float4 x = win[(o + r) % 3][c];
+                    const float4 k = w[r * 3 + c];
+                    acc2.x = fmaf(x.x, k.x, acc2.x); acc2.y = fmaf(x.y, k.y, acc2.y);
+                    acc2.z = fmaf(x.z, k.z, acc2.z); acc2.w = fmaf(x.w, k.w, acc2.w);
+                }
+            acc2.x = act_bf(acc2.x, nscale); acc2.y = act_bf(acc2.y, nscale);
+            acc2.z = act_bf(acc2.z, nscale); acc2.w = act_bf(acc2.w, nscale);
+            if (ok) dst[(size_t)oh * a.Wo * 4] = acc2;
+        }
+    }
+}
+
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
@@ -1450,6 +1610,53 @@ int conv_pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt,
     return SMALL_HIP_OK;
 }
 
+// First layer + bias + activation + DepthwiseConv2D 3x3 stride 1 (one pixel of padding) + bias + activation in one launch
+int stem_dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int dw_kh, int dw_kw,
+                int dw_stride, int dpt, int dpb, int dpl, int dpr, int Co, int Ci, int H, int W, const float *in,
+                const float *filt, const float *bias, const float *dw_filt, const float *dw_bias, int act, float slope,
+                float *out, small_hip_stream_t stream)
+{
+    if (Ci != 1 && Ci != 2 && Ci != 3)
+    { set_error("%s: only first layers (1-3 input channels) are fused with the depthwise layer", op); return SMALL_HIP_EINVAL; }
+    if (stride != 1 && stride != 2) return SMALL_HIP_ESTRIDE;
+    if (kh != 3 || kw != 3 || dw_kh != 3 || dw_kw != 3 || dw_stride != 1 || dpt != 1 || dpb != 1 || dpl != 1 || dpr != 1)
+    { set_error("%s: fused for a 3x3 convolution followed by a 3x3 stride-1 depthwise convolution with padding 1", op); return SMALL_HIP_EINVAL; }
+    if (batch <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(pt, pb, pl, pr)) { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (Co % CB != 0) { set_error("%s: output_channels must be a multiple of 16 (pad the filter)", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !dw_filt || !out || !aligned16(filt) || !aligned16(dw_filt) || !aligned16(out) ||
+        (bias && !aligned16(bias)) || (dw_bias && !aligned16(dw_bias)))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place operation is not supported", op); return SMALL_HIP_EINVAL; }
+    if (act < SMALL_HIP_ACT_NONE || act > SMALL_HIP_ACT_LEAKY) { set_error("%s: bad activation", op); return SMALL_HIP_EINVAL; }
+
+    ConvArgs a{};
+    a.in = in; a.filt = filt; a.bias = bias; a.out = out;
+    a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W;
+    a.kh = 3; a.kw = 3; a.stride = stride; a.stride_h = stride; a.pt = pt; a.pl = pl;
+    a.Ho = out_dim(H, pt, pb, 3, stride);
+    a.Wo = out_dim(W, pl, pr, 3, stride);
+    a.act = act; a.slope = slope; a.accumulate = 0;
+    if (a.Ho <= 0 || a.Wo <= 0) return SMALL_HIP_OK;
+    if ((long)Ci * H * W > 0x7fffffffL / 2) { set_error("%s: one image too large for 32-bit offsets", op); return SMALL_HIP_EINVAL; }
+    const int tiles_x = (a.Wo + 13) / 14, tiles_y = (a.Ho + 13) / 14;
+    const long nt = (long)batch * tiles_x * tiles_y;
+    if (nt > 0x7fffffffL || (long)batch * Co * a.Ho * a.Wo > 0x7fffffffL * 4L)
+    { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
+    a.P = batch * a.Ho * a.Wo;
+    const int CoB = Co / CB;
+    const int ncob = CoB % 2 == 0 ? 2 : 1;
+    const StemDwArgs d{dw_filt, dw_bias};
+    const dim3 gs((unsigned)nt, (unsigned)(CoB / ncob));
+    void (*ks)(const ConvArgs, const StemDwArgs, int, int) = nullptr;
+#define SHP_SD(CI_, S_) (ncob == 2 ? conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 2> : conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 1>)
+    if (stride == 1) ks = Ci == 1 ? SHP_SD(1, 1) : Ci == 2 ? SHP_SD(2, 1) : SHP_SD(3, 1);
+    else ks = Ci == 1 ? SHP_SD(1, 2) : Ci == 2 ? SHP_SD(2, 2) : SHP_SD(3, 2);
+#undef SHP_SD
+    hipLaunchKernelGGL(ks, gs, dim3(256), 0, as_stream(stream), a, d, tiles_x, tiles_y);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -1496,6 +1703,16 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kh, int kw, int strid
 {
     return conv_pool_f32("small_hip_conv2d_bias_act_maxpool2d_f32", batch, kh, kw, stride, pt, pb, pl, pr, pool_kh,
                          pool_kw, pool_stride, ppt, ppb, ppl, ppr, Co, Ci, H, W, in, filt, bias, act, slope, out, stream);
+}
+
+int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                                    int dw_kh, int dw_kw, int dw_stride, int dpt, int dpb, int dpl, int dpr,
+                                                    int Co, int Ci, int H, int W, const float *in, const float *filt,
+                                                    const float *bias, const float *dw_filt, const float *dw_bias, int act,
+                                                    float slope, float *out, small_hip_stream_t stream)
+{
+    return stem_dw_f32("small_hip_conv2d_bias_act_dwconv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw,
+                       dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
 }
 
 // One convolution of `channels` -> `channels` per slab of `channels` channels; slab g of image n starts

@@ -394,6 +394,20 @@ class HipExecutor:
                 self.plan.append((conv, pool, False))
                 i = j + 1
                 continue
+            if (fused and model.dtype == "f32" and op.kind == "conv" and op.C in (1, 2, 3) and (op.kh, op.kw) == (3, 3)
+                    and j < len(ops) and ops[j].kind == "dw" and ops[j].src == op.dst
+                    and (ops[j].kh, ops[j].kw, ops[j].stride) == (3, 3, 1) and ops[j].pads == (1, 1, 1, 1)
+                    and ops[j].act == op.act and ops[j].slope == op.slope
+                    and not self._read_before_rewritten(ops[j + 1:], op.dst, model.out)):
+                # a first layer and the depthwise layer after it in one launch (the first layer's output is never
+                # written); as above, the result must not land on the convolution's input
+                conv, dw = at(op), at(ops[j])
+                if dw.dst == conv.src:
+                    phys[ops[j].dst], phys[op.dst] = conv.dst, dw.dst
+                    dw = replace(dw, dst=conv.dst)
+                self.plan.append((conv, dw, False))
+                i = j + 1
+                continue
             if fused and model.dtype == "u8" and op.kind == "conv":
                 if j < len(ops) and ops[j].kind == "accum" and ops[j].dst == op.dst and ops[j].src != op.dst:
                     acc_op = ops[j]
@@ -460,6 +474,8 @@ class HipExecutor:
         op, acc_op, relu = entry
         if acc_op is not None and acc_op.kind == "maxpool":
             self.run_conv_pool_f32(op, acc_op, st)
+        elif acc_op is not None and acc_op.kind == "dw":
+            self.run_conv_dw_f32(op, acc_op, st)
         elif acc_op is not None or relu:
             self.run_fused_u8(op, acc_op, relu, st)
         else:
@@ -473,6 +489,15 @@ class HipExecutor:
         capi.check(L.small_hip_conv2d_bias_act_maxpool2d_f32(
             self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 2, 2, 2, 0, 0, 0, 0, op.Co, op.C, op.H, op.W,
             p(b[op.src]), p(self.w[op.weight]), None, act, op.slope, p(b[pool.dst]), st))
+
+    def run_conv_dw_f32(self, op, dw, st):
+        """First-layer Conv2D + activation + DepthwiseConv2D 3x3 stride 1 + activation in one launch."""
+        L, p, b = self.lib, self._p, self.buf
+        act = {None: capi.ACT_NONE, "relu": capi.ACT_RELU, "leaky": capi.ACT_LEAKY}[op.act]
+        t_, b_, l_, r_ = op.pads
+        capi.check(L.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(
+            self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 3, 3, 1, 1, 1, 1, 1, op.Co, op.C, op.H, op.W,
+            p(b[op.src]), p(self.w[op.weight]), None, p(self.w[dw.weight]), None, act, op.slope, p(b[dw.dst]), st))
 
     def run_op(self, op: Op, st):
         L, p, B, b = self.lib, self._p, self.batch, self.buf

@@ -1,0 +1,93 @@
+"""A first layer and the depthwise layer after it in one launch (small_hip_conv2d_bias_act_dwconv2d_bias_act_f32; the
+reference's Conv2D_ReLU_DepthwiseConv2D_ReLU family, fused_interface_abstract.hpp:1840): checked through the C ABI
+against the two layers of the CPU oracle (float32 bar) and, bit for bit, against this library's own two launches."""
+import numpy as np
+import pytest
+
+from smallframework_amd import capi, synth
+from util import assert_close_f32, assert_equal_exact
+import hip_util as hu
+
+pytestmark = pytest.mark.gpu
+CB = 16
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return capi.load()
+
+
+# (batch, stride, conv pads(t,b,l,r), Co, Ci, H, W, conv bias, depthwise bias, act)
+CASES = [
+    (1, 2, (0, 1, 0, 1), 32, 3, 32, 32, False, False, capi.ACT_RELU),        # MobileNetV1's first two layers, small
+    (2, 1, (1, 1, 1, 1), 16, 3, 20, 23, True, True, capi.ACT_RELU),          # one channel block, ragged 14 x 14 tiles
+    (3, 2, (0, 1, 0, 1), 48, 1, 37, 29, True, False, capi.ACT_LEAKY),        # three channel blocks (one per pass), 1 channel
+    (1, 1, (1, 1, 1, 1), 32, 2, 14, 14, False, True, capi.ACT_NONE),         # exactly one tile
+    (2, 2, (1, 1, 1, 1), 64, 3, 57, 61, True, True, capi.ACT_RELU),          # odd sizes, four channel blocks
+    (1, 1, (0, 0, 0, 0), 16, 3, 5, 5, True, True, capi.ACT_RELU),            # 3 x 3 first-layer output
+    (4, 2, (0, 1, 0, 1), 32, 3, 224, 224, False, False, capi.ACT_RELU),      # MobileNetV1's real size
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=str)
+def test_conv_dw_vs_oracle_and_two_launches(lib, oracle, case):
+    batch, s, (pt, pb, pl, pr), Co, Ci, H, W, has_b, has_db, act = case
+    x = synth.normal(1, batch * Ci * H * W)
+    f = synth.he_normal(2, Co * Ci * 9, Ci * 9)
+    bias = synth.normal(3, Co)
+    dwf = synth.he_normal(4, Co * 9, 9)
+    dwb = synth.normal(5, Co)
+    Ho, Wo = oracle.out_hw(3, 3, s, pt, pb, pl, pr, H, W)
+    dx, df, ddf = hu.dev(x), hu.dev(f), hu.dev(dwf)
+    db = hu.dev(bias) if has_b else None
+    ddb = hu.dev(dwb) if has_db else None
+    do = hu.dev_empty(batch * Co * Ho * Wo, np.float32)
+    rc = lib.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(batch, 3, 3, s, pt, pb, pl, pr, 3, 3, 1, 1, 1, 1, 1, Co, Ci, H, W,
+                                                             hu.ptr(dx), hu.ptr(df), hu.ptr(db), hu.ptr(ddf), hu.ptr(ddb), act, 0.1,
+                                                             hu.ptr(do), hu.stream())
+    assert rc == 0, lib.small_hip_last_error()
+    got = hu.host(do)
+
+    # this library's two launches: bit for bit
+    dmid = hu.dev_empty(batch * Co * Ho * Wo, np.float32)
+    d2 = hu.dev_empty(batch * Co * Ho * Wo, np.float32)
+    assert lib.small_hip_conv2d_bias_act_f32(batch, 3, 3, s, pt, pb, pl, pr, Co, Ci, H, W, hu.ptr(dx), hu.ptr(df), hu.ptr(db), act, 0.1,
+                                             hu.ptr(dmid), hu.stream()) == 0, lib.small_hip_last_error()
+    assert lib.small_hip_depthwise_conv2d_bias_act_f32(batch, 3, 3, 1, 1, 1, 1, 1, Co, Ho, Wo, hu.ptr(dmid), hu.ptr(ddf), hu.ptr(ddb),
+                                                       act, 0.1, hu.ptr(d2), hu.stream()) == 0, lib.small_hip_last_error()
+    assert_equal_exact(got, hu.host(d2), "fused first layer + depthwise against the two launches %s" % (case,))
+
+    # the oracle's two layers
+    if batch * Ho * Wo * Co * Ci * 9 <= 2e9:
+        rc, mid = oracle.conv2d_bias_act_f32(batch, CB, 3, 3, s, pt, pb, pl, pr, Co, Ci, H, W, x, f, bias if has_b else None, act, 0.1)
+        assert rc == 0
+        # the depthwise layer as the reference composes it: bias, convolution added onto it, activation
+        o1 = None
+        if has_db:
+            _, o1 = oracle.bias_f32(batch, CB, Co, Ho, Wo, dwb)
+        rc, want = oracle.dwconv2d_f32(batch, CB, 3, 3, 1, 1, 1, 1, 1, Co, Ho, Wo, mid, dwf, out=o1, accumulate=1 if has_db else 0)
+        assert rc == 0
+        if act == capi.ACT_RELU:
+            _, want = oracle.relu_f32(batch, CB, Co, Ho, Wo, want)
+        elif act == capi.ACT_LEAKY:
+            _, want = oracle.leaky_relu_f32(batch, CB, Co, Ho, Wo, want, 0.1)
+        assert_close_f32(got, want, what=str(case))
+        assert np.abs(want).max() > 0.05
+
+
+def test_conv_dw_refusals(lib):
+    import torch
+    t = torch.zeros(1 << 16, device="cuda")
+    p, st = hu.ptr(t), hu.stream()
+    call = lambda Ci=3, k=3, s=2, dk=3, ds=1, dp=1, Co=32: lib.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(
+        1, k, k, s, 0, 1, 0, 1, dk, dk, ds, dp, dp, dp, dp, Co, Ci, 16, 16, p, p, None, p, None, capi.ACT_RELU, 0.0, hu.ptr(t[4096:]), st)
+    assert call() == capi.OK
+    assert call(Ci=16) == capi.EINVAL            # not a first layer
+    assert call(k=5) == capi.EINVAL
+    assert call(s=3) == capi.ESTRIDE
+    assert call(dk=5) == capi.EINVAL
+    assert call(ds=2) == capi.EINVAL
+    assert call(dp=0) == capi.EINVAL
+    assert call(Co=24) == capi.EINVAL
