@@ -983,44 +983,67 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
     tile -= n * (tiles_x * tiles_y);
     const int ty = tile / tiles_x, tx = tile - ty * tiles_x;
     const int oh0 = ty * T, ow0 = tx * T;
-    const int ih_base = oh0 * S - a.pt, iw_base = ow0 * S - a.pl;
+    const int iw_base = ow0 * S - a.pl;
+
+    // the first channel block's filter and bias are requested before the patch, so that one memory latency covers both
+    // filter: element k of channel co at w_blk[k * 16 + co % 16]; this lane's k in step s is 4s + kq
+    float av[NS];
+    float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto load_filter = [&](const int cob) {
+        const float *w_blk = a.filt + (size_t)cob * (K * CB) + col;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            const int k = 4 * s + kq;
+            const float *wp = k < K ? w_blk + k * CB : g_zero_block;
+            av[s] = *wp;
+        }
+        if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
+    };
+    load_filter(blockIdx.y * NCOB);
 
     // ---- stage the patch --------------------------------------------------------------------------------
-    const float *img = a.in + (size_t)n * a.H * a.W * CI;
+    // stage_patch(tile id, LDS base of round 0, LDS floats between rounds): requests the patch under tile `t` of the launch
     const int row_el = a.W * CI;                             // floats per image row
-    int lead = 0;
-    if (VEC)
-    {
-        const int x0 = iw_base * CI;
-        lead = x0 & 3;                                       // two's complement: also right for x0 = -CI
-        const int xa = x0 - lead;                            // multiple of 4
-        const int j = tid & (J - 1), r0 = tid / J;
-#pragma unroll
-        for (int ps = 0; ps < VPASS; ++ps)
+    const int lead = VEC ? ((iw_base * CI) & 3) : 0;         // two's complement: also right for -CI; the same for every tile
+    auto stage_patch = [&](int t, float *dst, const int round_floats) {
+        const int n_ = t / (tiles_x * tiles_y);
+        t -= n_ * (tiles_x * tiles_y);
+        const int ty_ = t / tiles_x, tx_ = t - ty_ * tiles_x;
+        const int ih_base = ty_ * T * S - a.pt, iw_b = tx_ * T * S - a.pl;
+        const float *img = a.in + (size_t)n_ * a.H * a.W * CI;
+        if (VEC)
         {
-            const int py = r0 + ps * VROWS, ih = ih_base + py, xe = xa + 4 * j;
-            const bool ok = j < P4 && py < PH && (unsigned)ih < (unsigned)a.H && xe >= 0 && xe < row_el;
-            const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
-            // lane (row r0, piece j) of round ps writes patch[(ps * VROWS + r0) * PITCH + 4 j] = 16 bytes at 16 (ps * 256 + tid)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)&patch[(ps * 256 + wave * 64) * 4], 16, 0, 0);
-        }
-    }
-    else
-    {
-        // element e = (patch row, position inside the row segment)
+            const int xa = iw_b * CI - lead;                 // multiple of 4
+            const int j = tid & (J - 1), r0 = tid / J;
 #pragma unroll
-        for (int j = 0; j < SPASS; ++j)
-        {
-            const int e = tid + j * 256;
-            const int py = e / PITCH, x = e - py * PITCH;
-            const int ih = ih_base + py, xe = iw_base * CI + x;
-            const bool ok = py < PH && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
-            const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)&patch[j * 256 + wave * 64], 4, 0, 0);
+            for (int ps = 0; ps < VPASS; ++ps)
+            {
+                const int py = r0 + ps * VROWS, ih = ih_base + py, xe = xa + 4 * j;
+                const bool ok = j < P4 && py < PH && (unsigned)ih < (unsigned)a.H && xe >= 0 && xe < row_el;
+                const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
+                // lane (row r0, piece j) of round ps writes patch[(ps * VROWS + r0) * PITCH + 4 j] = 16 bytes at 16 (ps * 256 + tid)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                                 (__attribute__((address_space(3))) void *)&dst[ps * round_floats + wave * 64 * 4], 16, 0, 0);
+            }
         }
-    }
+        else
+        {
+            // element e = (patch row, position inside the row segment)
+#pragma unroll
+            for (int j = 0; j < SPASS; ++j)
+            {
+                const int e = tid + j * 256;
+                const int py = e / PITCH, x = e - py * PITCH;
+                const int ih = ih_base + py, xe = iw_b * CI + x;
+                const bool ok = py < PH && (unsigned)ih < (unsigned)a.H && (unsigned)xe < (unsigned)row_el;
+                const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                                 (__attribute__((address_space(3))) void *)&dst[j * round_floats + wave * 64], 4, 0, 0);
+            }
+        }
+    };
+    stage_patch(blockIdx.x, patch, VEC ? 256 * 4 : 256);
     __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0): this lane's pieces have landed
     __syncthreads();
 
@@ -1046,16 +1069,7 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
     for (int cb_i = 0; cb_i < NCOB; ++cb_i)
     {
         const int cob = blockIdx.y * NCOB + cb_i;            // the launcher makes Co / 16 a multiple of NCOB
-        // filter: element k of channel co at w_blk[k * 16 + co % 16]; this lane's k in step s is 4s + kq
-        const float *w_blk = a.filt + (size_t)cob * (K * CB) + col;
-        float av[NS];
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-        {
-            const int k = 4 * s + kq;
-            const float *wp = k < K ? w_blk + k * CB : g_zero_block;
-            av[s] = *wp;
-        }
+        if (cb_i > 0) load_filter(cob);
         floatx4v acc[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[t] = floatx4v{0.f, 0.f, 0.f, 0.f};
@@ -1068,8 +1082,6 @@ __global__ __launch_bounds__(256) void conv_stem3x3_lds_f32_kernel(const ConvArg
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], kvalid[s] ? b : 0.f, acc[t], 0, 0, 0);
             }
         // lane: channels cob*16 + 4*kq .. +3 of pixel (oh0 + 4w + t, ow0 + col)
-        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
         if (POOL)
         {
             // MaxPool2D 2x2 stride 2 (no padding) of the activated result, in registers: tile rows t and
@@ -1144,6 +1156,11 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
     constexpr int K = 9 * CI, NS = (K + 3) / 4;
     __shared__ __align__(16) float patch[NEL];
     __shared__ float4 mid[T * T * 4];                        // [row][column][channel quad] of one channel block
+    // Both layers' filters and biases of the workgroup's channel blocks, staged with the patch: the passes below then read
+    // them from LDS instead of waiting for memory twice per pass.  Per block: F4 pieces of first-layer filter, 36 of
+    // depthwise filter, 4 + 4 of the two biases (zeros where there is none); a piece is 16 bytes.
+    constexpr int F4 = K * CB / 4, PB = F4 + 44, NP = NCOB * PB, PRND = (NP + 255) / 256;
+    __shared__ float4 par[PRND * 256];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1170,6 +1187,26 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
         const float *gp = ok ? img + ih * row_el + xe : g_zero_block;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
                                          (__attribute__((address_space(3))) void *)&patch[j * 256 + wave * 64], 4, 0, 0);
+    }
+    {
+        const int cob0 = blockIdx.y * NCOB;
+        const float4 *zero4 = reinterpret_cast<const float4 *>(g_zero_block);
+#pragma unroll
+        for (int r = 0; r < PRND; ++r)
+        {
+            const int piece = tid + r * 256;
+            const int b = piece / PB, i = piece - b * PB, cob = cob0 + b;
+            const float4 *gp = zero4;
+            if (piece < NP)
+            {
+                if (i < F4) gp = reinterpret_cast<const float4 *>(a.filt + (size_t)cob * (K * CB)) + i;
+                else if (i < F4 + 36) gp = reinterpret_cast<const float4 *>(d.dw_filt) + (size_t)cob * 36 + (i - F4);
+                else if (i < F4 + 40) { if (a.bias) gp = reinterpret_cast<const float4 *>(a.bias + cob * CB) + (i - F4 - 36); }
+                else if (d.dw_bias) gp = reinterpret_cast<const float4 *>(d.dw_bias + cob * CB) + (i - F4 - 40);
+            }
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                             (__attribute__((address_space(3))) void *)&par[r * 256 + wave * 64], 16, 0, 0);
+        }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
@@ -1201,14 +1238,14 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
     {
         const int cob = blockIdx.y * NCOB + cb_i;
         // ---- first layer on the 16 x 16 tile ---------------------------------------------------------------
-        const float *w_blk = a.filt + (size_t)cob * (K * CB) + col;
+        const float4 *pb = par + cb_i * PB;                  // this block's staged parameters
+        const float *w_blk = reinterpret_cast<const float *>(pb) + col;
         float av[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
             const int k = 4 * s + kq;
-            const float *wp = k < K ? w_blk + k * CB : g_zero_block;
-            av[s] = *wp;
+            av[s] = k < K ? w_blk[(k < K ? k : 0) * CB] : 0.f;
         }
         floatx4v acc[4];
 #pragma unroll
@@ -1221,8 +1258,7 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
                 const float b = patch[off[s] + t * (S * PITCH)];
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], kvalid[s] ? b : 0.f, acc[t], 0, 0, 0);
             }
-        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (a.bias) bb = *reinterpret_cast<const float4 *>(a.bias + cob * CB + 4 * kq);
+        const float4 bb = pb[F4 + 36 + kq];
         if (cb_i > 0) __syncthreads();                       // the previous block's depthwise reads are done
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -1237,12 +1273,10 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
         __syncthreads();
 
         // ---- depthwise 3x3 on the parked tile ----------------------------------------------------------------
-        const float4 *wq = reinterpret_cast<const float4 *>(d.dw_filt) + (size_t)cob * 36 + q;
         float4 w[9];
 #pragma unroll
-        for (int t = 0; t < 9; ++t) w[t] = wq[t * 4];
-        float4 dbias = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (d.dw_bias) dbias = *reinterpret_cast<const float4 *>(d.dw_bias + cob * CB + 4 * q);
+        for (int t = 0; t < 9; ++t) w[t] = pb[F4 + t * 4 + q];
+        const float4 dbias = pb[F4 + 40 + q];
         const float4 *xs = mid + ((sy * 4) * T + (dx < TO ? dx : 0)) * 4 + q;     // idle columns read in bounds
         float4 *dst = reinterpret_cast<float4 *>(a.out) + ((size_t)(n * CoB + cob) * HoWo + dwo) * 4 + q;
         float4 win[3][3];
