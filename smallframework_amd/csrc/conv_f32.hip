@@ -106,7 +106,8 @@ __device__ __forceinline__ float act_bf(float v, float neg_scale)
 // per channel quad, PartialConv2D (ACC) is a compile-time variant.
 template <int COT, int PXT, bool ACC>
 __device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
-                                                   int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+                                                   int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT],
+                                                   const float *lds_bias)
 {
     const float nscale = act_scale(a.act, a.slope);
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -115,7 +116,15 @@ __device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (
     for (int c = 0; c < COT; ++c)
 #pragma unroll
         for (int q = 0; q < 4; ++q) bb[c][q] = zero;
-    if (a.bias)
+    if (lds_bias)
+    {
+        // the workgroup's bias values (zeros without a bias or past the last channel), parked in LDS before the K loop
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) bb[c][q] = *reinterpret_cast<const float4 *>(lds_bias + c * 32 + 8 * q + 4 * half);
+    }
+    else if (a.bias)
     {
 #pragma unroll
         for (int c = 0; c < COT; ++c)
@@ -159,10 +168,11 @@ __device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (
 
 template <int COT, int PXT>
 __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
-                                              int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT])
+                                              int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT],
+                                              const float *lds_bias = nullptr)
 {
-    if (a.accumulate) conv_epilogue_impl<COT, PXT, true>(a, acc, cg, half, HoWo, pvalid, out_pix);
-    else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    if (a.accumulate) conv_epilogue_impl<COT, PXT, true>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
+    else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
 }
 
 // Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 8 pooling windows of
@@ -171,7 +181,8 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
 // into [N][Co/16][Ho/2][Wo/2][16].
 template <int COT, int PXT>
 __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
-                                                   const bool (&pool_ok)[PXT], const size_t (&pool_pix)[PXT])
+                                                   const bool (&pool_ok)[PXT], const size_t (&pool_pix)[PXT],
+                                                   const float *lds_bias = nullptr)
 {
     const float nscale = act_scale(a.act, a.slope);
     const int HpWp = (a.Ho >> 1) * (a.Wo >> 1);
@@ -182,7 +193,8 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
         {
             const int co4 = (cg * COT + c) * 32 + 8 * q + 4 * half;
             float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (a.bias && co4 < a.Co) bb = *reinterpret_cast<const float4 *>(a.bias + co4);
+            if (lds_bias) bb = *reinterpret_cast<const float4 *>(lds_bias + c * 32 + 8 * q + 4 * half);
+            else if (a.bias && co4 < a.Co) bb = *reinterpret_cast<const float4 *>(a.bias + co4);
             const float b4[4] = {bb.x, bb.y, bb.z, bb.w};
 #pragma unroll
             for (int t = 0; t < PXT; ++t)
@@ -242,7 +254,10 @@ constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks
 // channel vector, channel block after channel block, so a K-step needs one address instruction per pixel tile where the
 // general form needs about ten (window position, bounds, select).  Every vector instruction between the MFMAs takes an
 // issue slot of the SIMD away from them (measured on a loop of this shape: 12 vector instructions per 16 MFMAs = 4%).
-template <int COT, int PXT, bool POOL = false, bool PW = false>
+// BLDS: the workgroup runs this body once; its bias values are requested first of all and parked in LDS under the K loop, so
+// the epilogue does not wait for memory once more (a caller that runs several tiles per workgroup would overwrite them
+// while another wave still reads)
+template <int COT, int PXT, bool POOL = false, bool PW = false, bool BLDS = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
                                               const int cg, const int pxb, const int s_begin = 0, const int s_count = -1,
                                               float *raw = nullptr)
@@ -252,6 +267,13 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     const int wave = tid >> 6;
     const int col = lane & 31;
     const int half = lane >> 5;
+    __shared__ __align__(16) float s_bias[BLDS ? COT * 32 : 4];
+    float my_bias = 0.f;
+    if (BLDS && tid < COT * 32)
+    {
+        const int co = cg * COT * 32 + tid;
+        if (a.bias && co < a.Co) my_bias = a.bias[co];
+    }
 
     const int HoWo = a.Ho * a.Wo;
     const int CiB = a.Ci / CB;
@@ -410,6 +432,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     float4 B0[PXT][2], B1[PXT][2];
     fetch(Areg, B0);                 // step 0
     stage(0, Areg);
+    if (BLDS && tid < COT * 32) s_bias[tid] = my_bias;      // requested before the filter, so it is here by now
     fetch(Areg, B1);                 // step 1
     __syncthreads();
     const int npairs = nsteps >> 1;
@@ -439,8 +462,8 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
                     r4[((c * PXT + t) * 4 + q) * WAVE] = make_float4(acc[c][t][4 * q], acc[c][t][4 * q + 1], acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
         return;
     }
-    if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix);
-    else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix);
+    if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix, BLDS ? s_bias : nullptr);
+    else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix, BLDS ? s_bias : nullptr);
 }
 
 // The second launch bound (minimum waves per SIMD: 6 / 5 / 2 for one / two / four MFMA tiles per
@@ -454,7 +477,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
-    conv_lds_tile<COT, PXT, POOL, PW>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+    conv_lds_tile<COT, PXT, POOL, PW, true>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -647,7 +670,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     {
         // n_main is a multiple of NUM_XCD: consecutive logical ids share an XCD
         const int lid = (bid % NUM_XCD) * (a.n_main / NUM_XCD) + bid / NUM_XCD;
-        conv_lds_tile<COT, PXT, POOL, PW>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+        conv_lds_tile<COT, PXT, POOL, PW, true>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
         return;
     }
     constexpr int SUB = 4 * COT * PXT;            // 32x32 tiles per whole workgroup tile
