@@ -579,8 +579,15 @@ def main():
                                                     if "stream_floor_ms" in r else ""))
 
     # dominant kernel = the one with the largest summed time
+    # convolutions that carry the depthwise layer after them run in kernels of their own (first layer: conv_stem3x3_dw3x3,
+    # pointwise: conv_pw_dw3x3); the depthwise layer's row has no launch
+    with_dw = {e[0].name for e in getattr(ex, "plan", []) if e[1] is not None and e[1].kind == "dw"} \
+        if model.dtype == "f32" and getattr(ex, "fused", False) else set()
+
     def kernel_of(op):
         if op.kind in ("conv", "dense"):
+            if op.name in with_dw:
+                return "conv_stem3x3_dw3x3_f32_kernel" if op.C % 16 != 0 else "conv_pw_dw3x3_f32_kernel"
             if op.C % 16 != 0:
                 return "conv_smallci_%s_kernel" % model.dtype
             return "conv_mfma_%s_*" % model.dtype
@@ -588,7 +595,9 @@ def main():
                 "avgpool": "pool_%s_kernel" % model.dtype}.get(op.kind, "ew_%s_kernel" % model.dtype)
 
     per_kernel = {}
-    for op, t in zip(model.ops, ms):
+    for i, (op, t) in enumerate(zip(model.ops, ms)):
+        if t == 0.0 and op.kind in ("maxpool", "dw") and i > 0 and model.ops[i - 1].kind == "conv":
+            continue                                   # ran inside the previous convolution's launch
         k = kernel_of(op)
         d = per_kernel.setdefault(k, {"ms": 0.0, "launches": 0, "flops": 0.0, "bytes": 0.0})
         d["ms"] += t

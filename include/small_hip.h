@@ -125,13 +125,18 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kernel_height, int ke
                                             const float *bias, int act, float negative_slope, float *output,
                                             small_hip_stream_t stream);
 /* small::Conv2D_ReLU_DepthwiseConv2D_ReLU / Conv2D_Bias_ReLU_DepthwiseConv2D_Bias_ReLU
- * (include/small/fused_interface_abstract.hpp:1840, 1513-2500) in one launch for a first layer:
+ * (include/small/fused_interface_abstract.hpp:1840, 1513-2500) in one launch:
  *     out = act( DepthwiseConv2D( act( Conv2D(in, filter) + bias ), dw_filter ) + dw_bias )
- * Fused here for 1-3 input channels, a 3x3 convolution of stride 1 or 2, and a 3x3 stride-1 depthwise convolution
- * with one pixel of padding on every side (EINVAL otherwise: issue the two layers).  The first layer's output never
- * goes to memory; no intermediate buffer is needed.  dw_filter is [Co/16][3][3][16], either bias may be null; one
- * activation for both layers.  output is [batch][Co/16][Ho][Wo][16] with Ho, Wo the convolution's output size.  The
- * result equals the two layers run one after the other bit for bit. */
+ * Fused here (EINVAL otherwise: issue the two layers) for
+ *  - a first layer: 1-3 input channels, a 3x3 convolution of stride 1 or 2, and a 3x3 stride-1 depthwise convolution
+ *    with one pixel of padding on every side;
+ *  - a pointwise convolution (1x1 window, stride 1, no padding) of 32, 64 or 128 input channels and output channels in
+ *    whole groups of 32, and a 3x3 depthwise convolution of stride 1 or 2 with any padding (ESTRIDE for other strides).
+ * The convolution's output never goes to memory; no intermediate buffer is needed.  dw_filter is [Co/16][3][3][16],
+ * either bias may be null; one activation for both layers.  output is [batch][Co/16][Hd][Wd][16] with Hd, Wd the
+ * depthwise layer's output size.  The result equals the two layers run one after the other bit for bit where the
+ * stand-alone convolution adds its products in one pass (always but for 128 input channels, where it may split
+ * left-over tiles along the input channels: float32 rounding then). */
 int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,
                                                     int t_pad, int b_pad, int l_pad, int r_pad, int dw_kernel_height,
                                                     int dw_kernel_width, int dw_stride, int dw_t_pad, int dw_b_pad,

@@ -1334,6 +1334,222 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
     }
 }
 
+// Pointwise convolution (1x1 window, stride 1, no padding; 16 * CIB input channels) + bias + activation followed by a 3x3
+// depthwise convolution of stride S + bias + activation, in one launch: the reference's Conv2D_ReLU_DepthwiseConv2D_ReLU
+// pairing (fused_interface_abstract.hpp:1840) for the blocked layers, MobileNetV1's 1x1 -> 3x3 depthwise sequence.  The
+// pointwise layer's output, the largest tensor of such a pair, is neither written nor read.
+// A workgroup owns 32 * COT channels and a tile of TOH x TOW depthwise outputs of one image (14 x 14 at stride 1, 7 x 8 at
+// stride 2).  The PH x PW pointwise pixels under that tile (16 x 16 / 15 x 17, at most 256) are eight 32-pixel MFMA tiles,
+// two per wave; the filter slice of the workgroup is staged in LDS once (memory pipeline, padded 16 x 16 tiles), the
+// activation operand goes from memory to the MFMA register as in conv_lds_tile, and the K loop is unrolled: no barrier
+// and no staging inside it.  The products are added in conv_lds_tile's order.  The activated result is parked in LDS as
+// [pixel][channel] (zeros outside the pointwise layer's map: the depthwise layer's padding) and the depthwise window
+// runs on it like dw3x3_f32_tile_kernel (a lane = four channels of one column, a run of rows, the same order of operations).
+// The halo is computed again by the neighbouring workgroups: 256 / 196 = 1.31 x the pointwise work at stride 1,
+// 255 / 224 = 1.14 x at stride 2.
+template <int S>
+struct PwDwTile
+{
+    static constexpr int TOH = S == 1 ? 14 : 7, TOW = S == 1 ? 14 : 8;
+    static constexpr int PH = (TOH - 1) * S + 3, PW = (TOW - 1) * S + 3;
+    static constexpr int NPX = PH * PW;
+    static_assert(NPX <= 256, "pointwise pixels of a tile vs eight MFMA tiles");
+};
+
+struct PwDwGeom
+{
+    int Hd, Wd;          // depthwise output map
+    int dpt, dpl;        // depthwise padding, top and left
+    int tiles_x, tiles_y, n_wgs, per_xcd;
+};
+
+template <int S, int COT, int CIB>
+__global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArgs a, const StemDwArgs d, const PwDwGeom g)
+{
+    using TL = PwDwTile<S>;
+    constexpr int TOH = TL::TOH, TOW = TL::TOW, PW = TL::PW, NPX = TL::NPX;
+    constexpr int CG = 32 * COT;                             // channels of the workgroup
+    constexpr int MIDP = CG + 4;                             // floats per parked pixel: 16 bytes of padding spread the banks
+    constexpr int NFT = 2 * COT * CIB;                       // 16 x 16 filter tiles of the workgroup
+    // the filter slice is dead when the K loop ends and the parked tile is born after it: they share their LDS
+    constexpr int MID_FLOATS = 256 * MIDP, FILT_FLOATS = NFT * A_TILE_FLOATS;
+    __shared__ __align__(16) float lds[MID_FLOATS > FILT_FLOATS ? MID_FLOATS : FILT_FLOATS];
+    __shared__ __align__(16) float s_bias[CG];
+    float *const filt = lds, *const mid = lds;
+
+    const int bid = blockIdx.x;
+    const int lid = (bid % NUM_XCD) * g.per_xcd + bid / NUM_XCD;   // neighbouring tiles share an XCD's L2
+    if (lid >= g.n_wgs) return;                              // the whole workgroup leaves, before any barrier
+    const int cg = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, half = lane >> 5;
+    const int tiles = g.tiles_x * g.tiles_y;
+    const int n = lid / tiles, trem = lid - n * tiles;
+    const int ty = trem / g.tiles_x, tx = trem - ty * g.tiles_x;
+    const int py0 = ty * TOH * S - g.dpt, px0 = tx * TOW * S - g.dpl;   // pointwise pixel of patch position (0, 0)
+    const int HW = a.H * a.W, CoB = a.Co / CB;
+    const float nscale = act_scale(a.act, a.slope);
+
+    // ---- requests first: filter slice to LDS, biases, depthwise taps ------------------------------------------------
+    {
+        // the slice is 2 COT consecutive channel blocks of CIB tiles each: contiguous in memory, tile after tile
+        const float *fsrc = a.filt + (size_t)cg * NFT * (CB * CB) + lane * 4;
+#pragma unroll
+        for (int t = wave; t < NFT; t += 4)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(fsrc + t * (CB * CB)),
+                                             (__attribute__((address_space(3))) void *)&filt[t * A_TILE_FLOATS], 16, 0, 0);
+    }
+    float my_bias = 0.f;
+    if (tid < CG && a.bias) my_bias = a.bias[cg * CG + tid];
+    // depthwise phase: lane = (channel quad q, column dx, row group rg)
+    constexpr int NQ = CG / 4, TCOLS = S == 1 ? 16 : 8, NRG = 256 / (NQ * TCOLS), RPG = (TOH + NRG - 1) / NRG;
+    const int q = tid % NQ, dslot = tid / NQ, dx = dslot % TCOLS, rg = dslot / TCOLS;
+    const int dcob = cg * (CG / CB) + q / 4, dq4 = (q & 3) * 4;   // channel block and first channel inside it
+    float4 w[9];
+    {
+        const float4 *wq = reinterpret_cast<const float4 *>(d.dw_filt + (size_t)dcob * (9 * CB) + dq4);
+#pragma unroll
+        for (int t = 0; t < 9; ++t) w[t] = wq[t * 4];
+    }
+    float4 dbias = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d.dw_bias) dbias = *reinterpret_cast<const float4 *>(d.dw_bias + dcob * CB + dq4);
+
+    // ---- pointwise layer on the patch --------------------------------------------------------------------------------
+    // this lane's two pixels: patch index p = (2 wave + t) * 32 + col -> position (p / PW, p % PW)
+    const float *in_px[2];
+    bool pin[2];                                             // inside the pointwise layer's map
+    int pidx[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+    {
+        const int pp = (2 * wave + t) * 32 + col;
+        const int py = pp / PW, pxx = pp - py * PW;
+        const int oh = py0 + py, ow = px0 + pxx;
+        pin[t] = pp < NPX && (unsigned)oh < (unsigned)a.H && (unsigned)ow < (unsigned)a.W;
+        pidx[t] = pp;
+        in_px[t] = pin[t] ? a.in + ((size_t)n * CIB * HW + oh * a.W + ow) * CB + half * 8 : g_zero_block + half * 8;
+    }
+    const int in_blk32 = HW * CB;
+    float4 B[2][2][2];                                       // [buffer][pixel tile][half of the eight channels]
+    auto fetch = [&](const int buf, const int cib) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+        {
+            const float4 *p4 = reinterpret_cast<const float4 *>(in_px[t] + (pin[t] ? cib * in_blk32 : 0));
+            B[buf][t][0] = p4[0];
+            B[buf][t][1] = p4[1];
+        }
+    };
+    fetch(0, 0);
+    if (CIB > 1) fetch(1, 1);
+    if (tid < CG) s_bias[tid] = my_bias;
+    __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0): the filter tiles have landed
+    __syncthreads();
+
+    int a_rd[COT];
+#pragma unroll
+    for (int c = 0; c < COT; ++c) a_rd[c] = (c * 2 + (col >> 4)) * CIB * A_TILE_FLOATS + half * 8 * CB + (col & 15);
+    floatx16 acc[COT][2];
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[c][t][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < CIB; ++s)
+    {
+        float A[COT][8];
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) A[c][kk] = filt[a_rd[c] + s * A_TILE_FLOATS + kk * CB];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+            {
+                const float4 bv = B[s & 1][t][kk >> 2];
+                const float b = (kk & 3) == 0 ? bv.x : (kk & 3) == 1 ? bv.y : (kk & 3) == 2 ? bv.z : bv.w;
+#pragma unroll
+                for (int c = 0; c < COT; ++c)
+                    acc[c][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(A[c][kk], b, acc[c][t], 0, 0, 0);
+            }
+        if (s + 2 < CIB) fetch(s & 1, s + 2);
+    }
+
+    __syncthreads();                                         // every wave has read its last filter operand
+    // ---- bias, activation, park in LDS: a lane holds channels c*32 + 8 qq + 4 half + 0..3 of its pixel -------------
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int c = 0; c < COT; ++c)
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq)
+            {
+                const int ch = c * 32 + 8 * qq + 4 * half;
+                const float4 bb = *reinterpret_cast<const float4 *>(&s_bias[ch]);
+                float4 v = make_float4(act_bf(acc[c][t][4 * qq + 0] + bb.x, nscale), act_bf(acc[c][t][4 * qq + 1] + bb.y, nscale),
+                                       act_bf(acc[c][t][4 * qq + 2] + bb.z, nscale), act_bf(acc[c][t][4 * qq + 3] + bb.w, nscale));
+                if (!pin[t]) v = make_float4(0.f, 0.f, 0.f, 0.f);      // outside the map: the depthwise layer's padding
+                *reinterpret_cast<float4 *>(&mid[pidx[t] * MIDP + ch]) = v;
+            }
+    __syncthreads();
+
+    // ---- depthwise 3x3 on the parked patch ---------------------------------------------------------------------------
+    const int dwo = tx * TOW + dx;                           // depthwise output column
+    const bool dcol_ok = dx < TOW && dwo < g.Wd;
+    const int dxc = dx < TOW ? dx : 0;                       // idle columns read in bounds
+    const float *xs = mid + (dxc * S) * MIDP + q * 4;        // window column 0 of this lane, patch row 0
+    float4 *dst = reinterpret_cast<float4 *>(a.out + (((size_t)n * CoB + dcob) * g.Hd * g.Wd + dwo) * CB + dq4);
+    auto at = [&](const int row, const int c) { return *reinterpret_cast<const float4 *>(xs + (row * PW + c) * MIDP); };
+    const int r0 = rg * RPG;                                 // first output row of this lane inside the tile
+    float4 win[3][3];
+    if (S == 1)
+    {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[r][c] = at(r0 + r, c);
+    }
+#pragma unroll
+    for (int o = 0; o < RPG; ++o)
+    {
+        const int lr = r0 + o;                               // output row inside the tile
+        const bool row_in = lr < TOH;
+        const int lrc = row_in ? lr : TOH - 1;               // rows past the tile read in bounds, nothing is stored
+        if (S == 1)
+        {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) win[(o + 2) % 3][c] = at(lrc + 2, c);
+        }
+        else
+        {
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int c = 0; c < 3; ++c) win[(o + r) % 3][c] = at(lrc * S + r, c);
+        }
+        const int oh = ty * TOH + lr;
+        const bool ok = dcol_ok && row_in && oh < g.Hd;
+        float4 acc2 = dbias;
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+            {
+                const float4 x = win[(o + r) % 3][c];
+                const float4 k = w[r * 3 + c];
+                acc2.x = fmaf(x.x, k.x, acc2.x); acc2.y = fmaf(x.y, k.y, acc2.y);
+                acc2.z = fmaf(x.z, k.z, acc2.z); acc2.w = fmaf(x.w, k.w, acc2.w);
+            }
+        acc2.x = act_bf(acc2.x, nscale); acc2.y = act_bf(acc2.y, nscale);
+        acc2.z = act_bf(acc2.z, nscale); acc2.w = act_bf(acc2.w, nscale);
+        if (ok) dst[(size_t)oh * g.Wd * 4] = acc2;
+    }
+}
+
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
@@ -1714,6 +1930,53 @@ int stem_dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, i
     return SMALL_HIP_OK;
 }
 
+// Pointwise convolution + depthwise 3x3 in one launch (conv_pw_dw3x3_f32_kernel).
+int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dpl, int dpr, int Co, int Ci, int H, int W,
+              const float *in, const float *filt, const float *bias, const float *dw_filt, const float *dw_bias, int act,
+              float slope, float *out, small_hip_stream_t stream)
+{
+    if (dw_stride != 1 && dw_stride != 2) return SMALL_HIP_ESTRIDE;
+    const int cib = Ci / CB;
+    if (Ci % CB != 0 || !(cib == 2 || cib == 4 || cib == 8) || Co % 32 != 0)
+    { set_error("%s: the pointwise form is built for 32, 64 or 128 input channels and output channels in whole groups of 32", op); return SMALL_HIP_EINVAL; }
+    if (batch <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(dpt, dpb, dpl, dpr)) { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
+    if (!in || !filt || !dw_filt || !out || !aligned16(in) || !aligned16(filt) || !aligned16(dw_filt) || !aligned16(out) ||
+        (bias && !aligned16(bias)) || (dw_bias && !aligned16(dw_bias)))
+    { set_error("%s: null or misaligned pointer", op); return SMALL_HIP_EINVAL; }
+    if (in == out) { set_error("%s: in-place operation is not supported", op); return SMALL_HIP_EINVAL; }
+    if (act < SMALL_HIP_ACT_NONE || act > SMALL_HIP_ACT_LEAKY) { set_error("%s: bad activation", op); return SMALL_HIP_EINVAL; }
+    ConvArgs a{};
+    a.in = in; a.filt = filt; a.bias = bias; a.out = out;
+    a.batch = batch; a.Co = Co; a.Ci = Ci; a.H = H; a.W = W; a.Ho = H; a.Wo = W;
+    a.kh = 1; a.kw = 1; a.stride = 1; a.stride_h = 1;
+    a.act = act; a.slope = slope;
+    PwDwGeom g{};
+    g.Hd = out_dim(H, dpt, dpb, 3, dw_stride);
+    g.Wd = out_dim(W, dpl, dpr, 3, dw_stride);
+    g.dpt = dpt; g.dpl = dpl;
+    if (g.Hd <= 0 || g.Wd <= 0) return SMALL_HIP_OK;
+    if ((long)Ci * H * W > 0x7fffffffL / 2) { set_error("%s: one image too large for 32-bit offsets", op); return SMALL_HIP_EINVAL; }
+    const int toh = dw_stride == 1 ? PwDwTile<1>::TOH : PwDwTile<2>::TOH, tow = dw_stride == 1 ? PwDwTile<1>::TOW : PwDwTile<2>::TOW;
+    g.tiles_x = (g.Wd + tow - 1) / tow; g.tiles_y = (g.Hd + toh - 1) / toh;
+    const long nt = (long)batch * g.tiles_x * g.tiles_y;
+    if (nt > 0x7fffffffL / 2) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
+    g.n_wgs = (int)nt; g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
+    const StemDwArgs d{dw_filt, dw_bias};
+    // channels per workgroup: 64 (the activation operand is loaded once per 64 output channels) up to 64 input channels,
+    // 32 beyond.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
+    int cot = (cib <= 4 && Co % 64 == 0) ? 2 : 1;
+    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && cib <= 4 && Co % 64 == 0)) cot = v; }
+    const dim3 grid(g.per_xcd * NUM_XCD, Co / (32 * cot));
+    void (*k)(const ConvArgs, const StemDwArgs, const PwDwGeom) = nullptr;
+#define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : conv_pw_dw3x3_f32_kernel<S_, 2, 4>) \
+                             : (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4> : conv_pw_dw3x3_f32_kernel<S_, 1, 8>))
+    k = dw_stride == 1 ? SHP_PD(1) : SHP_PD(2);
+#undef SHP_PD
+    hipLaunchKernelGGL(k, grid, dim3(256), 0, as_stream(stream), a, d, g);
+    SHP_LAUNCH_CHECK(op);
+    return SMALL_HIP_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -1768,7 +2031,11 @@ int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kh, int kw, i
                                                     const float *bias, const float *dw_filt, const float *dw_bias, int act,
                                                     float slope, float *out, small_hip_stream_t stream)
 {
-    return stem_dw_f32("small_hip_conv2d_bias_act_dwconv2d_bias_act_f32", batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw,
+    const char *op = "small_hip_conv2d_bias_act_dwconv2d_bias_act_f32";
+    // a pointwise convolution of whole channel blocks in front of a 3x3 depthwise layer
+    if (Ci > 3 && kh == 1 && kw == 1 && stride == 1 && pt == 0 && pb == 0 && pl == 0 && pr == 0 && dw_kh == 3 && dw_kw == 3)
+        return pw_dw_f32(op, batch, dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
+    return stem_dw_f32(op, batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw,
                        dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
 }
 

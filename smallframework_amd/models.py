@@ -394,13 +394,13 @@ class HipExecutor:
                 self.plan.append((conv, pool, False))
                 i = j + 1
                 continue
-            if (fused and model.dtype == "f32" and op.kind == "conv" and op.C in (1, 2, 3) and (op.kh, op.kw) == (3, 3)
-                    and j < len(ops) and ops[j].kind == "dw" and ops[j].src == op.dst
-                    and (ops[j].kh, ops[j].kw, ops[j].stride) == (3, 3, 1) and ops[j].pads == (1, 1, 1, 1)
+            if (fused and model.dtype == "f32" and op.kind == "conv" and j < len(ops) and ops[j].kind == "dw"
+                    and ops[j].src == op.dst and (ops[j].kh, ops[j].kw) == (3, 3)
                     and ops[j].act == op.act and ops[j].slope == op.slope
+                    and (self._first_layer_dw(op, ops[j]) or self._pointwise_dw_pays(op, ops[j]))
                     and not self._read_before_rewritten(ops[j + 1:], op.dst, model.out)):
-                # a first layer and the depthwise layer after it in one launch (the first layer's output is never
-                # written); as above, the result must not land on the convolution's input
+                # a first layer or a short pointwise convolution and the depthwise layer after it in one launch (the
+                # convolution's output is never written); as above, the result must not land on the convolution's input
                 conv, dw = at(op), at(ops[j])
                 if dw.dst == conv.src:
                     phys[ops[j].dst], phys[op.dst] = conv.dst, dw.dst
@@ -490,13 +490,40 @@ class HipExecutor:
             self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 2, 2, 2, 0, 0, 0, 0, op.Co, op.C, op.H, op.W,
             p(b[op.src]), p(self.w[op.weight]), None, act, op.slope, p(b[pool.dst]), st))
 
+    @staticmethod
+    def _first_layer_dw(op, dw):
+        """A first layer (1-3 input channels, 3x3 window) in front of a 3x3 stride-1 depthwise layer with one pixel of
+        padding: the pair small_hip_conv2d_bias_act_dwconv2d_bias_act_f32 runs on 16 x 16 first-layer tiles."""
+        return (op.C in (1, 2, 3) and (op.kh, op.kw) == (3, 3) and dw.stride == 1 and dw.pads == (1, 1, 1, 1))
+
+    @staticmethod
+    def _pointwise_dw_pays(op, dw):
+        """A pointwise convolution in front of a 3x3 depthwise layer, where one launch is faster than two (measured on
+        MobileNetV1's pairs at batch 64: 32 -> 64 @112x112 stride 2 104 -> 56 us, 64 -> 128 @56x56 70 -> 60 us,
+        128 -> 256 @28x28 53 -> 47 us; 128 -> 128 @56x56 stride 2 81 -> 85 us: not fused): up to 64 input channels, or
+        128 in front of a stride-1 depthwise layer, and depthwise tiles (14 x 14 at stride 1, 7 x 8 at stride 2) that
+        the output map fills to 70% at least."""
+        if not ((op.kh, op.kw, op.stride) == (1, 1, 1) and op.pads == (0, 0, 0, 0) and op.C % CB == 0 and op.Co % 32 == 0):
+            return False
+        cib = op.C // CB
+        if not (cib in (2, 4) or (cib == 8 and dw.stride == 1)) or dw.stride not in (1, 2):
+            return False
+        toh, tow = (14, 14) if dw.stride == 1 else (7, 8)
+        hd = capi.out_dim(op.H, dw.pads[0], dw.pads[1], 3, dw.stride)
+        wd = capi.out_dim(op.W, dw.pads[2], dw.pads[3], 3, dw.stride)
+        if hd <= 0 or wd <= 0:
+            return False
+        fill = hd * wd / float(-(-hd // toh) * toh * -(-wd // tow) * tow)
+        return fill >= 0.7
+
     def run_conv_dw_f32(self, op, dw, st):
-        """First-layer Conv2D + activation + DepthwiseConv2D 3x3 stride 1 + activation in one launch."""
+        """Conv2D + activation + DepthwiseConv2D 3x3 + activation in one launch."""
         L, p, b = self.lib, self._p, self.buf
         act = {None: capi.ACT_NONE, "relu": capi.ACT_RELU, "leaky": capi.ACT_LEAKY}[op.act]
         t_, b_, l_, r_ = op.pads
+        dt, db, dl, dr = dw.pads
         capi.check(L.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(
-            self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 3, 3, 1, 1, 1, 1, 1, op.Co, op.C, op.H, op.W,
+            self.batch, op.kh, op.kw, op.stride, t_, b_, l_, r_, 3, 3, dw.stride, dt, db, dl, dr, op.Co, op.C, op.H, op.W,
             p(b[op.src]), p(self.w[op.weight]), None, p(self.w[dw.weight]), None, act, op.slope, p(b[dw.dst]), st))
 
     def run_op(self, op: Op, st):

@@ -26,6 +26,8 @@ TWO_LAYER_CASES = [
     (3, 1, (1, 1, 1, 1), 2, 2, (0, 0, 0, 0), 16, 3, 32, 32),       # first layer, whole 16 x 16 tiles
     (3, 2, (0, 1, 0, 1), 3, 1, (1, 1, 1, 1), 32, 3, 30, 30),       # first layer + 3x3 depthwise (one launch on the GPU), MobileNetV1's pairing
     (3, 1, (1, 1, 1, 1), 3, 1, (1, 1, 1, 1), 16, 3, 20, 17),       # the same at stride 1, ragged 14 x 14 tiles
+    (1, 1, (0, 0, 0, 0), 3, 2, (0, 1, 0, 1), 64, 32, 28, 24),      # pointwise + 3x3 depthwise stride 2 (one launch on the GPU)
+    (1, 1, (0, 0, 0, 0), 3, 1, (1, 1, 1, 1), 64, 64, 14, 14),      # the same at stride 1, 64 input channels
 ]
 
 
