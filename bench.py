@@ -30,7 +30,7 @@ PEAK_MFMA_I8 = 5.0e15      # OP/s, dense int8 MFMA
 # WRITE_SIZE (two runs) over this same benchmark and scaled by what the counters read for an
 # in-place ReLU of 822 MB (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); the summary is
 # profiles/mobilenet_v1_b64_traffic_and_mfma.md.  Keyed by (model, batch, kernel family).
-MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_*"): 93.7}
+MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_*"): 70.0}
 
 
 def log(*a):
