@@ -1962,13 +1962,13 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     if (nt > 0x7fffffffL / 2) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
     g.n_wgs = (int)nt; g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
     const StemDwArgs d{dw_filt, dw_bias};
-    // channels per workgroup: 64 (the activation operand is loaded once per 64 output channels) up to 64 input channels,
-    // 32 beyond.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
-    int cot = (cib <= 4 && Co % 64 == 0) ? 2 : 1;
-    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && cib <= 4 && Co % 64 == 0)) cot = v; }
+    // channels per workgroup: 32 (four workgroups per compute unit) is measured ahead of 64 (two; the activation operand is
+    // loaded once per 64 output channels) on every MobileNetV1 pair at batch 64, by 1-3 us.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
+    int cot = 1;
+    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && Co % 64 == 0)) cot = v; }
     const dim3 grid(g.per_xcd * NUM_XCD, Co / (32 * cot));
     void (*k)(const ConvArgs, const StemDwArgs, const PwDwGeom) = nullptr;
-#define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : conv_pw_dw3x3_f32_kernel<S_, 2, 4>) \
+#define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 2, 4> : conv_pw_dw3x3_f32_kernel<S_, 2, 8>) \
                              : (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4> : conv_pw_dw3x3_f32_kernel<S_, 1, 8>))
     k = dw_stride == 1 ? SHP_PD(1) : SHP_PD(2);
 #undef SHP_PD
