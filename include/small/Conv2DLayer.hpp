@@ -366,6 +366,45 @@ public:
             throw std::invalid_argument("Conv2DLayer::compute_output_pooled() ERROR: float32 only.");
     }
 
+    // This layer and the depthwise layer after it as one launch (the reference's Conv2D_ReLU_DepthwiseConv2D_ReLU pairing,
+    // fused_interface_abstract.hpp:1840): true for the pairs small::detail::conv_dw_one_launch names, when both layers have
+    // the same ReLU / LeakyReLU / no activation and this layer's channels are not padded.  DwLayerT: DepthwiseConv2DLayer.
+    template <class DwLayerT>
+    bool fusable_with_depthwise(DwLayerT const &dw) const
+    {
+        auto const &os = this->output_shape();
+        auto const &w = dw.window();
+        return std::is_same<BufferT, FloatBuffer>::value && m_activation_type != SOFTMAX && m_activation_type == dw.activation() &&
+               (m_activation_type != LEAKY || m_slope == dw.slope()) && m_effective_output_channels == os[CHANNEL] &&
+               detail::conv_dw_one_launch<BufferT>((int)m_window.kh, (int)m_window.kw, (int)m_window.stride, m_window.t, m_window.b,
+                                                   m_window.l, m_window.r, (int)w.kh, (int)w.kw, (int)w.stride, w.t, w.b, w.l, w.r,
+                                                   (int)os[CHANNEL], (int)m_input_shape[CHANNEL], (int)m_input_shape[HEIGHT],
+                                                   (int)m_input_shape[WIDTH]);
+    }
+
+    // `output` (not the input tensor) receives the depthwise layer's output; the caller checks fusable_with_depthwise() first
+    template <class DwLayerT>
+    void compute_output_depthwise(Tensor<BufferT> const *input, DwLayerT const &dw, Tensor<BufferT> *output) const
+    {
+        if constexpr (std::is_same<BufferT, FloatBuffer>::value)
+        {
+            this->check_single_input("Conv2DLayer", {input}, m_input_shape, output);
+            if (output->capacity() < compute_size(dw.output_shape()))
+                throw std::invalid_argument("Conv2DLayer::compute_output_depthwise() ERROR: insufficient output buffer space.");
+            auto const &os = this->output_shape();
+            auto const &w = dw.window();
+            batched::Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
+                (int)m_input_shape[BATCH], m_window.kh, m_window.kw, m_window.stride, m_window.t, m_window.b, m_window.l,
+                m_window.r, w.kh, w.kw, w.stride, w.t, w.b, w.l, w.r, (int)os[CHANNEL], (int)m_input_shape[CHANNEL],
+                (int)m_input_shape[HEIGHT], (int)m_input_shape[WIDTH], input->buffer(), m_packed_filters, m_packed_bias,
+                output->buffer() /* not touched: the pair runs as one launch */, dw.get_packed_filters(), dw.get_packed_bias(),
+                m_activation_type, m_slope, output->buffer());
+            output->set_shape(dw.output_shape());
+        }
+        else
+            throw std::invalid_argument("Conv2DLayer::compute_output_depthwise() ERROR: float32 only.");
+    }
+
 private:
     shape_type const m_input_shape;
     detail::Window const m_window;

@@ -3,7 +3,8 @@
 // run in topological order, each output lives in a pooled tensor until its last consumer has run, and a layer
 // that accumulates (AddLayer, PartialConv2DLayer) writes into the tensor of its FIRST parent, which must have
 // no other consumer.  With save_outputs every layer's output stays readable until the next inference().
-// A float32 convolution whose only consumer is a max-pooling layer runs together with it (not with save_outputs).
+// A float32 convolution whose only consumer is a max-pooling layer runs together with it, and so does one whose only
+// consumer is a depthwise layer that it can take into its launch (neither with save_outputs).
 #pragma once
 
 #include <deque>
@@ -12,6 +13,7 @@
 
 #include "AddLayer.hpp"
 #include "Conv2DLayer.hpp"
+#include "DepthwiseConv2DLayer.hpp"
 #include "MaxPool2DLayer.hpp"
 #include "Model.hpp"
 #include "PartialConv2DLayer.hpp"
@@ -97,6 +99,30 @@ public:
                 ++step;                  // the pooling layer has run
                 continue;
             }
+            if (!m_save_outputs && m_dw_after[cur] != NO_POOL && step + 1 < m_order.size() && m_order[step + 1] == m_dw_after[cur])
+            {
+                // convolution whose only consumer is a depthwise layer it can run in its own launch: one call, the
+                // convolution's output is never written or cached
+                const size_t dl = m_dw_after[cur];
+                auto *conv = static_cast<Conv2DLayer<BufferT> *>(this->m_layers[cur]);
+                auto *dw = static_cast<DepthwiseConv2DLayer<BufferT> *>(this->m_layers[dl]);
+                try
+                {
+                    conv->compute_output_depthwise(ins[0], *dw, out);
+                }
+                catch (...)
+                {
+                    m_pool.push_buffer(out);
+                    throw;
+                }
+                if (step != 0)
+                    for (size_t k = 0; k < parents.size(); ++k)
+                        if (m_count[parents[k]] > 0 && --m_count[parents[k]] == 0) release(parents[k]);
+                m_count[dl] = m_graph.out_neighbors(dl).size();
+                m_cached[dl] = out;
+                ++step;                  // the depthwise layer has run
+                continue;
+            }
             try
             {
                 this->m_layers[cur]->compute_output(ins, out);
@@ -158,6 +184,16 @@ protected:
             if (dynamic_cast<MaxPool2DLayer<BufferT> *>(this->m_layers[outs[0]]) && m_graph.in_neighbors(outs[0]).size() == 1)
                 m_pool_after[i] = outs[0];
         }
+        // convolution -> depthwise pairs that run as one launch (Conv2DLayer::fusable_with_depthwise), same conditions
+        m_dw_after.assign(this->m_layers.size(), NO_POOL);
+        for (size_t i = 0; i < this->m_layers.size(); ++i)
+        {
+            auto *conv = dynamic_cast<Conv2DLayer<BufferT> *>(this->m_layers[i]);
+            auto const &outs = m_graph.out_neighbors(i);
+            if (!conv || outs.size() != 1 || m_graph.in_neighbors(outs[0]).size() != 1) continue;
+            auto *dw = dynamic_cast<DepthwiseConv2DLayer<BufferT> *>(this->m_layers[outs[0]]);
+            if (dw && conv->fusable_with_depthwise(*dw)) m_dw_after[i] = outs[0];
+        }
     }
 
     // Takes over a finished layer list as the graph's vertices 0..n-1 and initialises the DAG.  parents[i] lists
@@ -199,6 +235,7 @@ private:
 
     bool m_save_outputs;
     std::vector<size_t> m_pool_after;          // per layer: the max-pooling layer fused behind it, or NO_POOL
+    std::vector<size_t> m_dw_after;            // per layer: the depthwise layer that runs in its launch, or NO_POOL
     std::deque<size_t> m_order;
     BufferPool<BufferT> m_pool;
     std::vector<size_t> m_count;

@@ -82,6 +82,9 @@ public:
 
     BufferT const &get_packed_filters() const { return m_packed_filters; }
     BufferT const &get_packed_bias() const { return m_packed_bias; }
+    detail::Window const &window() const { return m_window; }
+    ActivationType activation() const { return m_activation_type; }
+    float slope() const { return m_slope; }
 
 
     virtual bool one_launch(small_hip_flayer &d) const

@@ -88,6 +88,41 @@ inline bool pool_fusion_enabled()
     }();
     return on;
 }
+
+// Does Conv2D_*_DepthwiseConv2D_* run this pair as one launch?  (a) a first layer (1-3 input channels, 3x3 window) in front of
+// a 3x3 stride-1 depthwise layer with one pixel of padding; (b) a pointwise convolution of 32 or 64 input channels in front
+// of a 3x3 depthwise layer whose output fills its 14 x 14 (stride 1) or 7 x 8 (stride 2) tiles to 70%: the pairs where one
+// launch is measured faster than two AND gives the two launches' result bit for bit (the reference's model tests compare
+// a model class with its layer functions for equality).  SMALL_HIP_FUSE_CONV_DW=0 switches it off; =2 adds 128 input
+// channels in front of a stride-1 depthwise layer, also faster, where the stand-alone convolution may add its products in
+// another order (float32 rounding).
+template <class BufferT>
+inline bool conv_dw_one_launch(int conv_kernel_height, int conv_kernel_width, int conv_stride, int conv_t_pad, int conv_b_pad,
+                               int conv_l_pad, int conv_r_pad, int dw_kernel_height, int dw_kernel_width, int dw_stride,
+                               int dw_t_pad, int dw_b_pad, int dw_l_pad, int dw_r_pad, int output_channels, int input_channels,
+                               int input_height, int input_width)
+{
+    if (!std::is_same<typename BufferT::value_type, float>::value) return false;
+    static const int fuse = [] { const char *e = std::getenv("SMALL_HIP_FUSE_CONV_DW"); return e ? e[0] - '0' : 1; }();
+    if (fuse <= 0 || dw_kernel_height != 3 || dw_kernel_width != 3) return false;
+    const bool first_layer = input_channels >= 1 && input_channels <= 3 && input_channels % (int)BufferT::C_ib != 0;
+    if (first_layer && conv_kernel_height == 3 && conv_kernel_width == 3 && (conv_stride == 1 || conv_stride == 2) && dw_stride == 1 &&
+        dw_t_pad == 1 && dw_b_pad == 1 && dw_l_pad == 1 && dw_r_pad == 1 && output_channels % (int)BufferT::C_ob == 0)
+        return true;
+    if (conv_kernel_height == 1 && conv_kernel_width == 1 && conv_stride == 1 && conv_t_pad == 0 && conv_b_pad == 0 &&
+        conv_l_pad == 0 && conv_r_pad == 0 && input_channels % 16 == 0 && output_channels % 32 == 0 && (dw_stride == 1 || dw_stride == 2))
+    {
+        const int cib = input_channels / 16;
+        if (cib == 2 || cib == 4 || (cib == 8 && dw_stride == 1 && fuse >= 2))
+        {
+            const int toh = dw_stride == 1 ? 14 : 7, tow = dw_stride == 1 ? 14 : 8;
+            if (input_height + dw_t_pad + dw_b_pad < 3 || input_width + dw_l_pad + dw_r_pad < 3) return false;
+            const int hd = 1 + (input_height + dw_t_pad + dw_b_pad - 3) / dw_stride, wd = 1 + (input_width + dw_l_pad + dw_r_pad - 3) / dw_stride;
+            return 10L * hd * wd >= 7L * ((hd + toh - 1) / toh * toh) * ((wd + tow - 1) / tow * tow);
+        }
+    }
+    return false;
+}
 } // namespace detail
 
 // =================================================================================================
@@ -346,12 +381,9 @@ void DepthwiseConv2D_Bias_Act(int batch, int kernel_height, int kernel_width, in
 
 // Conv2D [+ bias] [+ act] followed by DepthwiseConv2D [+ bias] [+ act] (the reference's Conv2D_*_DepthwiseConv2D_*
 // family, fused_interface_abstract.hpp:1513-2500).  ONE launch (small_hip_conv2d_bias_act_dwconv2d_bias_act_f32: the
-// convolution's output never goes to memory, inter_output_buf is not touched; SMALL_HIP_FUSE_CONV_DW=0 switches it off)
-// for (a) a first layer (1-3 input channels, 3x3 window) followed by a 3x3 stride-1 depthwise layer with one pixel of
-// padding, and (b) a pointwise convolution of 32 or 64 input channels (128 in front of a stride-1 depthwise layer)
-// followed by a 3x3 depthwise layer whose output fills its 14 x 14 (stride 1) or 7 x 8 (stride 2) tiles to 70%: the
-// pairs where one launch is measured faster than two.  Any other pair: two launches through inter_output_buf, which
-// ends up holding the whole first layer's output.  Bias buffers may be empty.
+// convolution's output never goes to memory, inter_output_buf is not touched) for the pairs detail::conv_dw_one_launch
+// names.  Any other pair: two launches through inter_output_buf, which ends up holding the whole first layer's output.
+// Bias buffers may be empty.
 template <class BufferT, detail::if_float<BufferT> = true>
 void Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
     int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride, uint8_t conv_t_pad, uint8_t conv_b_pad,
@@ -361,25 +393,9 @@ void Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
     BufferT &inter_output_buf, BufferT const &dwise_filter_buf, BufferT const &dwise_bias_buf, ActivationType act,
     float negative_slope, BufferT &output_buf)
 {
-    static const bool fuse_on = [] { const char *e = std::getenv("SMALL_HIP_FUSE_CONV_DW"); return !(e && e[0] == '0'); }();
-    const bool first_layer = input_channels >= 1 && input_channels <= 3 && input_channels % (int)BufferT::C_ib != 0;
-    const bool stem_pair = first_layer && conv_kernel_height == 3 && conv_kernel_width == 3 && (conv_stride == 1 || conv_stride == 2) &&
-                           dw_stride == 1 && dw_t_pad == 1 && dw_b_pad == 1 && dw_l_pad == 1 && dw_r_pad == 1 &&
-                           output_channels % (int)BufferT::C_ob == 0;
-    bool pointwise_pair = false;
-    if (conv_kernel_height == 1 && conv_kernel_width == 1 && conv_stride == 1 && conv_t_pad == 0 && conv_b_pad == 0 &&
-        conv_l_pad == 0 && conv_r_pad == 0 && input_channels % 16 == 0 && output_channels % 32 == 0 && (dw_stride == 1 || dw_stride == 2))
-    {
-        const int cib = input_channels / 16;
-        if (cib == 2 || cib == 4 || (cib == 8 && dw_stride == 1))
-        {
-            const int toh = dw_stride == 1 ? 14 : 7, tow = dw_stride == 1 ? 14 : 8;
-            const int hd = 1 + (input_height + dw_t_pad + dw_b_pad - 3) / dw_stride, wd = 1 + (input_width + dw_l_pad + dw_r_pad - 3) / dw_stride;
-            if (input_height + dw_t_pad + dw_b_pad >= 3 && input_width + dw_l_pad + dw_r_pad >= 3)
-                pointwise_pair = 10L * hd * wd >= 7L * ((hd + toh - 1) / toh * toh) * ((wd + tow - 1) / tow * tow);
-        }
-    }
-    if (fuse_on && (stem_pair || pointwise_pair) && dw_kernel_height == 3 && dw_kernel_width == 3)
+    if (detail::conv_dw_one_launch<BufferT>(conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
+                                            conv_r_pad, dw_kernel_height, dw_kernel_width, dw_stride, dw_t_pad, dw_b_pad, dw_l_pad,
+                                            dw_r_pad, output_channels, input_channels, input_height, input_width))
     {
         detail::raise<BufferT>(
             small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(

@@ -58,23 +58,37 @@ public:
         prev = this->add(new Conv2DLayer<BufferT>(prev->output_shape(), 1, 1, 1, PADDING_V, num_classes,
                                                   *filters[f++], filters_are_packed));
         cap0 = std::max(cap0, prev->output_size());
+        // a fused convolution + depthwise step shifts which of the two tensors a layer writes: one size for both
+        cap0 = std::max(cap0, cap1);
         m_buffer_0.reset(new Tensor<BufferT>(cap0));
-        m_buffer_1.reset(new Tensor<BufferT>(cap1));
+        m_buffer_1.reset(new Tensor<BufferT>(cap0));
     }
 
     virtual ~MobileNetTiny() {}
 
     virtual std::vector<Tensor<BufferT> *> inference(Tensor<BufferT> const *input_tensor)
     {
-        Tensor<BufferT> *a = m_buffer_0.get(), *b = m_buffer_1.get();
-        size_t l = 0;
-        this->m_layers[l++]->compute_output({input_tensor}, a);
-        while (l < this->m_layers.size())
+        // every step reads the tensor the previous step wrote and writes the other one; a convolution and the depthwise
+        // layer after it are one step (one launch) where that is faster than two (Conv2DLayer::fusable_with_depthwise)
+        Tensor<BufferT> *bufs[2] = {m_buffer_0.get(), m_buffer_1.get()};
+        Tensor<BufferT> const *cur = input_tensor;
+        int w = 0;
+        const size_t n = this->m_layers.size();
+        for (size_t l = 0; l < n; w ^= 1)
         {
-            this->m_layers[l++]->compute_output({a}, b);   // depthwise / pooling
-            this->m_layers[l++]->compute_output({b}, a);   // pointwise / classifier
+            Tensor<BufferT> *out = bufs[w];
+            auto *conv = dynamic_cast<Conv2DLayer<BufferT> *>(this->m_layers[l]);
+            auto *dw = l + 1 < n ? dynamic_cast<DepthwiseConv2DLayer<BufferT> *>(this->m_layers[l + 1]) : nullptr;
+            if (conv && dw && conv->fusable_with_depthwise(*dw))
+            {
+                conv->compute_output_depthwise(cur, *dw, out);
+                l += 2;
+            }
+            else
+                this->m_layers[l++]->compute_output({cur}, out);
+            cur = out;
         }
-        return {a};
+        return {bufs[w ^ 1]};
     }
 
 private:
