@@ -90,10 +90,10 @@ inline bool pool_fusion_enabled()
 }
 
 // Does Conv2D_*_DepthwiseConv2D_* run this pair as one launch?  (a) a first layer (1-3 input channels, 3x3 window) in front of
-// a 3x3 stride-1 depthwise layer with one pixel of padding; (b) a pointwise convolution of 32 or 64 input channels in front
+// a 3x3 stride-1 depthwise layer with one pixel of padding; (b) a pointwise convolution of 16 to 64 input channels in front
 // of a 3x3 depthwise layer whose output fills its 14 x 14 (stride 1) or 7 x 8 (stride 2) tiles to 70%: the pairs where one
 // launch is measured faster than two AND gives the two launches' result bit for bit (the reference's model tests compare
-// a model class with its layer functions for equality).  SMALL_HIP_FUSE_CONV_DW=0 switches it off; =2 adds 128 input
+// a model class with its layer functions for equality).  SMALL_HIP_FUSE_CONV_DW=0 switches it off; =2 adds 96 and 128 input
 // channels in front of a stride-1 depthwise layer, also faster, where the stand-alone convolution may add its products in
 // another order (float32 rounding).
 template <class BufferT>
@@ -113,7 +113,7 @@ inline bool conv_dw_one_launch(int conv_kernel_height, int conv_kernel_width, in
         conv_l_pad == 0 && conv_r_pad == 0 && input_channels % 16 == 0 && output_channels % 32 == 0 && (dw_stride == 1 || dw_stride == 2))
     {
         const int cib = input_channels / 16;
-        if (cib == 2 || cib == 4 || (cib == 8 && dw_stride == 1 && fuse >= 2))
+        if ((cib >= 1 && cib <= 4) || ((cib == 6 || cib == 8) && dw_stride == 1 && fuse >= 2))
         {
             const int toh = dw_stride == 1 ? 14 : 7, tow = dw_stride == 1 ? 14 : 8;
             if (input_height + dw_t_pad + dw_b_pad < 3 || input_width + dw_l_pad + dw_r_pad < 3) return false;

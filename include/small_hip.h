@@ -130,12 +130,12 @@ int small_hip_conv2d_bias_act_maxpool2d_f32(int batch, int kernel_height, int ke
  * Fused here (EINVAL otherwise: issue the two layers) for
  *  - a first layer: 1-3 input channels, a 3x3 convolution of stride 1 or 2, and a 3x3 stride-1 depthwise convolution
  *    with one pixel of padding on every side;
- *  - a pointwise convolution (1x1 window, stride 1, no padding) of 32, 64 or 128 input channels and output channels in
+ *  - a pointwise convolution (1x1 window, stride 1, no padding) of 16, 32, 48, 64, 96 or 128 input channels and output channels in
  *    whole groups of 32, and a 3x3 depthwise convolution of stride 1 or 2 with any padding (ESTRIDE for other strides).
  * The convolution's output never goes to memory; no intermediate buffer is needed.  dw_filter is [Co/16][3][3][16],
  * either bias may be null; one activation for both layers.  output is [batch][Co/16][Hd][Wd][16] with Hd, Wd the
  * depthwise layer's output size.  The result equals the two layers run one after the other bit for bit where the
- * stand-alone convolution adds its products in one pass (always but for 128 input channels, where it may split
+ * stand-alone convolution adds its products in one pass (always up to 112 input channels; from 128 on it may split
  * left-over tiles along the input channels: float32 rounding then). */
 int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,
                                                     int t_pad, int b_pad, int l_pad, int r_pad, int dw_kernel_height,

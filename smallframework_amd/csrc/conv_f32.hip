@@ -1334,7 +1334,7 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
     }
 }
 
-// Pointwise convolution (1x1 window, stride 1, no padding; 16 * CIB input channels) + bias + activation followed by a 3x3
+// Pointwise convolution (1x1 window, stride 1, no padding; 16 * CIB input channels, CIB <= 8) + bias + activation followed by a 3x3
 // depthwise convolution of stride S + bias + activation, in one launch: the reference's Conv2D_ReLU_DepthwiseConv2D_ReLU
 // pairing (fused_interface_abstract.hpp:1840) for the blocked layers, MobileNetV1's 1x1 -> 3x3 depthwise sequence.  The
 // pointwise layer's output, the largest tensor of such a pair, is neither written nor read.
@@ -1937,8 +1937,8 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
 {
     if (dw_stride != 1 && dw_stride != 2) return SMALL_HIP_ESTRIDE;
     const int cib = Ci / CB;
-    if (Ci % CB != 0 || !(cib == 2 || cib == 4 || cib == 8) || Co % 32 != 0)
-    { set_error("%s: the pointwise form is built for 32, 64 or 128 input channels and output channels in whole groups of 32", op); return SMALL_HIP_EINVAL; }
+    if (Ci % CB != 0 || !(cib == 1 || cib == 2 || cib == 3 || cib == 4 || cib == 6 || cib == 8) || Co % 32 != 0)
+    { set_error("%s: the pointwise form is built for 16, 32, 48, 64, 96 or 128 input channels and output channels in whole groups of 32", op); return SMALL_HIP_EINVAL; }
     if (batch <= 0 || H <= 0 || W <= 0 || Co <= 0 || !pads_ok(dpt, dpb, dpl, dpr)) { set_error("%s: bad size", op); return SMALL_HIP_EINVAL; }
     if (!in || !filt || !dw_filt || !out || !aligned16(in) || !aligned16(filt) || !aligned16(dw_filt) || !aligned16(out) ||
         (bias && !aligned16(bias)) || (dw_bias && !aligned16(dw_bias)))
@@ -1965,11 +1965,12 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     // channels per workgroup: 32 (four workgroups per compute unit) is measured ahead of 64 (two; the activation operand is
     // loaded once per 64 output channels) on every MobileNetV1 pair at batch 64, by 1-3 us.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
     int cot = 1;
-    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && Co % 64 == 0)) cot = v; }
+    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && Co % 64 == 0 && (cib == 2 || cib == 4 || cib == 8))) cot = v; }
     const dim3 grid(g.per_xcd * NUM_XCD, Co / (32 * cot));
     void (*k)(const ConvArgs, const StemDwArgs, const PwDwGeom) = nullptr;
 #define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 2, 4> : conv_pw_dw3x3_f32_kernel<S_, 2, 8>) \
-                             : (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4> : conv_pw_dw3x3_f32_kernel<S_, 1, 8>))
+                             : (cib == 1 ? conv_pw_dw3x3_f32_kernel<S_, 1, 1> : cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 3 ? conv_pw_dw3x3_f32_kernel<S_, 1, 3> \
+                                : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4> : cib == 6 ? conv_pw_dw3x3_f32_kernel<S_, 1, 6> : conv_pw_dw3x3_f32_kernel<S_, 1, 8>))
     k = dw_stride == 1 ? SHP_PD(1) : SHP_PD(2);
 #undef SHP_PD
     hipLaunchKernelGGL(k, grid, dim3(256), 0, as_stream(stream), a, d, g);

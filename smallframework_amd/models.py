@@ -501,12 +501,12 @@ class HipExecutor:
         """A pointwise convolution in front of a 3x3 depthwise layer, where one launch is faster than two (measured on
         MobileNetV1's pairs at batch 64: 32 -> 64 @112x112 stride 2 104 -> 56 us, 64 -> 128 @56x56 70 -> 60 us,
         128 -> 256 @28x28 53 -> 47 us; 128 -> 128 @56x56 stride 2 81 -> 85 us: not fused): up to 64 input channels, or
-        128 in front of a stride-1 depthwise layer, and depthwise tiles (14 x 14 at stride 1, 7 x 8 at stride 2) that
+        96 / 128 in front of a stride-1 depthwise layer (the kernel is built for 16, 32, 48, 64, 96 and 128 input channels), and depthwise tiles (14 x 14 at stride 1, 7 x 8 at stride 2) that
         the output map fills to 70% at least."""
         if not ((op.kh, op.kw, op.stride) == (1, 1, 1) and op.pads == (0, 0, 0, 0) and op.C % CB == 0 and op.Co % 32 == 0):
             return False
         cib = op.C // CB
-        if not (cib in (2, 4) or (cib == 8 and dw.stride == 1)) or dw.stride not in (1, 2):
+        if not (cib in (1, 2, 3, 4) or (cib in (6, 8) and dw.stride == 1)) or dw.stride not in (1, 2):
             return False
         toh, tow = (14, 14) if dw.stride == 1 else (7, 8)
         hd = capi.out_dim(op.H, dw.pads[0], dw.pads[1], 3, dw.stride)

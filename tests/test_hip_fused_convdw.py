@@ -106,6 +106,9 @@ PW_CASES = [
     (5, 1, (1, 1, 1, 1), 256, 128, 28, 28, False, False, capi.ACT_RELU),     # MobileNetV1's 128 -> 256 pair
     (4, 2, (0, 1, 0, 1), 64, 32, 112, 112, False, False, capi.ACT_RELU),     # MobileNetV1's 32 -> 64 pair, real size
     (1, 1, (1, 1, 1, 1), 64, 32, 3, 2, True, True, capi.ACT_RELU),           # smaller than a tile
+    (2, 2, (0, 1, 0, 1), 32, 16, 33, 20, True, True, capi.ACT_RELU),         # one K-step
+    (2, 1, (1, 1, 1, 1), 96, 48, 15, 18, True, False, capi.ACT_LEAKY),       # three K-steps
+    (1, 1, (1, 1, 1, 1), 64, 96, 20, 14, False, True, capi.ACT_RELU),        # six K-steps
 ]
 
 
@@ -165,7 +168,7 @@ def test_pointwise_dw_refusals(lib):
     call = lambda Ci=32, Co=64, ds=1, dk=3: lib.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(
         1, 1, 1, 1, 0, 0, 0, 0, dk, dk, ds, 1, 1, 1, 1, Co, Ci, 16, 16, p, p, None, p, None, capi.ACT_RELU, 0.0, hu.ptr(t[1 << 17:]), st)
     assert call() == capi.OK
-    assert call(Ci=48) == capi.EINVAL            # three K-steps: not built
+    assert call(Ci=80) == capi.EINVAL            # five K-steps: not built
     assert call(Ci=256) == capi.EINVAL
     assert call(Co=48) == capi.EINVAL
     assert call(ds=3) == capi.ESTRIDE
