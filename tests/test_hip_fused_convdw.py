@@ -173,3 +173,40 @@ def test_pointwise_dw_refusals(lib):
     assert call(Co=48) == capi.EINVAL
     assert call(ds=3) == capi.ESTRIDE
     assert call(dk=5) == capi.EINVAL             # falls to the first-layer form, which refuses 32 input channels
+
+
+def test_pointwise_dw_random_shapes(lib):
+    """Seeded random shapes, paddings and options: the one launch against this library's two launches, bit for bit (fewer
+    than eight K-steps, so the stand-alone convolution adds its products in the same order)."""
+    rng = np.random.default_rng(20240611)
+    for it in range(24):
+        batch = int(rng.integers(1, 4))
+        Ci = int(rng.choice([16, 32, 48, 64, 96]))
+        Co = int(rng.choice([32, 64, 96, 128]))
+        H, W = int(rng.integers(3, 41)), int(rng.integers(3, 41))
+        ds = int(rng.integers(1, 3))
+        dt, db_, dl, dr = (int(v) for v in rng.integers(0, 2, 4))
+        has_b, has_db = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        act = int(rng.choice([capi.ACT_NONE, capi.ACT_RELU, capi.ACT_LEAKY]))
+        Hd, Wd = (H + dt + db_ - 3) // ds + 1, (W + dl + dr - 3) // ds + 1
+        if H + dt + db_ < 3 or W + dl + dr < 3:
+            continue
+        what = "case %d: batch %d Ci %d Co %d %dx%d stride %d pads %s bias %s/%s act %d" % (
+            it, batch, Ci, Co, H, W, ds, (dt, db_, dl, dr), has_b, has_db, act)
+        print(what, flush=True)
+        dx = hu.dev(synth.normal(100 + it, batch * Ci * H * W))
+        df = hu.dev(synth.he_normal(200 + it, Co * Ci, Ci))
+        ddf = hu.dev(synth.he_normal(300 + it, Co * 9, 9))
+        db = hu.dev(synth.normal(400 + it, Co)) if has_b else None
+        ddb = hu.dev(synth.normal(500 + it, Co)) if has_db else None
+        do = hu.dev(np.full(batch * Co * Hd * Wd, 7.0, np.float32))
+        assert lib.small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(
+            batch, 1, 1, 1, 0, 0, 0, 0, 3, 3, ds, dt, db_, dl, dr, Co, Ci, H, W, hu.ptr(dx), hu.ptr(df), hu.ptr(db), hu.ptr(ddf),
+            hu.ptr(ddb), act, 0.1, hu.ptr(do), hu.stream()) == 0, lib.small_hip_last_error()
+        dmid = hu.dev_empty(batch * Co * H * W, np.float32)
+        d2 = hu.dev_empty(batch * Co * Hd * Wd, np.float32)
+        assert lib.small_hip_conv2d_bias_act_f32(batch, 1, 1, 1, 0, 0, 0, 0, Co, Ci, H, W, hu.ptr(dx), hu.ptr(df), hu.ptr(db), act, 0.1,
+                                                 hu.ptr(dmid), hu.stream()) == 0, lib.small_hip_last_error()
+        assert lib.small_hip_depthwise_conv2d_bias_act_f32(batch, 3, 3, ds, dt, db_, dl, dr, Co, H, W, hu.ptr(dmid), hu.ptr(ddf),
+                                                           hu.ptr(ddb), act, 0.1, hu.ptr(d2), hu.stream()) == 0, lib.small_hip_last_error()
+        assert_equal_exact(hu.host(do), hu.host(d2), what)
