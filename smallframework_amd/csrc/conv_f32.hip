@@ -1360,7 +1360,9 @@ struct PwDwGeom
 {
     int Hd, Wd;          // depthwise output map
     int dpt, dpl;        // depthwise padding, top and left
-    int tiles_x, tiles_y, n_wgs, per_xcd;
+    int tiles_x, tiles_y;
+    int n_cg;            // channel groups (32 COT channels each)
+    int n_wgs, per_xcd;  // workgroups = tiles x channel groups, and their share per XCD
 };
 
 template <int S, int COT, int CIB>
@@ -1377,15 +1379,17 @@ __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArg
     __shared__ __align__(16) float s_bias[CG];
     float *const filt = lds, *const mid = lds;
 
+    // logical id = (tile, channel group), the channel group fastest; consecutive logical ids run on one XCD: the channel
+    // groups of a tile find its input pixels in that XCD's L2, and so do neighbouring tiles their shared halo
     const int bid = blockIdx.x;
-    const int lid = (bid % NUM_XCD) * g.per_xcd + bid / NUM_XCD;   // neighbouring tiles share an XCD's L2
+    const int lid = (bid % NUM_XCD) * g.per_xcd + bid / NUM_XCD;
     if (lid >= g.n_wgs) return;                              // the whole workgroup leaves, before any barrier
-    const int cg = blockIdx.y;
+    const int cg = lid % g.n_cg, tile_id = lid / g.n_cg;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
     const int tiles = g.tiles_x * g.tiles_y;
-    const int n = lid / tiles, trem = lid - n * tiles;
+    const int n = tile_id / tiles, trem = tile_id - n * tiles;
     const int ty = trem / g.tiles_x, tx = trem - ty * g.tiles_x;
     const int py0 = ty * TOH * S - g.dpt, px0 = tx * TOW * S - g.dpl;   // pointwise pixel of patch position (0, 0)
     const int HW = a.H * a.W, CoB = a.Co / CB;
@@ -1959,14 +1963,15 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     const int toh = dw_stride == 1 ? PwDwTile<1>::TOH : PwDwTile<2>::TOH, tow = dw_stride == 1 ? PwDwTile<1>::TOW : PwDwTile<2>::TOW;
     g.tiles_x = (g.Wd + tow - 1) / tow; g.tiles_y = (g.Hd + toh - 1) / toh;
     const long nt = (long)batch * g.tiles_x * g.tiles_y;
-    if (nt > 0x7fffffffL / 2) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
-    g.n_wgs = (int)nt; g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
     const StemDwArgs d{dw_filt, dw_bias};
     // channels per workgroup: 32 (four workgroups per compute unit) is measured ahead of 64 (two; the activation operand is
     // loaded once per 64 output channels) on every MobileNetV1 pair at batch 64, by 1-3 us.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
     int cot = 1;
     if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && Co % 64 == 0 && (cib == 2 || cib == 4 || cib == 8))) cot = v; }
-    const dim3 grid(g.per_xcd * NUM_XCD, Co / (32 * cot));
+    g.n_cg = Co / (32 * cot);
+    if (nt * g.n_cg > 0x7fffffffL / 2) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
+    g.n_wgs = (int)(nt * g.n_cg); g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
+    const dim3 grid(g.per_xcd * NUM_XCD);
     void (*k)(const ConvArgs, const StemDwArgs, const PwDwGeom) = nullptr;
 #define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 2, 4> : conv_pw_dw3x3_f32_kernel<S_, 2, 8>) \
                              : (cib == 1 ? conv_pw_dw3x3_f32_kernel<S_, 1, 1> : cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 3 ? conv_pw_dw3x3_f32_kernel<S_, 1, 3> \
