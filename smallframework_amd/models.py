@@ -499,8 +499,8 @@ class HipExecutor:
     @staticmethod
     def _pointwise_dw_pays(op, dw):
         """A pointwise convolution in front of a 3x3 depthwise layer, where one launch is faster than two (measured on
-        MobileNetV1's pairs at batch 64: 32 -> 64 @112x112 stride 2 104 -> 56 us, 64 -> 128 @56x56 70 -> 60 us,
-        128 -> 256 @28x28 53 -> 47 us; 128 -> 128 @56x56 stride 2 81 -> 85 us: not fused): up to 64 input channels, or
+        MobileNetV1's pairs at batch 64: 32 -> 64 @112x112 stride 2 104 -> 54 us, 64 -> 128 @56x56 70 -> 54 us,
+        128 -> 256 @28x28 53 -> 46 us; 128 -> 128 @56x56 stride 2 81 -> 85 us: not fused): up to 64 input channels, or
         96 / 128 in front of a stride-1 depthwise layer (the kernel is built for 16, 32, 48, 64, 96 and 128 input channels), and depthwise tiles (14 x 14 at stride 1, 7 x 8 at stride 2) that
         the output map fills to 70% at least."""
         if not ((op.kh, op.kw, op.stride) == (1, 1, 1) and op.pads == (0, 0, 0, 0) and op.C % CB == 0 and op.Co % 32 == 0):
