@@ -9,7 +9,7 @@ line also carries ResNet-8 uint8 at batch 64 and 256, the per-layer roofline tab
 of the dominant kernel and the reference's CPU build timed on this host.
 
 Prints ONE compact JSON line on stdout (headline, roofline, cpu_baseline, a per-configuration summary);
-the per-layer tables go to gpurun_out/bench_<workload>_full.json, progress and readable tables to stderr.
+the per-layer tables go to bench_<workload>_full.json in the output folder (OUT_DIR), progress and readable tables to stderr.
 """
 import argparse
 import json
@@ -19,6 +19,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
+OUT_DIR = "gpurun_out"      # results that are too long for the one JSON line on stdout
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
@@ -66,10 +67,10 @@ def table_summary(entry, batch):
 
 
 def emit(out, tag):
-    """The full result (per-layer tables, extras) goes to gpurun_out/bench_<tag>_full.json and to stderr; stdout gets
+    """The full result (per-layer tables, extras) goes to bench_<tag>_full.json in OUT_DIR and to stderr; stdout gets
     ONE compact JSON line: the headline fields, roofline, cpu_baseline and a short per-configuration summary."""
     full = json.dumps(out)
-    path = os.path.join(ROOT, "gpurun_out", "bench_%s_full.json" % tag)
+    path = os.path.join(ROOT, OUT_DIR, "bench_%s_full.json" % tag)
     try:
         os.makedirs(os.path.dirname(path), exist_ok=True)
         with open(path, "w") as f:

@@ -51,7 +51,7 @@ STRICT_LOG = os.path.join(os.path.dirname(os.path.dirname(GOLDEN)), "gpurun_out"
 def strict_bar(got, truth, what, max_outside_frac, max_excess, reference=None):
     """The stated float32 bar without any scaling: against `truth` (the same computation with float64
     accumulation), count the elements outside |a - b| <= 1e-4 * |b| + 1e-5 and take the worst excess over that
-    bound.  Prints the figures, appends them to gpurun_out/strict_f32_bar.jsonl and asserts the given limits
+    bound.  Prints the figures, appends them to STRICT_LOG and asserts the given limits
     (a fraction of the elements, and an absolute excess).  `reference`: the float32 sequential-order oracle's result
     for the same inputs; its own count against the same truth is recorded beside the GPU's."""
     import json
