@@ -231,8 +231,9 @@ def layer_table(model, batch, ms):
         if op.kind == "conv" and i + 1 < len(ops) and ops[i + 1].kind in ("maxpool", "dw") and ms[i + 1] == 0.0:
             nbytes = batch * (op.act_elems()[0] + ops[i + 1].act_elems()[1]) * es + \
                 (op.weight_elems() + ops[i + 1].weight_elems()) * es
-            if kind == "hbm" or nbytes / PEAK_HBM > tb:
-                tb, kind = nbytes / PEAK_HBM, "hbm"
+            # the fused launch's own roofline: its bytes at the HBM peak, or the convolution's flops at the MFMA peak
+            t_mfma = batch * op.flops() / (PEAK_MFMA_F32 if model.dtype == "f32" else PEAK_MFMA_I8) if op.C % 16 == 0 else 0.0
+            tb, kind = (t_mfma, "mfma") if t_mfma > nbytes / PEAK_HBM else (nbytes / PEAK_HBM, "hbm")
         rows.append({"layer": op.name, "ms": round(t, 5), "bound": kind,
                      "roofline_frac": round(tb / (t * 1e-3), 4) if t > 0 else None,
                      "GB/s": round(nbytes / (t * 1e-3) / 1e9, 1) if t > 0 else None,
