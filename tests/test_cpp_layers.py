@@ -339,13 +339,14 @@ def test_resnet8_quantised_model(hip, oracle, one_launch):
 @pytest.mark.gpu
 def test_model_class_throughput(hip):
     """MobileNetTiny<FloatBuffer> built as MobileNetV1 (224x224, 1000 classes) at batch 64: one
-    Model::inference() call is the same 29 launches bench.py times through the C ABI, so it must land in the
-    same range (the bound below is loose: 2x the bench figure recorded for this build, ~1.05 ms)."""
+    Model::inference() call is the launches bench.py times through the C ABI (one more: the class keeps the
+    128-channel pointwise + depthwise pair as two launches), so it must land in the same range (the bound below is
+    loose: 2x the figure recorded for this build, ~0.9 ms)."""
     sizes = [int(np.prod(f.shape)) for f in ol.make_filters(synth, ol.mobilenet_specs(), 1000)]
     ms = hip.model_time_f32(0, 1, (64, 3, 224, 224), sizes)
     print("MobileNetTiny<FloatBuffer> (MobileNetV1 224x224, 1000 classes) batch 64: %.3f ms per inference, %.0f images/s"
           % (ms, 64 / ms * 1e3))
-    assert ms < 2.2
+    assert ms < 1.8
     # TinyYoloV2<FloatBuffer> as Tiny-YOLOv2 (416x416, LeakyReLU, 125 outputs) at batch 16: the class fuses its
     # convolution + pooling pairs like the benchmark's executor (recorded: ~1.2 ms)
     sizes = [int(np.prod(f.shape)) for f in ol.make_filters(synth, ol.yolo_specs(), 125)]
