@@ -376,7 +376,7 @@ public:
         auto const &w = dw.window();
         return std::is_same<BufferT, FloatBuffer>::value && m_activation_type != SOFTMAX && m_activation_type == dw.activation() &&
                (m_activation_type != LEAKY || m_slope == dw.slope()) && m_effective_output_channels == os[CHANNEL] &&
-               detail::conv_dw_one_launch<BufferT>((int)m_window.kh, (int)m_window.kw, (int)m_window.stride, m_window.t, m_window.b,
+               detail::conv_dw_one_launch<BufferT>((int)m_input_shape[BATCH], (int)m_window.kh, (int)m_window.kw, (int)m_window.stride, m_window.t, m_window.b,
                                                    m_window.l, m_window.r, (int)w.kh, (int)w.kw, (int)w.stride, w.t, w.b, w.l, w.r,
                                                    (int)os[CHANNEL], (int)m_input_shape[CHANNEL], (int)m_input_shape[HEIGHT],
                                                    (int)m_input_shape[WIDTH]);

@@ -182,14 +182,14 @@ protected:
     std::vector<Layer<BufferT> *> m_layers;
 
 private:
-    // QUInt8Buffer: on unless SMALL_HIP_ONE_LAUNCH=0 (the launch is bit-identical to the layer calls).  FloatBuffer: off
-    // unless SMALL_HIP_ONE_LAUNCH=1 or set_one_launch(true): its sums run in another order, and callers (the reference's
+    // QUInt8Buffer: on unless SMALL_HIP_TUNE="one_launch=0" (the launch is bit-identical to the layer calls).  FloatBuffer: off
+    // unless SMALL_HIP_TUNE="one_launch=1" or set_one_launch(true): its sums run in another order, and callers (the reference's
     // own model tests among them) compare a model's output with the layer functions' bit for bit.
     static bool one_launch_default()
     {
-        char const *e = std::getenv("SMALL_HIP_ONE_LAUNCH");
-        if (std::is_same<BufferT, QUInt8Buffer>::value) return !(e && e[0] == '0');
-        return e && e[0] == '1';
+        int const v = small_hip_tune_int("one_launch", -1);
+        if (std::is_same<BufferT, QUInt8Buffer>::value) return v != 0;
+        return v == 1;
     }
     bool m_one_launch = one_launch_default();
     small_hip_qmodel *m_qmodel = nullptr;

@@ -76,52 +76,38 @@ using if_quint8 = std::enable_if_t<std::is_same<QUInt8Buffer, BufferT>::value, b
 
 inline small_hip_stream_t st() { return current_stream(); }
 
-// SMALL_HIP_FUSE_POOL=0 makes every convolution + pooling pair run as its two launches.  The one-launch form sums
+// SMALL_HIP_TUNE="fuse_pool=0" makes every convolution + pooling pair run as its two launches.  The one-launch form sums
 // in another float32 order than the stand-alone convolution (another kernel), so a model class and the same layers
 // called one by one agree within the float32 tolerance by default and bit for bit with this switch off (the
 // reference's test_tinyyolov2.cpp asserts the latter of its two call paths).
 inline bool pool_fusion_enabled()
 {
-    static const bool on = [] {
-        const char *e = std::getenv("SMALL_HIP_FUSE_POOL");
-        return !(e && e[0] == '0');
-    }();
+    static const bool on = small_hip_tune_int("fuse_pool", 1) != 0;
     return on;
 }
 
-// Does Conv2D_*_DepthwiseConv2D_* run this pair as one launch?  (a) a first layer (1-3 input channels, 3x3 window) in front of
-// a 3x3 stride-1 depthwise layer with one pixel of padding; (b) a pointwise convolution of 16 to 64 input channels in front
-// of a 3x3 depthwise layer whose output fills its 14 x 14 (stride 1) or 7 x 8 (stride 2) tiles to 70%: the pairs where one
-// launch is measured faster than two AND gives the two launches' result bit for bit (the reference's model tests compare
-// a model class with its layer functions for equality).  SMALL_HIP_FUSE_CONV_DW=0 switches it off; =2 adds 96 and 128 input
-// channels in front of a stride-1 depthwise layer, also faster, where the stand-alone convolution may add its products in
-// another order (float32 rounding).
+// Does Conv2D_*_DepthwiseConv2D_* run this pair as one launch?  The library answers (small_hip_conv2d_dwconv2d_one_launch_f32:
+// first layers in front of a 3x3 stride-1 depthwise layer; pointwise convolutions of 16 to 64, 96 or 128 input channels in
+// front of a 3x3 depthwise layer whose output fills the one-launch kernel's tiles), and says whether the one launch equals
+// the two launches bit for bit.  By default only those pairs are fused: the reference's model tests compare a model class
+// with its layer functions for equality.  SMALL_HIP_TUNE="fuse_conv_dw=0" switches the fusion off; =2 adds the pairs
+// (96 / 128 input channels) that are faster as one launch but may differ from the two launches by float32 rounding.
 template <class BufferT>
-inline bool conv_dw_one_launch(int conv_kernel_height, int conv_kernel_width, int conv_stride, int conv_t_pad, int conv_b_pad,
+inline bool conv_dw_one_launch(int batch, int conv_kernel_height, int conv_kernel_width, int conv_stride, int conv_t_pad, int conv_b_pad,
                                int conv_l_pad, int conv_r_pad, int dw_kernel_height, int dw_kernel_width, int dw_stride,
                                int dw_t_pad, int dw_b_pad, int dw_l_pad, int dw_r_pad, int output_channels, int input_channels,
                                int input_height, int input_width)
 {
     if (!std::is_same<typename BufferT::value_type, float>::value) return false;
-    static const int fuse = [] { const char *e = std::getenv("SMALL_HIP_FUSE_CONV_DW"); return e ? e[0] - '0' : 1; }();
-    if (fuse <= 0 || dw_kernel_height != 3 || dw_kernel_width != 3) return false;
-    const bool first_layer = input_channels >= 1 && input_channels <= 3 && input_channels % (int)BufferT::C_ib != 0;
-    if (first_layer && conv_kernel_height == 3 && conv_kernel_width == 3 && (conv_stride == 1 || conv_stride == 2) && dw_stride == 1 &&
-        dw_t_pad == 1 && dw_b_pad == 1 && dw_l_pad == 1 && dw_r_pad == 1 && output_channels % (int)BufferT::C_ob == 0)
-        return true;
-    if (conv_kernel_height == 1 && conv_kernel_width == 1 && conv_stride == 1 && conv_t_pad == 0 && conv_b_pad == 0 &&
-        conv_l_pad == 0 && conv_r_pad == 0 && input_channels % 16 == 0 && output_channels % 32 == 0 && (dw_stride == 1 || dw_stride == 2))
-    {
-        const int cib = input_channels / 16;
-        if ((cib >= 1 && cib <= 4) || ((cib == 6 || cib == 8) && dw_stride == 1 && fuse >= 2))
-        {
-            const int toh = dw_stride == 1 ? 14 : 7, tow = dw_stride == 1 ? 14 : 8;
-            if (input_height + dw_t_pad + dw_b_pad < 3 || input_width + dw_l_pad + dw_r_pad < 3) return false;
-            const int hd = 1 + (input_height + dw_t_pad + dw_b_pad - 3) / dw_stride, wd = 1 + (input_width + dw_l_pad + dw_r_pad - 3) / dw_stride;
-            return 10L * hd * wd >= 7L * ((hd + toh - 1) / toh * toh) * ((wd + tow - 1) / tow * tow);
-        }
-    }
-    return false;
+    static const int fuse = small_hip_tune_int("fuse_conv_dw", 1);
+    if (fuse <= 0) return false;
+    const int form = small_hip_conv2d_dwconv2d_one_launch_f32(batch, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad,
+                                                              conv_b_pad, conv_l_pad, conv_r_pad, dw_kernel_height, dw_kernel_width,
+                                                              dw_stride, dw_t_pad, dw_b_pad, dw_l_pad, dw_r_pad, output_channels,
+                                                              input_channels, input_height, input_width);
+    // six K-steps (96 channels) are bit-identical too but were measured with the 128-channel pairs: same switch
+    const bool short_reduction = input_channels <= 64;
+    return form == 1 ? (short_reduction || fuse >= 2) : form == 2 && fuse >= 2;
 }
 } // namespace detail
 
@@ -393,7 +379,7 @@ void Conv2D_Bias_Act_DepthwiseConv2D_Bias_Act(
     BufferT &inter_output_buf, BufferT const &dwise_filter_buf, BufferT const &dwise_bias_buf, ActivationType act,
     float negative_slope, BufferT &output_buf)
 {
-    if (detail::conv_dw_one_launch<BufferT>(conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
+    if (detail::conv_dw_one_launch<BufferT>(batch, conv_kernel_height, conv_kernel_width, conv_stride, conv_t_pad, conv_b_pad, conv_l_pad,
                                             conv_r_pad, dw_kernel_height, dw_kernel_width, dw_stride, dw_t_pad, dw_b_pad, dw_l_pad,
                                             dw_r_pad, output_channels, input_channels, input_height, input_width))
     {

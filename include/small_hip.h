@@ -82,6 +82,29 @@ int small_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, small_hip_str
 int small_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, small_hip_stream_t stream);
 int small_hip_memset(void *dst, int value, size_t bytes, small_hip_stream_t stream);
 int small_hip_stream_synchronize(small_hip_stream_t stream);
+/* Library-owned device scratch (no counterpart in the reference, whose layers work in place on the host).  Two kinds
+ * of entry point lease a block per (device, stream): small_hip_conv2d_u8 / small_hip_group_conv2d_u8 (the prepared
+ * filter: small_hip_conv2d_u8_prepared_filter_bytes, times the group count), and the float32 convolution entry points
+ * for a few long-reduction shapes (partial sums of the equal-share split: small_hip_conv2d_f32_workspace_bytes).
+ * The first such call on a stream allocates (hipMalloc); a larger request later allocates a new block and KEEPS the
+ * old one, so a pointer the library handed to a queued kernel or to a captured graph stays valid; nothing is freed
+ * until small_hip_workspace_release().  The pool's lock is held from the lease until the call's launches are
+ * enqueued, so such calls from several host threads take turns.  Callers with a latency budget or a graph to capture
+ * call small_hip_workspace_reserve() with their largest size first; every other entry point allocates nothing. */
+/* make the calling device's block of `stream` at least `bytes` long now */
+int small_hip_workspace_reserve(size_t bytes, small_hip_stream_t stream);
+/* free every scratch block of the calling device; call when no queued kernel or live graph of that device uses
+ * library scratch (it waits for the device) */
+int small_hip_workspace_release(void);
+/* bytes of scratch the library holds on the calling device */
+size_t small_hip_workspace_held(void);
+/* scratch bytes a small_hip_conv2d_f32-family call of this shape leases (0 for most shapes) */
+size_t small_hip_conv2d_f32_workspace_bytes(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                                            int b_pad, int l_pad, int r_pad, int output_channels, int input_channels,
+                                            int input_height, int input_width);
+/* One integer of SMALL_HIP_TUNE="key=value,..." (measurement switches; nothing in production needs them), or
+ * default_value.  The C++ headers read their own switches (fuse_pool, fuse_conv_dw, one_launch) through it. */
+int small_hip_tune_int(const char *key, int default_value);
 
 
 /* ---- float32 layers -------------------------------------------------------------------- */
@@ -145,6 +168,29 @@ int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kernel_height
                                                     const float *input, const float *filter, const float *bias,
                                                     const float *dw_filter, const float *dw_bias, int act,
                                                     float negative_slope, float *output, small_hip_stream_t stream);
+/* Does the library run this convolution + depthwise pair as ONE launch when both are available (the rule the entry
+ * point below applies; shapes only, no pointers)?  0: no (the one-launch kernels are not built for it, or the two
+ * launches are faster); 1: yes, and the result equals the two launches bit for bit; 2: yes, within float32 rounding of
+ * the two launches (the stand-alone convolution may add its products in another order). */
+int small_hip_conv2d_dwconv2d_one_launch_f32(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
+                                             int b_pad, int l_pad, int r_pad, int dw_kernel_height,
+                                             int dw_kernel_width, int dw_stride, int dw_t_pad, int dw_b_pad,
+                                             int dw_l_pad, int dw_r_pad, int output_channels, int input_channels,
+                                             int input_height, int input_width);
+/* The same pairing for ANY convolution + depthwise pair, given the intermediate buffer the reference's functions take
+ * (`inter_output_buf`, include/small/fused_interface_abstract.hpp:1840-1850): [batch][Co/16][Ho][Wo][16], the
+ * convolution's output size.  Succeeds wherever the two layers would.  One launch where a one-launch form exists and
+ * is the faster choice (the two forms above; the intermediate buffer is then not touched), the two layers through
+ * `intermediate` otherwise.  input, intermediate and output must not overlap. */
+int small_hip_conv2d_bias_act_dwconv2d_bias_act_via_f32(int batch, int kernel_height, int kernel_width, int stride,
+                                                        int t_pad, int b_pad, int l_pad, int r_pad, int dw_kernel_height,
+                                                        int dw_kernel_width, int dw_stride, int dw_t_pad, int dw_b_pad,
+                                                        int dw_l_pad, int dw_r_pad, int output_channels,
+                                                        int input_channels, int input_height, int input_width,
+                                                        const float *input, const float *filter, const float *bias,
+                                                        const float *dw_filter, const float *dw_bias, int act,
+                                                        float negative_slope, float *intermediate, float *output,
+                                                        small_hip_stream_t stream);
 /* PartialConv2DLayer::compute_output (include/small/PartialConv2DLayer.hpp:407-463) in one pass:
  * out = act((out + conv(in, filter)) + bias), i.e. PartialConv2D + PartialBias + activation. */
 int small_hip_partial_conv2d_bias_act_f32(int batch, int kernel_height, int kernel_width, int stride,

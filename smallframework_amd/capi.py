@@ -76,12 +76,19 @@ SIGNATURES = {
     "small_hip_memcpy_d2d": (_i, [_p, _p, _sz, _p]),
     "small_hip_memset": (_i, [_p, _i, _sz, _p]),
     "small_hip_stream_synchronize": (_i, [_p]),
+    "small_hip_workspace_reserve": (_i, [_sz, _p]),
+    "small_hip_workspace_release": (_i, []),
+    "small_hip_workspace_held": (_sz, []),
+    "small_hip_conv2d_f32_workspace_bytes": (_sz, _conv),
+    "small_hip_tune_int": (_i, [C.c_char_p, _i]),
     "small_hip_conv2d_f32": (_i, _conv + [_p, _p, _p, _p]),
     "small_hip_partial_conv2d_f32": (_i, _conv + [_p, _p, _p, _p]),
     "small_hip_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_partial_conv2d_bias_act_f32": (_i, _conv + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_conv2d_bias_act_maxpool2d_f32": (_i, [_i] * 19 + [_p, _p, _p, _i, _f, _p, _p]),
     "small_hip_conv2d_bias_act_dwconv2d_bias_act_f32": (_i, [_i] * 19 + [_p, _p, _p, _p, _p, _i, _f, _p, _p]),
+    "small_hip_conv2d_dwconv2d_one_launch_f32": (_i, [_i] * 19),
+    "small_hip_conv2d_bias_act_dwconv2d_bias_act_via_f32": (_i, [_i] * 19 + [_p, _p, _p, _p, _p, _i, _f, _p, _p, _p]),
     "small_hip_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_partial_depthwise_conv2d_f32": (_i, _win + [_p, _p, _p, _p]),
     "small_hip_depthwise_conv2d_bias_act_f32": (_i, _win + [_p, _p, _p, _i, _f, _p, _p]),

@@ -20,6 +20,21 @@ constexpr int NUM_CU = 256;
 
 void set_error(const char *fmt, ...);
 
+// Measurement switches, all in ONE environment variable read once per process: SMALL_HIP_TUNE="key=value,key=value".
+// Nothing in production needs it; every default is the measured best.  Keys (integers unless noted):
+//   conv_tile=CxP     force the float32 convolution's wave tile (1x1 1x2 2x1 2x2)
+//   conv_tail=0|2     never / always cut left-over tiles into split-K pieces        conv_pw=0   general K loop for 1x1
+//   conv_splitk=0|1   force the split-K kernel off / on                             conv_streamk=0|N  equal-share split off / N per CU
+//   conv_streamk_min  least K-steps for the equal-share split                       stem_lds=0  first layers without the LDS kernel
+//   stem_vec=0|1      16-byte staging of first-layer patches                        smallci_valu=1  vector-ALU first layers
+//   pwdw_cot=1|2      channels (x32) per workgroup of the LDS-parked pointwise + depthwise kernel
+//   fuse_form=3       convolution + depthwise pairs through an intermediate buffer: always the two launches
+//   dw_tile=0         depthwise without the LDS tile kernel                         dw_shape=N  force its tile shape
+//   convq_min_wg, convq_table_min_wg   workgroup targets of the uint8 convolution   fmodel_fuse=0  whole-model kernel without dw + 1x1 fusion
+//   fuse_conv_dw=0|2, fuse_pool=0, one_launch=0|1   the C++ wrappers' choices (read through small_hip_tune_int)
+int tune_int(const char *key, int dflt);
+bool tune_pair(const char *key, int *a, int *b);
+
 inline int fail_hip(hipError_t e, const char *what)
 {
     set_error("%s: %s", what, hipGetErrorString(e));
@@ -109,17 +124,17 @@ __device__ __forceinline__ size_t split_col(size_t col, int Wo, int *ow)
 }
 #endif
 
-// Library-owned device scratch of (current device, stream): grows on demand and is re-used by later calls on the
-// same stream; other streams get their own block.  The lease holds the pool's lock: keep it alive until the last
-// launch that uses `ptr` has been enqueued (a regrow on another thread frees blocks only under that lock, with a
-// call that waits for the device).
+// Library-owned device scratch of (current device, stream): grows on demand (a larger request allocates a new block
+// and keeps the old one allocated, so pointers handed out earlier stay valid) and is re-used by later calls on the
+// same stream; other streams get their own block.  Blocks are freed only by small_hip_workspace_release().  The
+// lease holds the pool's lock: keep it alive until the last launch that uses `ptr` has been enqueued (a release on
+// another thread waits for that lock).
 struct WorkspaceLease
 {
     std::unique_lock<std::mutex> lock;
     void *ptr = nullptr;
 };
 int lease_workspace(size_t bytes, hipStream_t stream, WorkspaceLease *lease);
-
 // uint8 convolution filter pre-pass (conv_u8.hip): packed filter [Co/16][Ci/16][tap][16 ci][16 co] -> signed bytes in
 // MFMA operand order [Co/16][S_pad][16 co][16 ci] (S = taps * Ci/16 steps, padded to a multiple of 4 with zeros),
 // followed at prepared_table_offset_u8() by the int32 prefix table P[(kh+1)*(kw+1)][Co] of the per-tap filter sums

@@ -1574,8 +1574,8 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
 template <int COT, int PXT>
 bool tail_pays(int n_main, int rest, int nsteps)
 {
-    // tuning knob SMALL_HIP_CONV_TAIL: 0 = never, 2 = whenever tiles are left over
-    static const int knob = [] { const char *e = std::getenv("SMALL_HIP_CONV_TAIL"); return e ? e[0] - '0' : 1; }();
+    // SMALL_HIP_TUNE key conv_tail: 0 = never, 2 = whenever tiles are left over
+    static const int knob = tune_int("conv_tail", 1);
     (void)n_main;
     if (knob == 0 || rest == 0 || nsteps < 8) return false;
     return knob == 2 || rest <= NUM_CU / 2;
@@ -1589,8 +1589,8 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
-    // pointwise form of the main loop (tuning knob SMALL_HIP_CONV_PW=0 switches it off)
-    static const bool pw_off = [] { const char *e = std::getenv("SMALL_HIP_CONV_PW"); return e && e[0] == '0'; }();
+    // pointwise form of the main loop (SMALL_HIP_TUNE key conv_pw=0 switches it off)
+    static const bool pw_off = tune_int("conv_pw", 1) == 0;
     const bool pw = !pw_off && a.kh == 1 && a.kw == 1 && a.stride == 1 && a.stride_h == 1 && a.pt == 0 && a.pl == 0 &&
                     a.Ho == a.H && a.Wo == a.W;
     const unsigned slabs_y = a.slabs > 0 ? a.slabs : 1;
@@ -1617,31 +1617,40 @@ struct GroupSlabs
     int stride_h = 0;        // > 0: another vertical stride (1 for the 1-D layers)
 };
 
-// the equal-share launch pair; false: the shape does not qualify
+// The equal-share split of a launch: fills the sk_* fields and the tile counts; returns the scratch bytes it needs, 0 when
+// the shape does not qualify.  Few tiles that do not fill whole rounds and a long reduction (measured, batch 16 on 13x13
+// maps: 512 -> 1024 3x3 287 -> 264 us, 1024 -> 1024 519 -> 467 us, 256 -> 512 (144 steps) 81 -> 69 us; with 72 steps or
+// fewer the fix-up pass costs more than the balance gains).  SMALL_HIP_TUNE keys conv_streamk=<workgroups per compute
+// unit> (default 2, 0 = never), conv_streamk_min=<steps> (default 128)
 template <int COT, int PXT>
-int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
+size_t streamk_plan(ConvArgs &a)
 {
-    *done = false;
+    static const int min_steps = tune_int("conv_streamk_min", 128);
+    static const int per_cu = tune_int("conv_streamk", 2);
+    if (per_cu <= 0 || a.slabs != 0 || a.Co % (32 * COT) != 0) return 0;
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     const int nsteps = a.kh * a.kw * (a.Ci / CB);
     const long total = (long)a.n_blocks * nsteps;
-    // few tiles that do not fill whole rounds and a long reduction (measured, batch 16 on 13x13 maps: 512 -> 1024 3x3 287 -> 264 us,
-    // 1024 -> 1024 519 -> 467 us, 256 -> 512 (144 steps) 81 -> 69 us; with 72 steps or fewer the fix-up pass costs more than
-    // the balance gains).  SMALL_HIP_CONV_STREAMK=<workgroups per compute unit> (default 2), _MIN=<steps> (default 128)
-    static const int min_steps = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK_MIN"); return e ? std::atoi(e) : 128; }();
-    static const int per_cu = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK"); const int v = e ? std::atoi(e) : 2; return v > 0 ? v : 2; }();
-    if (a.n_blocks <= NUM_CU / 2 || a.n_blocks >= 3 * NUM_CU || a.n_blocks % NUM_CU == 0 || nsteps < min_steps || a.Co % (32 * COT) != 0)
-        return SMALL_HIP_OK;
+    if (a.n_blocks <= NUM_CU / 2 || a.n_blocks >= 3 * NUM_CU || a.n_blocks % NUM_CU == 0 || nsteps < min_steps) return 0;
     const int chunks = per_cu * NUM_CU;
-    a.sk_chunks = chunks;
     a.sk_chunk = (int)((total + chunks - 1) / chunks);
     a.sk_chunks = (int)((total + a.sk_chunk - 1) / a.sk_chunk);
     a.sk_parts = (nsteps + a.sk_chunk - 1) / a.sk_chunk + 1;
     a.per_xcd = (a.sk_chunks + NUM_XCD - 1) / NUM_XCD;
+    return (size_t)a.n_blocks * a.sk_parts * sk_part_floats<COT, PXT>() * sizeof(float);
+}
+
+// the equal-share launch pair; *done = false: the shape does not qualify.  The first call on a stream allocates the
+// scratch block (small_hip_workspace_reserve does it ahead of time), like the uint8 convolution's filter pre-pass.
+template <int COT, int PXT>
+int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
+{
+    *done = false;
+    const size_t bytes = streamk_plan<COT, PXT>(a);
+    if (bytes == 0) return SMALL_HIP_OK;
     WorkspaceLease lease;            // held until both launches are enqueued
-    const size_t bytes = (size_t)a.n_blocks * a.sk_parts * sk_part_floats<COT, PXT>() * sizeof(float);
     if (int rc = lease_workspace(bytes, s, &lease)) return rc;
     a.sk_scratch = static_cast<float *>(lease.ptr);
     hipLaunchKernelGGL((conv_mfma_f32_streamk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
@@ -1650,6 +1659,14 @@ int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
     SHP_LAUNCH_CHECK(op);
     *done = true;
     return SMALL_HIP_OK;
+}
+
+// few tiles and a long reduction: K split over the four waves of a workgroup (measured: from one tile per SIMD the
+// whole-rounds + tail kernel with 1x1 wave tiles is ahead, e.g. 256->512 3x3 @13x13 batch 16, 1360 tiles: 81 us against 91 us)
+inline bool wants_splitk(long tiles32, int nsteps)
+{
+    static const int force = tune_int("conv_splitk", -1);
+    return force >= 0 ? force == 1 : (tiles32 < 4L * NUM_CU && nsteps >= 16);
 }
 
 int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co,
@@ -1696,8 +1713,8 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
 
     if (small_ci)
     {
-        // 3x3 windows: the LDS-staged 16x16x4 MFMA kernel (tuning knob SMALL_HIP_STEM_LDS=0 switches it off)
-        static const bool stem_lds_off = [] { const char *e = std::getenv("SMALL_HIP_STEM_LDS"); return e && e[0] == '0'; }();
+        // 3x3 windows: the LDS-staged 16x16x4 MFMA kernel (SMALL_HIP_TUNE key stem_lds=0 switches it off)
+        static const bool stem_lds_off = tune_int("stem_lds", 1) == 0;
         if (!stem_lds_off && kh == 3 && kw == 3 && (long)H * W * Ci < 0x7fffffffL)
         {
             const int tiles_x = (a.Wo + 15) / 16, tiles_y = (a.Ho + 15) / 16;
@@ -1710,7 +1727,7 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
                 void (*ks)(const ConvArgs, int, int) = nullptr;
                 // 16-byte staging (possible when every image row is whole 16-byte pieces) is measured level or slightly behind
                 // here (224x224x3 -> 32 stride 2: 33.6 against 34.6 us) and ahead in the pooling form below; on request only
-                static const bool vec_on = [] { const char *e = std::getenv("SMALL_HIP_STEM_VEC"); return e && e[0] == '1'; }();
+                static const bool vec_on = tune_int("stem_vec", 0) == 1;
                 const bool vec = vec_on && (W * Ci) % 4 == 0 && aligned16(in);
 #define SHP_STEM_V(CI_, S_, V_) (ncob == 4 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 4, false, V_> : ncob == 2 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 2, false, V_> : conv_stem3x3_lds_f32_kernel<CI_, S_, 1, false, V_>)
 #define SHP_STEM(CI_, S_) (vec ? SHP_STEM_V(CI_, S_, true) : SHP_STEM_V(CI_, S_, false))
@@ -1724,7 +1741,7 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
             }
         }
         const dim3 grid((unsigned)((a.P + 255) / 256), (unsigned)(Co / CB));
-        static const bool smallci_valu = [] { const char *e = std::getenv("SMALL_HIP_SMALLCI_VALU"); return e && e[0] == '1'; }();
+        static const bool smallci_valu = tune_int("smallci_valu", 0) == 1;
         // measured: with 16 output channels half of every 32-row MFMA tile is idle and the vector-ALU
         // kernel is faster
         if (!smallci_valu && Co >= 32 && (long)H * W * Ci < 0x7fffffffL)
@@ -1761,27 +1778,18 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
     int cot = 1, pxt = 1;
     if (Co % 64 == 0 && tiles32 >= 16 * simds && nsteps >= 32) { cot = 2; pxt = 2; }
     else if (Co % 64 == 0 && (tiles32 >= 4 * simds || (tiles32 >= 2 * simds && nsteps >= 72))) { cot = 2; pxt = 1; }
-    // few tiles and a long reduction: split K over the four waves of a workgroup
-    // (measured: from one tile per SIMD the whole-rounds + tail kernel with 1x1 wave tiles is ahead, e.g. 256->512 3x3
-    // @13x13 batch 16, 1360 tiles: 81 us against 91 us)
-    bool splitk = tiles32 < simds && nsteps >= 16;
-    if (const char *e = std::getenv("SMALL_HIP_CONV_SPLITK")) splitk = e[0] == '1';
-    if (splitk)
+    if (wants_splitk(tiles32, nsteps))
     {
         launch_splitk<1, 1>(a, s);
         SHP_LAUNCH_CHECK(op);
         return SMALL_HIP_OK;
     }
-    // tuning knob: SMALL_HIP_CONV_TILE="<cot>,<pxt>" forces a wave tile (32-channel x 32-pixel units; 1,1 1,2 2,1 2,2)
-    if (const char *e = std::getenv("SMALL_HIP_CONV_TILE"))
+    // SMALL_HIP_TUNE key conv_tile=<cot>x<pxt> forces a wave tile (32-channel x 32-pixel units; 1x1 1x2 2x1 2x2)
     {
         int c2 = 0, p2 = 0;
-        if (std::sscanf(e, "%d,%d", &c2, &p2) == 2) { cot = c2; pxt = p2; }
+        if (tune_pair("conv_tile", &c2, &p2)) { cot = c2; pxt = p2; }
     }
-    // few tiles, long reduction: equal shares of the K-steps (tuning knob SMALL_HIP_CONV_STREAMK=0 switches it off; the
-    // first call on a stream allocates the scratch block, like the uint8 convolution's filter pre-pass)
-    static const bool streamk_off = [] { const char *e = std::getenv("SMALL_HIP_CONV_STREAMK"); return e && e[0] == '0'; }();
-    if (!streamk_off && grp.slabs == 0 && Co % 64 == 0)
+    // few tiles, long reduction: equal shares of the K-steps
     {
         bool done = false;
         if (int rc = launch_streamk<2, 1>(op, a, s, &done)) return rc;
@@ -1860,7 +1868,7 @@ int conv_pool_f32(const char *op, int batch, int kh, int kw, int stride, int pt,
         const dim3 gs((unsigned)nt, (unsigned)(CoB / ncob));
         void (*ks)(const ConvArgs, int, int) = nullptr;
         // 16-byte staging when every image row is whole 16-byte pieces (416x416x3 -> 16 + pool, batch 16: 47.8 -> 43.8 us)
-        static const bool vec_off = [] { const char *e = std::getenv("SMALL_HIP_STEM_VEC"); return e && e[0] == '0'; }();
+        static const bool vec_off = tune_int("stem_vec", 1) == 0;
         const bool vec = !vec_off && (W * Ci) % 4 == 0 && aligned16(in);
 #define SHP_STEM_V(CI_, S_, V_) (ncob == 4 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 4, true, V_> : ncob == 2 ? conv_stem3x3_lds_f32_kernel<CI_, S_, 2, true, V_> : conv_stem3x3_lds_f32_kernel<CI_, S_, 1, true, V_>)
 #define SHP_STEM(CI_, S_) (vec ? SHP_STEM_V(CI_, S_, true) : SHP_STEM_V(CI_, S_, false))
@@ -1965,9 +1973,9 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     const long nt = (long)batch * g.tiles_x * g.tiles_y;
     const StemDwArgs d{dw_filt, dw_bias};
     // channels per workgroup: 32 (four workgroups per compute unit) is measured ahead of 64 (two; the activation operand is
-    // loaded once per 64 output channels) on every MobileNetV1 pair at batch 64, by 1-3 us.  Tuning knob SMALL_HIP_PWDW_COT=1|2.
+    // loaded once per 64 output channels) on every MobileNetV1 pair at batch 64, by 1-3 us.  SMALL_HIP_TUNE key pwdw_cot=1|2.
     int cot = 1;
-    if (const char *e = std::getenv("SMALL_HIP_PWDW_COT")) { const int v = std::atoi(e); if (v == 1 || (v == 2 && Co % 64 == 0 && (cib == 2 || cib == 4 || cib == 8))) cot = v; }
+    { static const int v = tune_int("pwdw_cot", 1); if (v == 1 || (v == 2 && Co % 64 == 0 && (cib == 2 || cib == 4 || cib == 8))) cot = v; }
     g.n_cg = Co / (32 * cot);
     if (nt * g.n_cg > 0x7fffffffL / 2) { set_error("%s: too many tiles for one launch", op); return SMALL_HIP_EINVAL; }
     g.n_wgs = (int)(nt * g.n_cg); g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
@@ -1982,6 +1990,7 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     SHP_LAUNCH_CHECK(op);
     return SMALL_HIP_OK;
 }
+
 
 } // namespace
 
@@ -2043,6 +2052,91 @@ int small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(int batch, int kh, int kw, i
         return pw_dw_f32(op, batch, dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
     return stem_dw_f32(op, batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw,
                        dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
+}
+
+size_t small_hip_conv2d_f32_workspace_bytes(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int Co, int Ci,
+                                            int H, int W)
+{
+    if (batch <= 0 || kh <= 0 || kw <= 0 || Co <= 0 || Ci <= 0 || Ci % CB != 0 || Co % CB != 0 || (stride != 1 && stride != 2) ||
+        !pads_ok(pt, pb, pl, pr))
+        return 0;
+    ConvArgs a{};
+    a.Co = Co; a.Ci = Ci; a.kh = kh; a.kw = kw;
+    const long P = (long)batch * out_dim(H, pt, pb, kh, stride) * out_dim(W, pl, pr, kw, stride);
+    if (P <= 0 || P > 0x7fffffffL / 64) return 0;
+    a.P = (int)P;
+    if (wants_splitk((long)((Co + 31) / 32) * ((P + 31) / 32), kh * kw * (Ci / CB))) return 0;
+    return streamk_plan<2, 1>(a);
+}
+
+int small_hip_conv2d_dwconv2d_one_launch_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr, int dw_kh,
+                                             int dw_kw, int dw_stride, int dpt, int dpb, int dpl, int dpr, int Co, int Ci, int H,
+                                             int W)
+{
+    if (batch <= 0 || H <= 0 || W <= 0 || Co <= 0 || Ci <= 0 || dw_kh != 3 || dw_kw != 3 || !pads_ok(pt, pb, pl, pr) ||
+        !pads_ok(dpt, dpb, dpl, dpr) || (long)Ci * H * W > 0x7fffffffL / 2)
+        return 0;
+    if (Ci <= 3)
+    {
+        // a first layer on 16 x 16 tiles in front of a stride-1 depthwise layer with one pixel of padding (stem_dw_f32)
+        if (kh != 3 || kw != 3 || (stride != 1 && stride != 2) || dw_stride != 1 || dpt != 1 || dpb != 1 || dpl != 1 || dpr != 1 ||
+            Co % CB != 0)
+            return 0;
+        const long Ho = out_dim(H, pt, pb, 3, stride), Wo = out_dim(W, pl, pr, 3, stride);
+        if (Ho <= 0 || Wo <= 0) return 0;
+        const long nt = (long)batch * ((Wo + 13) / 14) * ((Ho + 13) / 14);
+        return nt <= 0x7fffffffL && (long)batch * Co * Ho * Wo <= 0x7fffffffL * 4L ? 1 : 0;
+    }
+    // a pointwise convolution parked in LDS under 14 x 14 (stride 2: 7 x 8) depthwise tiles (pw_dw_f32): short reductions
+    // on maps that fill those tiles to 70%, where the recomputed halo costs less than the second launch.  Measured on
+    // MobileNetV1's pairs at batch 64: 32 -> 64 @112x112 stride 2 104 -> 54 us, 64 -> 128 @56x56 70 -> 54 us, 128 -> 256
+    // @28x28 53 -> 46 us; 128 -> 128 @56x56 stride 2 81 -> 85 us (two launches stay)
+    if (kh != 1 || kw != 1 || stride != 1 || pt || pb || pl || pr || Ci % CB != 0 || Co % 32 != 0 || (dw_stride != 1 && dw_stride != 2))
+        return 0;
+    const int cib = Ci / CB;
+    if (!(cib <= 4 || ((cib == 6 || cib == 8) && dw_stride == 1))) return 0;
+    const int Hd = out_dim(H, dpt, dpb, 3, dw_stride), Wd = out_dim(W, dpl, dpr, 3, dw_stride);
+    if (Hd <= 0 || Wd <= 0) return 0;
+    const int toh = dw_stride == 1 ? 14 : 7, tow = dw_stride == 1 ? 14 : 8;
+    const long tx = (Wd + tow - 1) / tow, ty = (Hd + toh - 1) / toh;
+    if (10L * Hd * Wd < 7 * (tx * tow) * (ty * toh)) return 0;
+    if ((long)batch * tx * ty * (Co / 32) > 0x7fffffffL / 2) return 0;
+    // the stand-alone convolution adds its products in one pass below eight K-steps; from eight on it may cut left-over
+    // tiles along the input channels
+    return cib < 8 ? 1 : 2;
+}
+
+int small_hip_conv2d_bias_act_dwconv2d_bias_act_via_f32(int batch, int kh, int kw, int stride, int pt, int pb, int pl, int pr,
+                                                        int dw_kh, int dw_kw, int dw_stride, int dpt, int dpb, int dpl, int dpr,
+                                                        int Co, int Ci, int H, int W, const float *in, const float *filt,
+                                                        const float *bias, const float *dw_filt, const float *dw_bias, int act,
+                                                        float slope, float *intermediate, float *out, small_hip_stream_t stream)
+{
+    const char *op = "small_hip_conv2d_bias_act_dwconv2d_bias_act_via_f32";
+    if (!intermediate || !in || !out) { set_error("%s: null tensor", op); return SMALL_HIP_EINVAL; }
+    {
+        // whichever form runs, no tensor may be written while another launch or workgroup still reads it
+        const long Ho = out_dim(H, pt, pb, kh, stride > 0 ? stride : 1), Wo = out_dim(W, pl, pr, kw, stride > 0 ? stride : 1);
+        const long Hd = out_dim((int)Ho, dpt, dpb, dw_kh, dw_stride > 0 ? dw_stride : 1), Wd = out_dim((int)Wo, dpl, dpr, dw_kw, dw_stride > 0 ? dw_stride : 1);
+        if (batch > 0 && Ci > 0 && Co > 0 && H > 0 && W > 0 && Ho > 0 && Wo > 0 && Hd > 0 && Wd > 0)
+        {
+            const size_t n_in = (size_t)batch * Ci * H * W, n_mid = (size_t)batch * Co * Ho * Wo, n_out = (size_t)batch * Co * Hd * Wd;
+            auto overlap = [](const float *p, size_t n, const float *q, size_t m) { return p < q + m && q < p + n; };
+            if (overlap(in, n_in, intermediate, n_mid) || overlap(in, n_in, out, n_out) || overlap(intermediate, n_mid, out, n_out))
+            { set_error("%s: input, intermediate and output tensors must not overlap", op); return SMALL_HIP_EINVAL; }
+        }
+    }
+    // SMALL_HIP_TUNE key fuse_form=3: always the two layers (read per call: tests switch it)
+    if (tune_int("fuse_form", 0) != 3 &&
+        small_hip_conv2d_dwconv2d_one_launch_f32(batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw, dw_stride, dpt, dpb, dpl, dpr, Co, Ci, H, W))
+        return small_hip_conv2d_bias_act_dwconv2d_bias_act_f32(batch, kh, kw, stride, pt, pb, pl, pr, dw_kh, dw_kw, dw_stride, dpt, dpb, dpl,
+                                                               dpr, Co, Ci, H, W, in, filt, bias, dw_filt, dw_bias, act, slope, out, stream);
+    // the two layers, one after the other
+    if (int rc = conv_f32(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, filt, bias, act, slope, 0, intermediate, stream)) return rc;
+    const int Ho = out_dim(H, pt, pb, kh, stride), Wo = out_dim(W, pl, pr, kw, stride);
+    if (Ho <= 0 || Wo <= 0) return SMALL_HIP_OK;
+    return small_hip_depthwise_conv2d_bias_act_f32(batch, dw_kh, dw_kw, dw_stride, dpt, dpb, dpl, dpr, Co, Ho, Wo, intermediate, dw_filt,
+                                                   dw_bias, act, slope, out, stream);
 }
 
 // One convolution of `channels` -> `channels` per slab of `channels` channels; slab g of image n starts

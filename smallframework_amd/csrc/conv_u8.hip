@@ -476,7 +476,7 @@ __global__ __launch_bounds__(256) void conv_smallci_u8_kernel(const QSmallArgs a
 // workgroups from which the post-op table pays (below, the launch is latency-bound and the table only adds a barrier)
 long table_min_wg()
 {
-    static const long v = [] { const char *e = std::getenv("SMALL_HIP_CONVQ_TABLE_MIN_WG"); return e ? std::atol(e) : 2L * NUM_CU; }();
+    static const long v = tune_int("convq_table_min_wg", 2 * NUM_CU);
     return v;
 }
 
@@ -618,7 +618,7 @@ int conv_u8_run(const char *op, int batch, int kh, int kw, int stride, int pt, i
     // The largest wave tile (COT channel blocks x PXT pixel groups of 16) that still leaves at least
     // `want` workgroups: these layers are small and latency-bound, so filling the chip with waves
     // comes before operand re-use.
-    static const long want = [] { const char *e = std::getenv("SMALL_HIP_CONVQ_MIN_WG"); return e ? std::atol(e) : 512L; }();
+    static const long want = tune_int("convq_min_wg", 512);
     auto nwg = [&](int cot, int pxt) { return (long)((CoB + cot - 1) / cot) * ((P + 64 * pxt - 1) / (64 * pxt)) * n_slabs; };
     if (CoB % 4 == 0 && nwg(4, 2) >= want) launch_q<4, 2>(a, s);
     else if (CoB % 2 == 0 && nwg(2, 2) >= want) launch_q<2, 2>(a, s);

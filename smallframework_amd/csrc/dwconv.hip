@@ -372,7 +372,7 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
     if (kh == 3 && kw == 3)
     {
         constexpr int R1 = 4, R2 = 3;      // output rows per lane at stride 1 / stride 2
-        static const bool tile_off = [] { const char *v = std::getenv("SMALL_HIP_DW_TILE"); return v && v[0] == '0'; }();
+        static const bool tile_off = tune_int("dw_tile", 1) == 0;
         // measured: the strip kernel wins below 7x7 outputs at stride 1 and below 14x14 at stride 2 (256 channels 28x28 -> 14x14,
         // batch 64: tile kernel 11.4 us, strip kernel 14.0 us; 512 channels 14x14 -> 7x7: 7.0 us either way)
         const int min_side = stride == 1 ? 7 : 14;
@@ -395,10 +395,9 @@ int dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int pb
                 if (stride == 1 && t == 4) util *= 0.92;
                 if (util > best_util + 1e-9) { best_util = util; best = t; }
             }
-            // tuning knob: force a shape of the table
-            if (const char *v = std::getenv("SMALL_HIP_DW_SHAPE"))
+            // SMALL_HIP_TUNE key dw_shape: force a shape of the table
             {
-                const int f = std::atoi(v);
+                static const int f = tune_int("dw_shape", -1);
                 if (f >= 0 && f < nshapes) best = f;
             }
             if (best >= 0)

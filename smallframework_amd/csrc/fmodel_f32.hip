@@ -767,8 +767,8 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
 
     // The launch's layer list.  A 3x3 depthwise convolution whose only reader is the 1x1 stride-1 convolution right
     // after it becomes one layer with it (their weights already lie back to back in the blob); the depthwise tensor
-    // then needs no LDS.  SMALL_HIP_FMODEL_FUSE=0 keeps the layers apart (a measurement aid).
-    static const bool fuse_off = [] { const char *e = std::getenv("SMALL_HIP_FMODEL_FUSE"); return e && e[0] == '0'; }();
+    // then needs no LDS.  SMALL_HIP_TUNE key fmodel_fuse=0 keeps the layers apart (a measurement aid).
+    static const bool fuse_off = tune_int("fmodel_fuse", 1) == 0;
     int tensor_floats[MAX_TENSORS] = {};
     int dev_src[MAX_LAYERS], dev_dst[MAX_LAYERS], n_dev = 0;
     // where a caller's tensor id lives: a fused pair must not write the tensor it reads (callers ping-pong between two

@@ -2,6 +2,7 @@
 #include "common.h"
 #include "workspace.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -37,10 +38,11 @@ struct HipMem
     }
 };
 
+// never destroyed: the blocks outlive static destruction order
 WorkspacePool<HipMem> &pool()
 {
     static WorkspacePool<HipMem> *p = [] {
-        auto *q = new WorkspacePool<HipMem>();       // never destroyed: blocks outlive static destruction order
+        auto *q = new WorkspacePool<HipMem>();
         q->set_full_code(SMALL_HIP_ENOMEM);
         return q;
     }();
@@ -50,16 +52,46 @@ WorkspacePool<HipMem> &pool()
 
 int lease_workspace(size_t bytes, hipStream_t stream, WorkspaceLease *lease)
 {
+    auto &pl = pool();
     int dev = 0;
     SHP_HIP(hipGetDevice(&dev));
-    lease->lock = pool().lock();
-    int rc = pool().acquire(dev, stream, bytes, &lease->ptr);
+    lease->lock = pl.lock();
+    int rc = pl.acquire(dev, stream, bytes, &lease->ptr);
     if (rc != SMALL_HIP_OK)
     {
-        if (rc == SMALL_HIP_ENOMEM && small_hip_last_error()[0] == 0) set_error("workspace: too many streams hold a block");
+        if (rc == SMALL_HIP_ENOMEM && small_hip_last_error()[0] == 0)
+            set_error("workspace: %zu streams hold a block already; small_hip_workspace_release() makes room", pl.blocks());
         lease->lock.unlock();
     }
     return rc;
+}
+
+// SMALL_HIP_TUNE="key=value,key=value": the value of `key`, or null
+static const char *tune_find(const char *key)
+{
+    const char *env = std::getenv("SMALL_HIP_TUNE");     // call sites on launch paths keep the answer in a static
+    if (!env) return nullptr;
+    const size_t n = std::strlen(key);
+    for (const char *p = env; *p;)
+    {
+        if (std::strncmp(p, key, n) == 0 && p[n] == '=') return p + n + 1;
+        const char *c = std::strchr(p, ',');
+        if (!c) break;
+        p = c + 1;
+    }
+    return nullptr;
+}
+
+int tune_int(const char *key, int dflt)
+{
+    const char *v = tune_find(key);
+    return v ? std::atoi(v) : dflt;
+}
+
+bool tune_pair(const char *key, int *a, int *b)
+{
+    const char *v = tune_find(key);
+    return v && std::sscanf(v, "%dx%d", a, b) == 2;
 }
 
 } // namespace shp
@@ -87,6 +119,8 @@ const char *small_hip_strerror(int status)
 
 const char *small_hip_last_error(void) { return g_err; }
 
+int small_hip_tune_int(const char *key, int default_value) { return key ? tune_int(key, default_value) : default_value; }
+
 int small_hip_device_count(void)
 {
     int n = 0;
@@ -98,6 +132,29 @@ int small_hip_set_device(int device)
 {
     SHP_HIP(hipSetDevice(device));
     return SMALL_HIP_OK;
+}
+
+int small_hip_workspace_reserve(size_t bytes, small_hip_stream_t stream)
+{
+    g_err[0] = 0;
+    WorkspaceLease lease;
+    return lease_workspace(bytes, as_stream(stream), &lease);
+}
+
+int small_hip_workspace_release(void)
+{
+    int dev = 0;
+    SHP_HIP(hipGetDevice(&dev));
+    auto lk = pool().lock();
+    return pool().release_device(dev);
+}
+
+size_t small_hip_workspace_held(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    auto lk = pool().lock();
+    return pool().held(dev);
 }
 
 int small_hip_malloc(void **ptr, size_t bytes)

@@ -1,6 +1,7 @@
 // CPU unit test of the scratch-block bookkeeping (smallframework_amd/csrc/workspace.h) with a fake allocator:
-// one block per (device, stream), a block only grows, the old block is released before the new one is made, nothing
-// is ever released twice or while another stream's block is handed out, and the lock serialises acquire-to-enqueue.
+// one current block per (device, stream); growth adds a block and keeps the old one allocated (a pointer handed out
+// stays valid until release_device); a full table refuses instead of evicting; nothing is released twice; the lock
+// serialises acquire-to-enqueue.
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -26,7 +27,7 @@ struct FakeMem
 {
     static std::map<void *, size_t> live;
     static std::set<void *> released;
-    static int fail_next_alloc;
+    static int fail_next_alloc, fail_next_release;
     static long allocs, releases;
     static int alloc(void **p, size_t bytes)
     {
@@ -38,6 +39,7 @@ struct FakeMem
     }
     static int release(void *p)
     {
+        if (fail_next_release) { int rc = fail_next_release; fail_next_release = 0; return rc; }
         if (!live.count(p)) { std::printf("release of a block that is not live\n"); ++g_failures; return 0; }
         live.erase(p);
         released.insert(p);                     // kept allocated so that addresses are never re-used in the test
@@ -47,7 +49,7 @@ struct FakeMem
 };
 std::map<void *, size_t> FakeMem::live;
 std::set<void *> FakeMem::released;
-int FakeMem::fail_next_alloc = 0;
+int FakeMem::fail_next_alloc = 0, FakeMem::fail_next_release = 0;
 long FakeMem::allocs = 0, FakeMem::releases = 0;
 
 using Pool = shp::WorkspacePool<FakeMem>;
@@ -66,13 +68,35 @@ static void test_per_stream_blocks()
     void *a2 = nullptr;
     CHECK(pool.acquire(0, &s1, 500, &a2) == 0 && a2 == a);          // smaller request: same block
     CHECK(pool.acquire(0, &s1, Pool::GRANULE, &a2) == 0 && a2 == a);
-    const long rel = FakeMem::releases;
-    CHECK(pool.acquire(0, &s1, Pool::GRANULE + 1, &a2) == 0 && a2 != a);   // growth: old block released first
-    CHECK(FakeMem::releases == rel + 1 && FakeMem::released.count(a) && !FakeMem::live.count(a));
-    CHECK(FakeMem::live.count(b) && FakeMem::live.count(c));        // the other streams' blocks are untouched
-    CHECK(pool.capacity(0, &s1) == 2 * Pool::GRANULE);
     CHECK(pool.release_device(0) == 0 && pool.blocks() == 1 && FakeMem::live.count(c) && !FakeMem::live.count(b));
     CHECK(pool.release_device(1) == 0 && FakeMem::live.empty());
+}
+
+static void test_a_pointer_handed_out_stays_valid_after_growth()
+{
+    // a kernel already queued, or a captured graph replayed later, may still use the smaller block: growth adds a
+    // block and retires the old one, which stays allocated until release_device()
+    Pool pool;
+    int s1, s2;
+    void *a = nullptr, *a2 = nullptr, *a3 = nullptr, *b = nullptr;
+    auto lk = pool.lock();
+    CHECK(pool.acquire(0, &s1, 1000, &a) == 0 && a);
+    CHECK(pool.acquire(0, &s2, 1000, &b) == 0 && b);
+    const long rel = FakeMem::releases;
+    CHECK(pool.acquire(0, &s1, Pool::GRANULE + 1, &a2) == 0 && a2 && a2 != a);
+    CHECK(FakeMem::releases == rel && FakeMem::live.count(a) && FakeMem::live.count(a2));   // nothing was freed
+    CHECK(pool.capacity(0, &s1) == 2 * Pool::GRANULE && pool.retired() == 1);
+    CHECK(pool.held(0) == 4 * Pool::GRANULE);                       // a, a2 (two granules), b
+    CHECK(pool.acquire(0, &s1, 10 * Pool::GRANULE, &a3) == 0 && a3 != a2 && a3 != a);
+    CHECK(FakeMem::releases == rel && FakeMem::live.count(a) && FakeMem::live.count(a2) && FakeMem::live.count(a3));
+    CHECK(pool.retired() == 2 && pool.blocks() == 2);
+    void *again = nullptr;
+    CHECK(pool.acquire(0, &s1, 1000, &again) == 0 && again == a3);  // later small requests use the large block
+    CHECK(FakeMem::live.count(b));                                  // the other stream's block is untouched
+    // the explicit release frees current and retired blocks of that device, each exactly once
+    CHECK(pool.release_device(0) == 0);
+    CHECK(FakeMem::releases == rel + 4 && FakeMem::live.empty() && pool.blocks() == 0 && pool.retired() == 0);
+    CHECK(pool.held(0) == 0);
 }
 
 static void test_failed_growth_leaves_a_consistent_entry()
@@ -84,29 +108,42 @@ static void test_failed_growth_leaves_a_consistent_entry()
     CHECK(pool.acquire(0, &s, 10, &a) == 0);
     FakeMem::fail_next_alloc = 7;
     CHECK(pool.acquire(0, &s, 5 * Pool::GRANULE, &b) == 7 && b == nullptr);
-    CHECK(pool.capacity(0, &s) == 0 && FakeMem::live.empty());      // the old block is gone, none is recorded
-    CHECK(pool.acquire(0, &s, 10, &b) == 0 && b && FakeMem::live.size() == 1);
+    CHECK(pool.capacity(0, &s) == Pool::GRANULE && FakeMem::live.count(a));   // the old block is still the current one
+    CHECK(pool.acquire(0, &s, 10, &b) == 0 && b == a && FakeMem::live.size() == 1);
     pool.release_device(0);
+    CHECK(FakeMem::live.empty());
 }
 
-static void test_eviction_when_full()
+static void test_a_full_table_refuses_instead_of_evicting()
 {
     Pool pool;
     pool.set_full_code(99);
     std::vector<int> streams(Pool::MAX_BLOCKS + 1);
-    void *p = nullptr, *first = nullptr;
+    std::vector<void *> ptrs(Pool::MAX_BLOCKS);
+    void *p = nullptr;
     auto lk = pool.lock();
-    for (size_t i = 0; i < Pool::MAX_BLOCKS; ++i)
-    {
-        CHECK(pool.acquire(0, &streams[i], 1, &p) == 0);
-        if (i == 0) first = p;
-    }
-    CHECK(pool.acquire(0, &streams[1], 1, &p) == 0);                // touch stream 1: stream 0 stays the oldest
-    CHECK(pool.acquire(0, &streams[Pool::MAX_BLOCKS], 1, &p) == 0); // full: the least recently used block goes
-    CHECK(pool.blocks() == Pool::MAX_BLOCKS && FakeMem::released.count(first));
-    CHECK(pool.acquire(5, &streams[0], 1, &p) == 99);               // no block of device 5 to evict
+    for (size_t i = 0; i < Pool::MAX_BLOCKS; ++i) CHECK(pool.acquire(0, &streams[i], 1, &ptrs[i]) == 0);
+    const long rel = FakeMem::releases;
+    CHECK(pool.acquire(0, &streams[Pool::MAX_BLOCKS], 1, &p) == 99 && p == nullptr);   // full: refused
+    CHECK(FakeMem::releases == rel && pool.blocks() == Pool::MAX_BLOCKS);              // and nothing was freed
+    for (size_t i = 0; i < Pool::MAX_BLOCKS; ++i) CHECK(FakeMem::live.count(ptrs[i]));
+    CHECK(pool.acquire(0, &streams[3], 1, &p) == 0 && p == ptrs[3]);                   // known streams still served
+    CHECK(pool.release_device(0) == 0);                                                // the way to make room
+    CHECK(pool.acquire(0, &streams[Pool::MAX_BLOCKS], 1, &p) == 0 && p);
     pool.release_device(0);
     CHECK(FakeMem::live.empty());
+}
+
+static void test_release_reports_the_first_error()
+{
+    Pool pool;
+    int s1, s2;
+    void *a = nullptr, *b = nullptr;
+    auto lk = pool.lock();
+    CHECK(pool.acquire(0, &s1, 1, &a) == 0 && pool.acquire(0, &s2, 1, &b) == 0);
+    FakeMem::fail_next_release = 5;
+    CHECK(pool.release_device(0) == 5 && pool.blocks() == 0);
+    FakeMem::live.clear();
 }
 
 static void test_lock_covers_acquire_to_enqueue()
@@ -139,8 +176,10 @@ static void test_lock_covers_acquire_to_enqueue()
 int main()
 {
     test_per_stream_blocks();
+    test_a_pointer_handed_out_stays_valid_after_growth();
     test_failed_growth_leaves_a_consistent_entry();
-    test_eviction_when_full();
+    test_a_full_table_refuses_instead_of_evicting();
+    test_release_reports_the_first_error();
     test_lock_covers_acquire_to_enqueue();
     std::printf(g_failures ? "%d CHECKS FAILED\n" : "ALL PASSED\n", g_failures);
     return g_failures ? 1 : 0;

@@ -57,3 +57,42 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.small_hip_upsample2d_f32(1, 3, 16, 4, 4, fake, fake, None) == capi.ESCALE
     assert lib.small_hip_maxpool2d_f32(1, 3, 3, 3, 0, 0, 0, 0, 16, 8, 8, fake, fake, None) == capi.ESTRIDE
     assert lib.small_hip_conv2d_f32(1, 3, 3, 1, 0, 0, 0, 0, 16, 16, 8, 8, None, fake, fake, None) == capi.EINVAL
+
+
+def test_one_launch_predicate_of_conv_dw_pairs():
+    """small_hip_conv2d_dwconv2d_one_launch_f32 is a pure function of the shapes: the rule the C++ wrappers and the
+    entry point with an intermediate buffer share."""
+    lib = capi.load()
+    f = lib.small_hip_conv2d_dwconv2d_one_launch_f32
+    pw = lambda Ci, Co, H, W, ds=1, pads=(1, 1, 1, 1), batch=4: f(batch, 1, 1, 1, 0, 0, 0, 0, 3, 3, ds, *pads, Co, Ci, H, W)
+    assert pw(32, 64, 112, 112, 2, (0, 1, 0, 1)) == 1          # MobileNetV1's fused pairs
+    assert pw(64, 128, 56, 56) == 1
+    assert pw(128, 256, 28, 28) == 2                           # eight K-steps: float32 rounding against two launches
+    assert pw(128, 128, 56, 56, 2, (0, 1, 0, 1)) == 0          # stride 2 behind eight K-steps: two launches are faster
+    assert pw(512, 512, 14, 14) == 0 and pw(80, 64, 28, 28) == 0 and pw(32, 48, 28, 28) == 0
+    assert pw(32, 64, 5, 40) == 0                              # fills the 14 x 14 tiles to 48%
+    assert pw(32, 64, 28, 28, 3) == 0
+    stem = lambda Ci, k, s, ds=1, dp=1, Co=32: f(4, k, k, s, 0, 1, 0, 1, 3, 3, ds, dp, dp, dp, dp, Co, Ci, 224, 224)
+    assert stem(3, 3, 2) == 1 and stem(1, 3, 1) == 1
+    assert stem(3, 5, 2) == 0 and stem(3, 3, 2, ds=2) == 0 and stem(3, 3, 2, dp=0) == 0 and stem(3, 3, 2, Co=24) == 0
+    assert f(4, 3, 3, 1, 1, 1, 1, 1, 3, 3, 1, 1, 1, 1, 1, 64, 32, 28, 28) == 0      # a 3x3 convolution of whole channel blocks
+    assert f(0, 1, 1, 1, 0, 0, 0, 0, 3, 3, 1, 1, 1, 1, 1, 64, 32, 28, 28) == 0
+
+
+def test_tune_string(monkeypatch):
+    lib = capi.load()
+    monkeypatch.delenv("SMALL_HIP_TUNE", raising=False)
+    assert lib.small_hip_tune_int(b"fuse_pool", 5) == 5
+    monkeypatch.setenv("SMALL_HIP_TUNE", "conv_tile=2x1,fuse_pool=0,one_launch=1")
+    assert lib.small_hip_tune_int(b"fuse_pool", 5) == 0
+    assert lib.small_hip_tune_int(b"one_launch", -1) == 1
+    assert lib.small_hip_tune_int(b"launch", 7) == 7           # a key is matched whole, not as a suffix
+    assert lib.small_hip_tune_int(b"conv_streamk", 2) == 2
+
+
+def test_workspace_queries_without_gpu():
+    lib = capi.load()
+    # Tiny-YOLOv2's 13x13 layers at batch 16 take the equal-share split and say how much scratch it leases
+    assert lib.small_hip_conv2d_f32_workspace_bytes(16, 3, 3, 1, 1, 1, 1, 1, 1024, 1024, 13, 13) > 1 << 20
+    assert lib.small_hip_conv2d_f32_workspace_bytes(64, 1, 1, 1, 0, 0, 0, 0, 512, 512, 14, 14) == 0
+    assert lib.small_hip_conv2d_f32_workspace_bytes(16, 3, 3, 1, 1, 1, 1, 1, 16, 3, 416, 416) == 0

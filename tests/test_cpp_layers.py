@@ -143,13 +143,13 @@ def test_models(hip, oracle, name):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["DSCNNTiny", "DSCNN_10x4_12", "DSCNNSquareTiny"])
 def test_dscnn_classes_one_launch(hip, oracle, name, monkeypatch):
-    """With SMALL_HIP_ONE_LAUNCH=1 (or Model::set_one_launch(true)) the float32 DS-CNN classes run their whole pass as
+    """With SMALL_HIP_TUNE="one_launch=1" (or Model::set_one_launch(true)) the float32 DS-CNN classes run their whole pass as
     one launch (small_hip_fmodel_forward): within the float32 bar of the oracle and of the layer-by-layer result, which
     stays the default because callers compare a model with the layer functions bit for bit."""
     which, variant, fn, filters, shape = _model_case(name)
     x = synth.normal(57, int(np.prod(shape))).reshape(shape)
     layered = hip.model_f32(which, x, filters, variant)
-    monkeypatch.setenv("SMALL_HIP_ONE_LAUNCH", "1")
+    monkeypatch.setenv("SMALL_HIP_TUNE", "one_launch=1")
     got = hip.model_f32(which, x, filters, variant)
     assert_close_f32(got, fn(oracle, x, filters), what=name + " one launch vs oracle")
     assert_close_f32(got, layered, what=name + " one launch vs layer by layer")

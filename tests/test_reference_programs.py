@@ -37,7 +37,7 @@ STOPS_AT_MISSING_FILE = {"test_yolo": "in__yolo_Ci255_H76_W76_k0_s0_f_1472880.bi
 # test_tinyyolov2.cpp asserts that its Model / DAGModel objects and the same layers called one by one give
 # bit-identical outputs; here that holds when both issue the same launches, i.e. with the convolution + pooling
 # one-launch form switched off (with it on the two paths agree within the float32 tolerance: test_cpp_layers.py)
-ENV = {"test_tinyyolov2": {"SMALL_HIP_FUSE_POOL": "0"}}
+ENV = {"test_tinyyolov2": {"SMALL_HIP_TUNE": "fuse_pool=0"}}
 
 
 @pytest.mark.skipif(not (os.path.isdir(REF_TESTS) and os.path.exists(LIB)),
