@@ -87,6 +87,7 @@ struct QMHeader
     int n_layers;
     int filter_bytes;                    // LDS image of all prepared filters (blob offset 0 -> LDS offset 0)
     int first_bytes;                     // ... of which the first layer's (needed before anything else)
+    int later_kib;                       // KiB behind it that hold the later layers' filters (the last one rounded up)
     int in_C, in_H, in_W, in_off;        // the model input and the LDS offset it is staged at
     int tab_lds, tab_bytes, pool_off;    // LDS scratch: tables[2][tab_bytes], pooling sums
     int in_elems, out_elems;             // bytes per image in global memory
@@ -196,24 +197,29 @@ __device__ __forceinline__ void zero_ring(uint8_t *t, int Cb, int H, int W, int 
 // requant_u8's short form (positive multiplier) with the layer's constants hoisted, in signed arithmetic: a
 // non-positive accumulator gives v <= 0, the rounding shift keeps it <= 0 and the clamp returns 0, exactly as the
 // unsigned form's explicit test does; a positive one is the same computation.
+// The rounding term: the remainder v mod 2^rs exceeds (2^rs - 1) / 2 exactly when its top bit, bit rs - 1 of v, is set
+// (never for rs == 0): one bit-field extract instead of a mask, a compare and a carry.
 struct FastQ
 {
-    int32_t mult, mask, half;
-    int ls, rs;
+    int32_t mult;
+    int ls, rs, bit, width;              // bit = (rs - 1) & 31, width = rs > 0
 };
 __device__ __forceinline__ uint32_t requant_fast(int32_t acc, const FastQ f)
 {
     const int32_t shifted = (int32_t)((uint32_t)acc << f.ls);
     const long long prod = (long long)shifted * (long long)f.mult + (1ll << 30);
     const int32_t v = (int32_t)(prod >> 31);
-    const int32_t r = (v >> f.rs) - ((v & f.mask) > f.half ? 1 : 0);
+    const int32_t r = (v >> f.rs) - (int32_t)__builtin_amdgcn_ubfe((uint32_t)v, (uint32_t)f.bit, (uint32_t)f.width);
     return (uint32_t)(r < 0 ? 0 : (r > 255 ? 255 : r));      // v_med3_i32
 }
 
 // TP pixel tiles (16 pixels each) of one channel block per wave step, sharing the filter operand.
 // NM > 0: the layer has exactly NM MFMA steps (4 K-steps each), the loop is unrolled and the lane's K-step offsets
 // live in registers; NM == 0: any count, offsets read from the table per step.
-template <bool STEM, int TP, int NM, bool FAST>
+// POST: what follows the requantisation, fixed per instantiation so that the epilogue is straight-line code:
+// 0 nothing, 1 the byte goes through post[] (in-place ReLU), 2 Accum (+ ReLU): post[byte + shortcut byte], -1 decided per
+// layer at run time (the general form, also the only one that writes the model's output to global memory).
+template <bool STEM, int TP, int NM, bool FAST, int POST = -1>
 __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
                                            int n_waves)
 {
@@ -229,8 +235,7 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
     const int32_t *T = reinterpret_cast<const int32_t *>(tab);
     const int *steps = reinterpret_cast<const int *>(tab + 64 * L.Co);
     const uint8_t *post = tab + 64 * L.Co + 4 * L.S_pad;
-    const FastQ fq{L.q.multiplier, (int32_t)((1u << L.q.rshift) - 1u), (int32_t)(((1u << L.q.rshift) - 1u) >> 1), L.q.lshift & 31,
-                   L.q.rshift};
+    const FastQ fq{L.q.multiplier, L.q.lshift & 31, L.q.rshift, (L.q.rshift - 1) & 31, L.q.rshift > 0 ? 1 : 0};
     // the lane's K-steps: offset from the window origin, and the vector the box sum multiplies by (0 past the end:
     // such a step reads valid memory, its filter rows are zero, and it must not count towards the box sum)
     int so[NM > 0 ? NM : 1], ones[NM > 0 ? NM : 1];
@@ -265,10 +270,12 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
             ih0[t] = (oh[t] << s_shift) - L.pt;
             iw0[t] = (ow[t] << s_shift) - L.pl;
         }
-        v4i acc[TP];
-        int si[TP];
+        // si: the pixel's box sum, from the matrix pipe too (a filter block of ones: every row of the product is the sum
+        // of the pixel's bytes over all K-steps, so each lane finds its pixel's sum in its own registers; the pipe is
+        // idle most of the time here, the vector ALU is what these layers wait for)
+        v4i acc[TP], si[TP];
 #pragma unroll
-        for (int t = 0; t < TP; ++t) { acc[t] = v4i{0, 0, 0, 0}; si[t] = 0; }
+        for (int t = 0; t < TP; ++t) { acc[t] = v4i{0, 0, 0, 0}; si[t] = v4i{0, 0, 0, 0}; }
         if (STEM)
         {
             // one MFMA: K group g = window row g (kw pixels x 4 channels), rows >= kh are zero
@@ -284,10 +291,9 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
                     for (int j = 0; j < 4; ++j)
                         if (j < L.kw) b[j] = row[j];
                 }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) si[t] = sdot_ones(b[j], si[t]);
-                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w},
-                                                               v4i{(int)b[0], (int)b[1], (int)b[2], (int)b[3]}, acc[t], 0, 0, 0);
+                const v4i bv{(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+                si[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101}, bv, si[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w}, bv, acc[t], 0, 0, 0);
             }
         }
         else
@@ -305,12 +311,9 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
                     for (int t = 0; t < TP; ++t)
                     {
                         const uint4 B = *reinterpret_cast<const uint4 *>(pix[t] + so[m]);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.x, ones[m], si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.y, ones[m], si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.z, ones[m], si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.w, ones[m], si[t], false);
-                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w},
-                                                                       v4i{(int)B.x, (int)B.y, (int)B.z, (int)B.w}, acc[t], 0, 0, 0);
+                        const v4i bv{(int)B.x, (int)B.y, (int)B.z, (int)B.w};
+                        si[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{ones[m], ones[m], ones[m], ones[m]}, bv, si[t], 0, 0, 0);
+                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w}, bv, acc[t], 0, 0, 0);
                     }
                 }
             }
@@ -325,12 +328,9 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
                     for (int t = 0; t < TP; ++t)
                     {
                         const uint4 B = *reinterpret_cast<const uint4 *>(pix[t] + (sv >= 0 ? sv : 0));
-                        si[t] = __builtin_amdgcn_sdot4((int)B.x, one, si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.y, one, si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.z, one, si[t], false);
-                        si[t] = __builtin_amdgcn_sdot4((int)B.w, one, si[t], false);
-                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w},
-                                                                       v4i{(int)B.x, (int)B.y, (int)B.z, (int)B.w}, acc[t], 0, 0, 0);
+                        const v4i bv{(int)B.x, (int)B.y, (int)B.z, (int)B.w};
+                        si[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{one, one, one, one}, bv, si[t], 0, 0, 0);
+                        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)A.x, (int)A.y, (int)A.z, (int)A.w}, bv, acc[t], 0, 0, 0);
                     }
                 }
             }
@@ -338,10 +338,7 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
 #pragma unroll
         for (int t = 0; t < TP; ++t)
         {
-            // box sum of the pixel over the four K groups
-            int sit = si[t];
-            sit += __shfl_xor(sit, 16);
-            sit += __shfl_xor(sit, 32);
+            const int sit = si[t][0];
             if (!pvalid[t]) continue;
             // border case of the pixel -> T
             const int ra = (ih0[t] < 0 ? 2 : 0) + (ih0[t] + L.kh > L.H ? 1 : 0);
@@ -351,7 +348,9 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
             const uint32_t base = (uint32_t)L.ZF * (uint32_t)sit;
             const int opos = (__mul24(cob * Hop + oh[t] + 1, Wop) + ow[t] + 1) * 16 + 4 * grp;
             uint32_t packed = 0;
-            if (L.acc_off >= 0)
+            const bool with_acc = POST >= 0 ? POST == 2 : L.acc_off >= 0;
+            const bool with_post = POST >= 0 ? POST != 0 : L.has_post != 0;
+            if (with_acc)
             {
                 const uint32_t sc = *reinterpret_cast<const uint32_t *>(lds + L.acc_off + opos) ^ 0x80808080u;
 #pragma unroll
@@ -369,28 +368,39 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
                 {
                     const int32_t v = (int32_t)((uint32_t)acc[t][r] + base + tc4[r]);
                     uint32_t y = FAST ? requant_fast(v, fq) : requant_u8(v, L.q);
-                    if (L.has_post) y = post[y];
+                    if (with_post) y = post[y];
                     packed |= y << (8 * r);
                 }
             }
+            if (POST >= 0) { *reinterpret_cast<uint32_t *>(lds + L.dst_off + opos) = packed ^ 0x80808080u; continue; }
             if (L.dst_off >= 0) *reinterpret_cast<uint32_t *>(lds + L.dst_off + opos) = packed ^ 0x80808080u;
             else *reinterpret_cast<uint32_t *>(gout + ((size_t)(cob * L.Ho + oh[t]) * L.Wo + ow[t]) * 16 + 4 * grp) = packed;
         }
     }
 }
 
-template <bool STEM, int TP>
+template <bool STEM, int TP, int POST>
 __device__ __forceinline__ void conv_tiles_nm(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
                                               int n_waves)
 {
     // the step counts of 3x3 windows over 16, 32 and 64 channels and of 1x1 windows get unrolled loops
-    if (STEM) return conv_tiles<true, TP, 1, true>(L, lds, tab, gout, tid, wave, n_waves);
+    if (STEM) return conv_tiles<true, TP, 1, true, POST>(L, lds, tab, gout, tid, wave, n_waves);
     const int nm = L.S_pad >> 2;
-    if (nm == 1) conv_tiles<false, TP, 1, true>(L, lds, tab, gout, tid, wave, n_waves);
-    else if (nm == 3) conv_tiles<false, TP, 3, true>(L, lds, tab, gout, tid, wave, n_waves);
-    else if (nm == 5) conv_tiles<false, TP, 5, true>(L, lds, tab, gout, tid, wave, n_waves);
-    else if (nm == 9) conv_tiles<false, TP, 9, true>(L, lds, tab, gout, tid, wave, n_waves);
-    else conv_tiles<false, TP, 0, true>(L, lds, tab, gout, tid, wave, n_waves);
+    if (nm == 1) conv_tiles<false, TP, 1, true, POST>(L, lds, tab, gout, tid, wave, n_waves);
+    else if (nm == 3) conv_tiles<false, TP, 3, true, POST>(L, lds, tab, gout, tid, wave, n_waves);
+    else if (nm == 5) conv_tiles<false, TP, 5, true, POST>(L, lds, tab, gout, tid, wave, n_waves);
+    else if (nm == 9) conv_tiles<false, TP, 9, true, POST>(L, lds, tab, gout, tid, wave, n_waves);
+    else conv_tiles<false, TP, 0, true, -1>(L, lds, tab, gout, tid, wave, n_waves);
+}
+
+template <bool STEM, int TP>
+__device__ __forceinline__ void conv_tiles_post(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
+                                                int n_waves)
+{
+    if (L.dst_off < 0) conv_tiles<STEM, TP, STEM ? 1 : 0, true, -1>(L, lds, tab, gout, tid, wave, n_waves);   // the model's output
+    else if (L.acc_off >= 0) conv_tiles_nm<STEM, TP, 2>(L, lds, tab, gout, tid, wave, n_waves);
+    else if (L.has_post) conv_tiles_nm<STEM, TP, 1>(L, lds, tab, gout, tid, wave, n_waves);
+    else conv_tiles_nm<STEM, TP, 0>(L, lds, tab, gout, tid, wave, n_waves);
 }
 
 // waves [wave0, wave0 + n_waves) of the workgroup compute the layer (all 16 but for the first layer)
@@ -401,8 +411,8 @@ __device__ __forceinline__ void conv_layer(const QMLayer &L, uint8_t *lds, const
     const int n_tiles = ((L.Ho * L.Wo + 15) >> 4) * (L.Co / CB);
     if (L.q.fast)
     {
-        if (n_tiles >= 2 * n_waves) conv_tiles_nm<STEM, 2>(L, lds, tab, gout, tid, wave, n_waves);
-        else conv_tiles_nm<STEM, 1>(L, lds, tab, gout, tid, wave, n_waves);
+        if (n_tiles >= 2 * n_waves) conv_tiles_post<STEM, 2>(L, lds, tab, gout, tid, wave, n_waves);
+        else conv_tiles_post<STEM, 1>(L, lds, tab, gout, tid, wave, n_waves);
     }
     else
         conv_tiles<STEM, 1, 0, false>(L, lds, tab, gout, tid, wave, n_waves);   // any int32 multiplier: general requantisation
@@ -463,6 +473,16 @@ __global__ __launch_bounds__(NT) void qmodel_u8_kernel(const QMHeader *__restric
         if (tid < hdr->layer[0].tab16)
             reinterpret_cast<uint4 *>(lds + hdr->tab_lds)[tid] = reinterpret_cast<const uint4 *>(blob + hdr->layer[0].tab_off)[tid];
     }
+    // The filters of all later layers: requested now, by the memory pipeline itself (global memory to LDS without
+    // passing through registers, a wave moves one KiB per instruction), and awaited after the first layer has been
+    // computed by all sixteen waves: the copy costs the layer neither waves nor registers.
+    {
+        const int lane = tid & 63;
+        const int first = hdr->first_bytes, kib = hdr->later_kib;
+        for (int c = wave; c < kib; c += NW)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(blob + first + c * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + first + c * 1024), 16, 0, 0);
+    }
     // the image, re-biased, with its ring of zeros
     {
         const int C = hdr->in_C, H = hdr->in_H, W = hdr->in_W, Hp = H + 2, Wp = W + 2;
@@ -519,29 +539,11 @@ __global__ __launch_bounds__(NT) void qmodel_u8_kernel(const QMHeader *__restric
         else
         {
             if (L.dst_off >= 0) zero_ring(lds + L.dst_off, L.Co / CB, L.Ho, L.Wo, tid);
-            // The first layer is computed by half of the waves while the other half brings the filters of all later
-            // layers into LDS (device-memory latency, few instructions): the copy costs the layer nothing but the
-            // waves, and its registers are not live in the tile code.
-            int w0 = wave, nw = NW;
-            if (li == 0 && n_layers > 1)
-            {
-                nw = NW / 2;
-                if (wave >= nw)
-                {
-                    const uint4 *s = reinterpret_cast<const uint4 *>(blob);
-                    uint4 *d = reinterpret_cast<uint4 *>(lds);
-                    const int n16 = hdr->filter_bytes >> 4;
-                    for (int i = (hdr->first_bytes >> 4) + tid - nw * WAVE; i < n16; i += NT - nw * WAVE) d[i] = s[i];
-                    w0 = -1;
-                }
-            }
-            if (w0 >= 0)
-            {
-                if (L.kind == K_STEM) conv_layer<true>(L, lds, tab, gout, tid, w0, nw);
-                else conv_layer<false>(L, lds, tab, gout, tid, w0, nw);
-            }
+            if (L.kind == K_STEM) conv_layer<true>(L, lds, tab, gout, tid, wave, NW);
+            else conv_layer<false>(L, lds, tab, gout, tid, wave, NW);
         }
         if (tid < next_tab16) reinterpret_cast<uint4 *>(tabs + nxt * tab_bytes)[tid] = tpre;
+        if (li == 0) __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this wave's share of the later layers' filters has landed
         __syncthreads();
     }
 }
@@ -703,9 +705,11 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
         { set_error("%s: layer %d: Accum source has another shape", op, i); return fail(SMALL_HIP_EINVAL); }
     }
 
-    // LDS plan: [filters][tables x2][pooling sums][input][tensors]
+    // LDS plan: [filters][tables x2][pooling sums][input][tensors]; the later layers' filters are copied in whole KiB
     h.filter_bytes = lds_filters;
-    int off = align_up(lds_filters, 16);
+    h.later_kib = (lds_filters - h.first_bytes + 1023) >> 10;
+    const int filters_end = h.first_bytes + (h.later_kib << 10);
+    int off = align_up(filters_end, 16);
     h.tab_lds = off; h.tab_bytes = max_t; off += 2 * max_t;
     int pool_c = 0;
     for (int i = 0; i < n_layers; ++i)
@@ -725,7 +729,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
                   lds_filters, LDS_LIMIT);
         return fail(SMALL_HIP_EINVAL);
     }
-    const int table_base = align_up(lds_filters, 256);
+    const int table_base = align_up(filters_end, 256);      // the copy reads the blob up to filters_end
     for (int i = 0; i < n_layers; ++i)
     {
         QMLayer &L = h.layer[i];

@@ -57,8 +57,9 @@ __host__ __device__ __forceinline__ uint32_t requant_u8(int32_t acc, const QOut 
         const int32_t shifted = (int32_t)((uint32_t)acc << (q.lshift & 31));
         const uint64_t prod = (uint64_t)(uint32_t)shifted * (uint64_t)(uint32_t)q.multiplier + (1ull << 30);
         const uint32_t v = (uint32_t)(prod >> 31);
-        const uint32_t mask = (1u << q.rshift) - 1u;
-        const int32_t r = (int32_t)(v >> q.rshift) - ((v & mask) > (mask >> 1) ? 1 : 0);   // -1 is possible
+        // (v mod 2^rshift) > (2^rshift - 1) / 2 exactly when bit rshift - 1 of v is set (never for rshift == 0)
+        const uint32_t round_bit = (v >> ((q.rshift - 1) & 31)) & (q.rshift > 0 ? 1u : 0u);
+        const int32_t r = (int32_t)(v >> q.rshift) - (int32_t)round_bit;   // -1 is possible
         const int32_t c = r < 0 ? 0 : (r > 255 ? 255 : r);
         return shifted > 0 ? (uint32_t)c : 0u;
     }
