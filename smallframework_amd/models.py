@@ -702,15 +702,22 @@ class HipExecutor:
             (self.lib.small_hip_qmodel_destroy if self.model.dtype == "u8" else self.lib.small_hip_fmodel_destroy)(self.qmodel)
             self.qmodel = None
 
-    def capture(self):
+    def capture(self, one_launch=False):
         """Record one forward pass into a HIP graph (the launches go to the capture stream through the
-        same C ABI calls).  Needs the prepared-filter path for uint8 models: capture must not allocate."""
+        same C ABI calls).  Needs the prepared-filter path for uint8 models: capture must not allocate.
+        one_launch: record forward_one_launch() instead of the layer-by-layer pass."""
         torch = self.torch
-        self.forward()                      # warm up outside the capture (lazy module loading)
+        step = self.forward_one_launch if one_launch else self.forward
+        # Warm up on the stream the capture will use: the library's scratch blocks belong to a (device, stream) pair and
+        # are allocated by the first call that needs them, which must not happen under capture.
+        self.graph_stream = torch.cuda.Stream()
+        self.graph_stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(self.graph_stream):
+            step()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            self.forward()
+        with torch.cuda.graph(g, stream=self.graph_stream):
+            step()
         self.graph = g
         return g
 

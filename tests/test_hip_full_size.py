@@ -70,9 +70,12 @@ def test_tiny_yolo_v2_batch16():
     assert_close_f32(got[:1], want, atol=1e-5 * max(1.0, float(np.abs(want).max())), what="tiny_yolo_v2 b16 image 0")
 
 
+@pytest.mark.parametrize("disc", [True, False], ids=["discriminating", "config"])
 @pytest.mark.parametrize("prepared", [True, False], ids=["prepared", "direct"])
-def test_resnet8_u8_batch256(prepared):
-    m = models.resnet8_u8(discriminating=True)
+def test_resnet8_u8_batch256(prepared, disc):
+    """Layer by layer at the configuration's batch: the variant whose logits depend on the data, and the configuration
+    as it is written (its requantisation saturates most activations; it is the one the metric names)."""
+    m = models.resnet8_u8(discriminating=disc)
     got, want = _tiled_run(m, 256, 4, prepared=prepared)
     _check_replicas(got, 4, "resnet8_u8 b256", exact=True)
     assert_equal_exact(got[:4], want, "resnet8_u8 b256 images 0..3")

@@ -164,10 +164,12 @@ def test_layer_sweep_batch1(m):
         assert_close_f32(got, want, what=m.name)
 
 
-@pytest.mark.parametrize("name,batch", [("resnet8_u8", 4), ("dscnn", 2)])
+@pytest.mark.parametrize("name,batch", [("resnet8_u8", 4), ("dscnn", 2), ("tiny_yolo_v2", 16), ("mobilenet_v1", 8)])
 def test_hip_graph_replays_match_eager(name, batch):
     """A captured forward pass must reproduce the eager result on every replay, with eager work and
-    synchronisations between the replays."""
+    synchronisations between the replays.  Tiny-YOLOv2 at batch 16 runs its 13x13 layers through the equal-share split,
+    whose partial sums live in a library-owned scratch block: the block the graph captured must be the one later eager
+    calls use too, and must still be there."""
     import torch
     m = getattr(models, name)(discriminating=True) if name == "resnet8_u8" else getattr(models, name)()
     w = models.make_weights(m)
@@ -176,6 +178,16 @@ def test_hip_graph_replays_match_eager(name, batch):
     ex.forward()
     eager = ex.output().copy()
     ex.capture()
+    if name == "tiny_yolo_v2":
+        # a larger request on the captured stream makes the library take a new scratch block; the one the graph holds
+        # stays allocated (nothing is freed before small_hip_workspace_release)
+        import ctypes as C
+        from smallframework_amd import capi
+        lib = capi.load()
+        held = lib.small_hip_workspace_held()
+        assert held >= lib.small_hip_conv2d_f32_workspace_bytes(16, 3, 3, 1, 1, 1, 1, 1, 1024, 1024, 13, 13) > 0
+        capi.check(lib.small_hip_workspace_reserve(2 * held, C.c_void_p(ex.graph_stream.cuda_stream)))
+        assert lib.small_hip_workspace_held() >= 3 * held - (1 << 21)
     for rep in range(4):
         # different input every replay so a stale result cannot pass
         xr = models.make_input(m, batch, seed=200 + rep)

@@ -73,3 +73,49 @@ def test_one_launch_repeats_bit_for_bit(name, batch):
         again = ex.output_one_launch()
         assert np.array_equal(again.view(np.uint8), first.view(np.uint8)), "launch %d differs from the first" % (i + 2)
     ex.close()
+
+
+@pytest.mark.parametrize("disc", [False, True], ids=["config", "discriminating"])
+@pytest.mark.parametrize("batch", [64, 256])
+def test_resnet8_u8_one_launch_at_the_benchmark_batches(disc, batch):
+    """The launch bench.py reports (batch 64 and 256), on a batch tiled from four distinct images: the four against the
+    oracle, every copy against its source, bit for bit."""
+    m = models.resnet8_u8(discriminating=disc)
+    w = models.make_weights(m)
+    distinct = 4
+    x = models.make_input(m, distinct, seed=31)
+    per = x.size // distinct
+    xt = np.ascontiguousarray(np.tile(x.reshape(distinct, per), (batch // distinct, 1))).ravel()
+    ex = models.HipExecutor(m, batch, w, xt)
+    ex.build_one_launch()
+    ex.forward_one_launch()
+    got = ex.output_one_launch().reshape(batch, -1).copy()
+    ex.close()
+    want = OracleExecutor(m, distinct, w, x).forward().reshape(distinct, -1)
+    assert_equal_exact(got[:distinct], want, "one launch, batch %d, images 0..3 vs oracle" % batch)
+    for i in range(distinct, batch):
+        assert_equal_exact(got[i], got[i % distinct], "one launch, batch %d: image %d vs its source" % (batch, i))
+    if disc:
+        assert len(np.unique(want)) > 1
+
+
+@pytest.mark.parametrize("name,batch", [("resnet8_u8", 8), ("dscnn", 4)])
+def test_one_launch_graph_replays_match_eager(name, batch):
+    """small_hip_qmodel_forward / small_hip_fmodel_forward recorded into a HIP graph: every replay, with eager launches
+    and synchronisations in between and another input each time, reproduces the eager launch bit for bit."""
+    import torch
+    m = models.resnet8_u8(discriminating=True) if name == "resnet8_u8" else models.dscnn()
+    ex = models.HipExecutor(m, batch, models.make_weights(m), models.make_input(m, batch))
+    ex.build_one_launch()
+    ex.capture(one_launch=True)
+    for rep in range(4):
+        xr = models.make_input(m, batch, seed=300 + rep)
+        ex.buf["in"].copy_(torch.from_numpy(xr))
+        ex.replay()
+        got = ex.output_one_launch().copy()
+        ex.one_out.zero_()
+        ex.forward_one_launch()
+        want = ex.output_one_launch().copy()
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "graph replay %d differs from the eager launch" % rep
+        assert np.unique(want.view(np.uint8)).size > 1
+    ex.close()
