@@ -4,6 +4,7 @@
 
 #include <cstdlib>
 #include <memory>
+#include <string>
 #include <type_traits>
 #include <vector>
 
@@ -49,6 +50,9 @@ public:
     void set_one_launch(bool on) { m_one_launch = on; }
     // true once inference() has planned (and used) the one-launch form
     bool one_launch_planned() const { return m_qmodel != nullptr || m_fmodel != nullptr; }
+    // why the whole-model launch was not planned (the library's message: which limit the model exceeds); empty if it was,
+    // or was never asked for.  Only "not built for this model" falls back to the layer calls; a bad argument throws.
+    std::string const &one_launch_refusal() const { return m_refusal; }
 
     shape_type const &get_input_shape() const { return m_input_shape; }
 
@@ -121,12 +125,13 @@ protected:
                 m_qsig = sig;
                 if (m_qrefused == sig) return false;
                 const int rc = small_hip_qmodel_create((int)recs.size(), recs.data(), &m_qmodel, detail::current_stream());
-                if (rc == SMALL_HIP_EINVAL || rc == SMALL_HIP_ECHANNELS || rc == SMALL_HIP_ESTRIDE)
+                if (rc == SMALL_HIP_EUNSUPPORTED)
                 {
-                    m_qrefused = sig;         // does not fit: not an error, and not worth asking again
+                    m_qrefused = sig;         // does not fit one launch: not an error, and not worth asking again
+                    m_refusal = small_hip_last_error();
                     return false;
                 }
-                detail::hip_check(rc, "small_hip_qmodel_create");
+                detail::hip_check(rc, "small_hip_qmodel_create");     // anything else is a genuine error: raised
             }
             Tensor<BufferT> *out = steps.back().dst;
             if (out->capacity() < steps.back().layer->output_size())
@@ -160,12 +165,13 @@ protected:
                     recs[i].dst = i + 1 == steps.size() ? SMALL_HIP_QM_OUTPUT : dst;
                 }
                 const int rc = small_hip_fmodel_create((int)recs.size(), recs.data(), &m_fmodel, detail::current_stream());
-                if (rc == SMALL_HIP_EINVAL || rc == SMALL_HIP_ECHANNELS || rc == SMALL_HIP_ESTRIDE)
+                if (rc == SMALL_HIP_EUNSUPPORTED)
                 {
-                    m_frefused = true;        // does not fit: not an error, and not worth asking again
+                    m_frefused = true;        // does not fit one launch: not an error, and not worth asking again
+                    m_refusal = small_hip_last_error();
                     return false;
                 }
-                detail::hip_check(rc, "small_hip_fmodel_create");
+                detail::hip_check(rc, "small_hip_fmodel_create");     // anything else is a genuine error: raised
             }
             Tensor<BufferT> *out = steps.back().dst;
             if (out->capacity() < steps.back().layer->output_size())
@@ -196,6 +202,7 @@ private:
     std::vector<int32_t> m_qsig, m_qrefused;
     small_hip_fmodel *m_fmodel = nullptr;
     bool m_frefused = false;
+    std::string m_refusal;
 };
 
 } // namespace small

@@ -46,6 +46,9 @@ extern "C" {
 #define SMALL_HIP_EINVAL 4    /* null / misaligned pointer, non-positive size, Co % 16 != 0 */
 #define SMALL_HIP_EHIP 5      /* a HIP runtime call failed; see small_hip_last_error() */
 #define SMALL_HIP_ENOMEM 6
+#define SMALL_HIP_EUNSUPPORTED 7 /* valid arguments that a specialised entry point is not built for (a model too
+                                    large for one compute unit's LDS, a layer shape outside the whole-model kernels):
+                                    use the general path; small_hip_last_error() says which limit was hit */
 
 #define SMALL_HIP_ACT_NONE 0
 #define SMALL_HIP_ACT_RELU 1

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libsmall_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "small_hip.h")
 
 CB = 16
-OK, ESTRIDE, ECHANNELS, ESCALE, EINVAL, EHIP, ENOMEM = range(7)
+OK, ESTRIDE, ECHANNELS, ESCALE, EINVAL, EHIP, ENOMEM, EUNSUPPORTED = range(8)
 ACT_NONE, ACT_RELU, ACT_LEAKY = 0, 1, 2
 
 
@@ -170,7 +170,7 @@ def check(status):
     """Raise SmallHipError for a non-zero status."""
     if status != OK:
         lib = load()
-        msg = lib.small_hip_last_error().decode() if status in (EINVAL, EHIP, ENOMEM) else \
+        msg = lib.small_hip_last_error().decode() if status in (EINVAL, EHIP, ENOMEM, EUNSUPPORTED) else \
             lib.small_hip_strerror(status).decode()
         raise SmallHipError(status, msg)
     return status

@@ -709,10 +709,10 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
         L.nscale = 1.f;
         if (pool)
         {
-            if (Ci % CB != 0 || Ci / 4 > NT) return fail(SMALL_HIP_ECHANNELS);
+            if (Ci % CB != 0 || Ci / 4 > NT) { set_error("%s: layer %d: pooling over %d channels", op, i, Ci); return fail(SMALL_HIP_EUNSUPPORTED); }
             if (l.kernel_height != H || l.kernel_width != W || l.t_pad || l.b_pad || l.l_pad || l.r_pad || from_input ||
                 l.act != SMALL_HIP_ACT_NONE)
-            { set_error("%s: layer %d: only whole-image pooling without padding or activation, after another layer", op, i); return fail(SMALL_HIP_EINVAL); }
+            { set_error("%s: layer %d: only whole-image pooling without padding or activation, after another layer", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
             L.kind = l.kind == SMALL_HIP_FL_GLOBAL_AVGPOOL ? K_POOL_AVG : K_POOL_MAX;
             L.Co = Ci; L.Ho = 1; L.Wo = 1; L.kh = H; L.kw = W; L.stride = 1;
             L.norm = (float)(1.0 / ((double)H * W));
@@ -724,10 +724,10 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
             const bool dw = l.kind == SMALL_HIP_FL_DWCONV;
             const int Co = dw ? Ci : l.output_channels;
             const bool stem = !dw && Ci < CB;
-            if (stem ? !(Ci >= 1 && Ci <= 3) : Ci % CB != 0) return fail(SMALL_HIP_ECHANNELS);
-            if (stem && !from_input) { set_error("%s: layer %d: 1..3 input channels only on the model input", op, i); return fail(SMALL_HIP_EINVAL); }
-            if (dw && from_input) { set_error("%s: layer %d: the first layer must be a convolution", op, i); return fail(SMALL_HIP_EINVAL); }
-            if (s != 1 && s != 2) return fail(SMALL_HIP_ESTRIDE);
+            if (stem ? !(Ci >= 1 && Ci <= 3) : Ci % CB != 0) { set_error("%s: layer %d: %d input channels", op, i, Ci); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (stem && !from_input) { set_error("%s: layer %d: 1..3 input channels only on the model input", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (dw && from_input) { set_error("%s: layer %d: the first layer must be a convolution", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (s != 1 && s != 2) { set_error("%s: layer %d: stride %d", op, i, s); return fail(SMALL_HIP_EUNSUPPORTED); }
             if (kh <= 0 || kw <= 0 || kh > 255 || kw > 255 || Co <= 0 || Co % CB != 0 || !l.filter || !aligned16(l.filter) ||
                 (l.bias && !aligned16(l.bias)) || !pads_ok(l.t_pad, l.b_pad, l.l_pad, l.r_pad))
             { set_error("%s: layer %d: bad convolution arguments", op, i); return fail(SMALL_HIP_EINVAL); }
@@ -749,7 +749,7 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
             else wf = (long)Co * Ci * taps;
             long bf = wf + Co + (stem ? L.chunks * 16 : 0);
             bf = (bf + 3) & ~3L;
-            if (bf > (long)NPRE * NT * 4) { set_error("%s: layer %d: more than %d KB of weights", op, i, NPRE * NT * 16 / 1024); return fail(SMALL_HIP_EINVAL); }
+            if (bf > (long)NPRE * NT * 4) { set_error("%s: layer %d: more than %d KB of weights", op, i, NPRE * NT * 16 / 1024); return fail(SMALL_HIP_EUNSUPPORTED); }
             w_floats[(size_t)i] = (int)wf;
             L.bias_off = (int)wf;
             L.ktab_off = (int)wf + Co;
@@ -761,7 +761,7 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
         L.r_cob = 1.0f / (float)(L.Co / CB);
         L.r_p = 1.0f / (float)(L.Ho * L.Wo);
         if ((long)L.Co * L.Ho * L.Wo > LDS_LIMIT / 4)
-        { set_error("%s: layer %d: output tensor larger than LDS", op, i); return fail(SMALL_HIP_EINVAL); }
+        { set_error("%s: layer %d: output tensor larger than LDS", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
         if (l.dst >= 0) written_by[l.dst] = i;
     }
 
@@ -846,7 +846,7 @@ int small_hip_fmodel_create(int n_layers, const small_hip_flayer *layers, small_
     {
         set_error("%s: the model needs %ld bytes of LDS (activations %ld, weights of two layers %d), the limit is %d: run it "
                   "layer by layer", op, (long)off * 4, (long)(off - h.in_off) * 4, 2 * max_blob * 4, LDS_LIMIT);
-        return fail(SMALL_HIP_EINVAL);
+        return fail(SMALL_HIP_EUNSUPPORTED);
     }
     for (int i = 0; i < n_dev; ++i)
     {

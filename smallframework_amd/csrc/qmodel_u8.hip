@@ -621,10 +621,10 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
         L.acc_off = -1;
         if (pool)
         {
-            if (Ci % CB != 0 || Ci > NT) return fail(SMALL_HIP_ECHANNELS);
+            if (Ci % CB != 0 || Ci > NT) { set_error("%s: layer %d: pooling over %d channels", op, i, Ci); return fail(SMALL_HIP_EUNSUPPORTED); }
             if (l.kernel_height != H || l.kernel_width != W || l.t_pad || l.b_pad || l.l_pad || l.r_pad || l.relu ||
                 l.accum_src != SMALL_HIP_QM_NONE || from_input)
-            { set_error("%s: layer %d: only whole-image pooling without padding, after a convolution", op, i); return fail(SMALL_HIP_EINVAL); }
+            { set_error("%s: layer %d: only whole-image pooling without padding, after a convolution", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
             L.kind = l.kind == SMALL_HIP_QL_GLOBAL_AVGPOOL ? K_POOL_AVG : K_POOL_MAX;
             L.Co = Ci; L.Ho = 1; L.Wo = 1; L.kh = H; L.kw = W; L.stride = 1;
             L.zI = l.input_q.zero;
@@ -633,24 +633,25 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
         {
             const int kh = l.kernel_height, kw = l.kernel_width, s = l.stride, Co = l.output_channels;
             const bool stem = Ci < CB;
-            if (stem ? !(Ci >= 1 && Ci <= 3) : Ci % CB != 0) return fail(SMALL_HIP_ECHANNELS);
-            if (stem && !from_input) { set_error("%s: layer %d: 1..3 input channels only on the model input", op, i); return fail(SMALL_HIP_EINVAL); }
-            if (s != 1 && s != 2) return fail(SMALL_HIP_ESTRIDE);
-            if (kh <= 0 || kw <= 0 || Co <= 0 || Co % CB != 0 || Co > MAX_CO || !l.filter || !aligned16(l.filter) ||
+            if (stem ? !(Ci >= 1 && Ci <= 3) : Ci % CB != 0) { set_error("%s: layer %d: %d input channels", op, i, Ci); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (stem && !from_input) { set_error("%s: layer %d: 1..3 input channels only on the model input", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (s != 1 && s != 2) { set_error("%s: layer %d: stride %d", op, i, s); return fail(SMALL_HIP_EUNSUPPORTED); }
+            if (kh <= 0 || kw <= 0 || Co <= 0 || Co % CB != 0 || !l.filter || !aligned16(l.filter) ||
                 !pads_ok(l.t_pad, l.b_pad, l.l_pad, l.r_pad))
-            { set_error("%s: layer %d: bad convolution arguments (output channels: multiples of 16 up to %d)", op, i, MAX_CO); return fail(SMALL_HIP_EINVAL); }
+            { set_error("%s: layer %d: bad convolution arguments (output channels: multiples of 16)", op, i); return fail(SMALL_HIP_EINVAL); }
+            if (Co > MAX_CO) { set_error("%s: layer %d: more than %d output channels", op, i, MAX_CO); return fail(SMALL_HIP_EUNSUPPORTED); }
             if (stem && (kh > 4 || kw > 4))
-            { set_error("%s: layer %d: first-layer windows up to 4x4", op, i); return fail(SMALL_HIP_EINVAL); }
+            { set_error("%s: layer %d: first-layer windows up to 4x4", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
             const int Ho = out_dim(H, l.t_pad, l.b_pad, kh, s), Wo = out_dim(W, l.l_pad, l.r_pad, kw, s);
             if (Ho <= 0 || Wo <= 0) { set_error("%s: layer %d: empty output", op, i); return fail(SMALL_HIP_EINVAL); }
             // the tensors carry a ring of one pixel: no tap may fall further outside the image
             if (l.t_pad > 1 || l.l_pad > 1 || (Ho - 1) * s + kh - 1 - l.t_pad > H || (Wo - 1) * s + kw - 1 - l.l_pad > W)
-            { set_error("%s: layer %d: padding beyond one pixel", op, i); return fail(SMALL_HIP_EINVAL); }
+            { set_error("%s: layer %d: padding beyond one pixel", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
             L.kind = stem ? K_STEM : K_CONV;
             L.Co = Co; L.Ho = Ho; L.Wo = Wo; L.kh = kh; L.kw = kw; L.stride = s; L.pt = l.t_pad; L.pl = l.l_pad;
             const int S = stem ? 4 : kh * kw * (Ci / CB);
             L.S_pad = (S + 3) & ~3;
-            if (L.S_pad > MAX_STEPS) { set_error("%s: layer %d: window x channels too large", op, i); return fail(SMALL_HIP_EINVAL); }
+            if (L.S_pad > MAX_STEPS) { set_error("%s: layer %d: window x channels too large", op, i); return fail(SMALL_HIP_EUNSUPPORTED); }
             ZI[(size_t)i] = (int32_t)((uint32_t)l.input_q.zero + 128u);
             L.ZF = (int32_t)((uint32_t)l.filter_q.zero + 128u);
             L.w_off = lds_filters;
@@ -727,7 +728,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
     {
         set_error("%s: the model needs %d bytes of LDS (filters %d), the limit is %d: run it layer by layer", op, off,
                   lds_filters, LDS_LIMIT);
-        return fail(SMALL_HIP_EINVAL);
+        return fail(SMALL_HIP_EUNSUPPORTED);
     }
     const int table_base = align_up(filters_end, 256);      // the copy reads the blob up to filters_end
     for (int i = 0; i < n_layers; ++i)

@@ -113,6 +113,7 @@ const char *small_hip_strerror(int status)
     case SMALL_HIP_EINVAL: return "invalid argument";
     case SMALL_HIP_EHIP: return "HIP runtime error";
     case SMALL_HIP_ENOMEM: return "out of memory";
+    case SMALL_HIP_EUNSUPPORTED: return "not built for this shape: use the general path";
     default: return "unknown status";
     }
 }

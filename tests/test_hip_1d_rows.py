@@ -2,7 +2,9 @@
 moves by `stride` along the width only, every row an independent signal (reference: interface_abstract_1D.hpp, whose
 batch_size argument is the row count).  Checked through the C ABI against the same library's 2-D entry point called
 row by row on the extracted row (one row: the 2-D and the 1-D function coincide), which test_hip_parity.py holds
-against the oracle; float32 convolutions within the float32 bar, everything else bit for bit."""
+against the oracle; float32 convolutions within the float32 bar, everything else bit for bit.  The row layout
+[C/16][rows][W][16] and the grouped form's slab order are pinned separately against the CPU oracle applied row by row
+(test_rows_against_the_oracle): a layout mistake shared by the 1-D and the 2-D entry points would not pass that."""
 import numpy as np
 import pytest
 
@@ -139,3 +141,66 @@ def test_conv1d_u8_rows(lib, case, groups):
     want = _stack(outs, batch, G * Co, rows, Wo)
     assert_equal_exact(hu.host(do), want, "conv1d u8 rows %s groups=%d" % (case, groups))
     assert len(np.unique(want)) > 4, "saturated: the case does not discriminate"
+
+
+@pytest.mark.parametrize("case", CASES, ids=str)
+def test_rows_against_the_oracle(lib, oracle, case):
+    """The CPU oracle (pinned against the reference's scalar build, whose 1-D functions take the row count as their
+    batch_size) on every row by itself, rows gathered and scattered with numpy: convolution, grouped convolution,
+    max-pooling and the quantised convolution of the multi-row stride-2 entry points."""
+    from oracle.binding import quant
+    batch, k, s, l, r, Co, Ci, rows, W = case
+    Wo = 1 + (W + l + r - k) // s
+    # convolution + bias + ReLU
+    x = synth.normal(11, batch * Ci * rows * W)
+    f = synth.he_normal(12, Co * Ci * k, Ci * k)
+    bias = synth.normal(13, Co)
+    do = hu.dev_empty(batch * Co * rows * Wo, np.float32)
+    assert lib.small_hip_conv1d_f32(batch, k, s, l, r, 0, Co, Ci, rows, W, hu.ptr(hu.dev(x)), hu.ptr(hu.dev(f)), hu.ptr(hu.dev(bias)),
+                                    capi.ACT_RELU, 0.0, 0, hu.ptr(do), hu.stream()) == 0, lib.small_hip_last_error()
+    outs = []
+    for xr in _rows(x, batch, Ci, rows, W):
+        rc, o = oracle.conv2d_bias_act_f32(batch, CB, 1, k, s, 0, 0, l, r, Co, Ci, 1, W, xr, f, bias, capi.ACT_RELU, 0.0)
+        assert rc == 0
+        outs.append(o)
+    want = _stack(outs, batch, Co, rows, Wo)
+    assert_close_f32(hu.host(do), want, what="conv1d rows vs oracle %s" % (case,))
+    assert np.abs(want).max() > 0.1
+    # grouped: two groups of Ci -> Ci
+    G = 2
+    xg = synth.normal(14, batch * G * Ci * rows * W)
+    fg = synth.he_normal(15, G * Ci * Ci * k, Ci * k)
+    dog = hu.dev_empty(batch * G * Ci * rows * Wo, np.float32)
+    assert lib.small_hip_conv1d_f32(batch, k, s, l, r, G, Ci, Ci, rows, W, hu.ptr(hu.dev(xg)), hu.ptr(hu.dev(fg)), None,
+                                    capi.ACT_NONE, 0.0, 0, hu.ptr(dog), hu.stream()) == 0, lib.small_hip_last_error()
+    outs = []
+    for xr in _rows(xg, batch, G * Ci, rows, W):
+        rc, o = oracle.group_conv2d_f32(batch, CB, 1, k, s, 0, 0, l, r, G, Ci, 1, W, xr, fg)
+        assert rc == 0
+        outs.append(o)
+    assert_close_f32(hu.host(dog), _stack(outs, batch, G * Ci, rows, Wo), what="grouped conv1d rows vs oracle %s" % (case,))
+    # max-pooling
+    dop = hu.dev_empty(batch * Ci * rows * Wo, np.float32)
+    assert lib.small_hip_pool1d_f32(1, batch, k, s, l, r, Ci, rows, W, hu.ptr(hu.dev(x)), hu.ptr(dop), hu.stream()) == 0
+    outs = []
+    for xr in _rows(x, batch, Ci, rows, W):
+        rc, o = oracle.maxpool2d_f32(batch, CB, 1, k, s, 0, 0, l, r, Ci, 1, W, xr)
+        assert rc == 0
+        outs.append(o)
+    assert_equal_exact(hu.host(dop), _stack(outs, batch, Ci, rows, Wo), "maxpool1d rows vs oracle %s" % (case,))
+    # quantised convolution
+    xq = synth.uniform_u8(16, batch * Ci * rows * W)
+    fq_ = synth.uniform_u8(17, Co * Ci * k)
+    iq, fq, oq = hu.q(-120, 1 << 30, 0, 0), hu.q(-131, 1 << 30, 0, 0), hu.q(5, (1 << 30) + 4321, 0, 9)
+    doq = hu.dev_empty(batch * Co * rows * Wo, np.uint8)
+    assert lib.small_hip_conv1d_u8(batch, k, s, l, r, 0, Co, Ci, rows, W, hu.ptr(hu.dev(xq)), hu.qref(iq), hu.ptr(hu.dev(fq_)),
+                                   hu.qref(fq), hu.ptr(doq), hu.qref(oq), hu.stream()) == 0, lib.small_hip_last_error()
+    outs = []
+    for xr in _rows(xq, batch, Ci, rows, W):
+        rc, o = oracle.conv2d_u8(batch, CB, 1, k, s, 0, 0, l, r, Co, Ci, 1, W, xr, quant(-120, 1 << 30, 0, 0), fq_,
+                                 quant(-131, 1 << 30, 0, 0), quant(5, (1 << 30) + 4321, 0, 9))
+        assert rc == 0
+        outs.append(o)
+    wq = _stack(outs, batch, Co, rows, Wo)
+    assert_equal_exact(hu.host(doq), wq, "conv1d u8 rows vs oracle %s" % (case,))
+    assert len(np.unique(wq)) > 4

@@ -50,12 +50,21 @@ def test_dscnn_f32_one_launch(batch):
 
 
 def test_fmodel_refuses_what_does_not_fit():
-    """Tiny-YOLOv2's tensors do not fit LDS: creation is refused with EINVAL and a message, nothing is launched."""
+    """Tiny-YOLOv2's tensors do not fit LDS: creation is refused with EUNSUPPORTED (use the layer path) and a message that
+    names the limit; nothing is launched.  A bad argument is another status."""
     m = models.tiny_yolo_v2()
     ex = models.HipExecutor(m, 1)
     with pytest.raises(capi.SmallHipError) as e:
         ex.build_one_launch()
-    assert e.value.status == capi.EINVAL
+    assert e.value.status == capi.EUNSUPPORTED and "LDS" in str(e.value)
+    ex.close()
+    # a genuine argument error (a misaligned filter pointer) is EINVAL, not a quiet fall-back
+    m = models.dscnn()
+    ex = models.HipExecutor(m, 1)
+    layers = ex.fmodel_layers()
+    layers[1].filter = layers[1].filter + 4
+    h = C.c_void_p()
+    assert ex.lib.small_hip_fmodel_create(len(layers), layers, C.byref(h), ex.stream()) == capi.EINVAL
     ex.close()
 
 

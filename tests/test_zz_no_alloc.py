@@ -73,3 +73,45 @@ def test_noalloc_small_channel_stem_and_limits(lib, oracle):
                                          hu.qref(q), hu.ptr(hu.dev_empty(1024, np.uint8)), hu.qref(q), hu.stream())
     assert rc == capi.EINVAL
     assert b"static scratch" in lib.small_hip_last_error()
+
+
+def test_noalloc_under_graph_capture(lib, oracle):
+    """The use the entry point exists for: recorded into a HIP graph (capture forbids hipMalloc), replayed several times
+    with eager calls on the same array and synchronisations in between, another input every time."""
+    import torch
+    batch, kh, kw, s, (pt, pb, pl, pr), Co, Ci, H, W = 2, 3, 3, 1, (1, 1, 1, 1), 48, 32, 14, 14
+    args = (batch, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W)
+    iq, fq, oq = hu.q(-120), hu.q(-131), hu.q(5, 1518500250, 0, 8)
+    f = synth.uniform_u8(7, Co * Ci * kh * kw)
+    df = hu.dev(f)
+    dx = hu.dev(synth.uniform_u8(8, batch * Ci * H * W))
+    n = batch * Co * H * W
+    d_graph, d_eager = hu.dev_empty(n, np.uint8), hu.dev_empty(n, np.uint8)
+
+    def call(dst):
+        rc = lib.small_hip_conv2d_u8_noalloc(*args, hu.ptr(dx), hu.qref(iq), hu.ptr(df), hu.qref(fq), hu.ptr(dst), hu.qref(oq),
+                                             hu.stream())
+        assert rc == 0, lib.small_hip_last_error()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(d_graph)                        # module loading and the symbol lookup happen outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        call(d_graph)
+    for rep in range(3):
+        x = synth.uniform_u8(20 + rep, batch * Ci * H * W)
+        dx.copy_(torch.from_numpy(x))
+        d_graph.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = hu.host(d_graph)
+        call(d_eager)                        # an eager call re-writes the shared array between the replays
+        assert_equal_exact(got, hu.host(d_eager), "graph replay %d vs eager" % rep)
+        rco, want = oracle.conv2d_u8(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, _oq(iq), f, _oq(fq), _oq(oq))
+        assert rco == 0
+        assert_equal_exact(got, want, "graph replay %d vs oracle" % rep)
+        assert len(np.unique(want)) > 20
