@@ -76,7 +76,7 @@ class MirroredStorage
 public:
     MirroredStorage() = default;
     explicit MirroredStorage(size_t n) : m_n(n) { allocate(); }
-    MirroredStorage(MirroredStorage const &o) : m_n(o.m_n)
+    MirroredStorage(MirroredStorage const &o) : m_n(o.m_n), m_extent(o.m_extent)
     {
         allocate();
         if (m_n == 0) return;
@@ -99,6 +99,8 @@ public:
 
     void swap(MirroredStorage &o) noexcept
     {
+        std::swap(m_upload, o.m_upload);
+        std::swap(m_extent, o.m_extent);
         std::swap(m_n, o.m_n);
         std::swap(m_host, o.m_host);
         std::swap(m_dev, o.m_dev);
@@ -110,6 +112,7 @@ public:
 
     T *host_rw()
     {
+        finish_upload();       // the host block is about to change: a copy in flight must have read it
         pull();
         m_dev_valid = false;
         return m_host;
@@ -130,6 +133,25 @@ public:
         m_host_valid = false;
         return m_dev;
     }
+    // The elements [0, n) are the ones in use (a tensor's shape inside a larger buffer): a download to the host copies
+    // only those.  Model classes ping-pong between two tensors sized for their largest activation; reading 64 x 1000
+    // logits back must not move 200 MB.  Growing the extent makes a host copy that was downloaded at the smaller
+    // extent stale again.
+    void set_extent(size_t n)
+    {
+        if (n > m_extent && m_dev_valid) m_host_valid = false;
+        m_extent = n;
+    }
+    // Starts the upload of host-side contents now, on the library's copy stream, behind the layer calls queued so far
+    // and without blocking the host: the layer calls that follow run while it is in flight, and the first call that
+    // uses this buffer makes its stream wait for it.  A caller that feeds batches from host memory fills and prefetches
+    // input tensor B while the model runs on input tensor A.
+    void prefetch() const
+    {
+        if (m_dev_valid || m_n == 0 || m_upload) return;
+        hip_check(small_hip_upload_begin(m_dev, m_host, m_n * sizeof(T), current_stream(), &m_upload), "prefetch");
+        m_dev_valid = true;
+    }
 
 private:
     void allocate()
@@ -146,8 +168,17 @@ private:
         m_host = static_cast<T *>(h);
         m_dev = static_cast<T *>(d);
     }
+    void finish_upload() const
+    {
+        if (!m_upload) return;
+        small_hip_event_t ev = m_upload;
+        m_upload = nullptr;
+        hip_check(small_hip_upload_finish(ev), "prefetch");
+    }
     void release() noexcept
     {
+        if (m_upload) (void)small_hip_upload_finish(m_upload);
+        m_upload = nullptr;
         if (m_dev) small_hip_free(m_dev);
         if (m_host) small_hip_host_free(m_host);
         m_dev = nullptr;
@@ -157,12 +188,20 @@ private:
     void pull() const
     {
         if (m_host_valid || m_n == 0) return;
-        hip_check(small_hip_memcpy_d2h(m_host, m_dev, m_n * sizeof(T), current_stream()), "device to host");
+        const size_t n = m_extent < m_n ? m_extent : m_n;
+        hip_check(small_hip_memcpy_d2h(m_host, m_dev, n * sizeof(T), current_stream()), "device to host");
         hip_check(small_hip_stream_synchronize(current_stream()), "synchronize");
         m_host_valid = true;
     }
     void push() const
     {
+        if (m_upload)
+        {
+            // a prefetch is in flight: the layer call that is about to use the buffer waits for it on its stream
+            small_hip_event_t ev = m_upload;
+            m_upload = nullptr;
+            hip_check(small_hip_upload_wait(ev, current_stream()), "prefetch");
+        }
         if (m_dev_valid || m_n == 0) return;
         hip_check(small_hip_memcpy_h2d(m_dev, m_host, m_n * sizeof(T), current_stream()), "host to device");
         // the pinned block may be rewritten by the caller as soon as this returns
@@ -171,10 +210,12 @@ private:
     }
 
     size_t m_n = 0;
+    size_t m_extent = ~size_t(0);                      // elements in use (downloads stop there)
     T *m_host = nullptr;
     T *m_dev = nullptr;
     mutable bool m_host_valid = true;
     mutable bool m_dev_valid = false;
+    mutable small_hip_event_t m_upload = nullptr;      // a prefetch whose completion no stream has waited for yet
 };
 
 } // namespace detail
@@ -235,6 +276,10 @@ public:
     // device side, used by the layer functions
     value_type const *device_in() const { return m_store.device_in(); }
     value_type *device_out() { return m_store.device_out(); }
+    // start uploading host-side contents now, overlapped with the layer calls that follow (see MirroredStorage::prefetch)
+    void prefetch() const { m_store.prefetch(); }
+    // only the first n elements are in use: downloads to the host stop there (Tensor::set_shape calls this)
+    void set_extent(size_t n) { m_store.set_extent(n); }
 
 private:
     detail::MirroredStorage<float> m_store;
@@ -309,6 +354,8 @@ public:
 
     value_type const *device_in() const { return m_store.device_in(); }
     value_type *device_out() { return m_store.device_out(); }
+    void prefetch() const { m_store.prefetch(); }
+    void set_extent(size_t n) { m_store.set_extent(n); }
     small_hip_quant quant() const { return small_hip_quant{m_zero, multiplier, lshift, rshift}; }
 
 public:

@@ -70,6 +70,7 @@ public:
         if (compute_size(new_shape) > m_buffer.size())
             throw std::invalid_argument("Tensor::set_shape() ERROR: insufficient buffer size.");
         m_shape = new_shape;
+        m_buffer.set_extent(compute_size(new_shape));      // a download to the host moves the tensor, not the capacity
     }
 
     shape_type const &shape() const { return m_shape; }
@@ -77,6 +78,11 @@ public:
     size_t capacity() const { return m_buffer.size(); }
     BufferT &buffer() { return m_buffer; }
     BufferT const &buffer() const { return m_buffer; }
+
+    // Not in the reference (whose tensors are host memory): start uploading the host-side contents now, overlapped with
+    // the layer calls that follow; the first layer that reads the tensor waits for the upload on its stream.  Feed a
+    // model from two input tensors in turn: fill and prefetch one while inference() runs on the other.
+    void prefetch() const { m_buffer.prefetch(); }
 
     void swap(Tensor<BufferT> &other) noexcept
     {

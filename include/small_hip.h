@@ -85,6 +85,21 @@ int small_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, small_hip_str
 int small_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, small_hip_stream_t stream);
 int small_hip_memset(void *dst, int value, size_t bytes, small_hip_stream_t stream);
 int small_hip_stream_synchronize(small_hip_stream_t stream);
+/* Uploads that overlap the layer calls (no counterpart in the reference, whose buffers are host memory): a caller
+ * that holds host buffers uploads batch i+1 while the layers of batch i run.
+ *   small_hip_upload_begin  queues a copy of `bytes` from PINNED host memory (small_hip_host_malloc) to device memory
+ *                           on the calling device's copy stream (one per device, created on first use), behind the
+ *                           work already queued on `after` (so that it cannot overwrite a tensor an earlier pass
+ *                           still reads); returns at once with an event handle in *done;
+ *   small_hip_upload_wait   makes `stream` wait for that copy without blocking the host, and releases the handle;
+ *   small_hip_upload_finish blocks the host until the copy has finished (before the host block is rewritten), and
+ *                           releases the handle.
+ * Exactly one of wait / finish per begin.  dst must not be a tensor that work queued AFTER the begin call reads or
+ * writes before it has waited for the copy: use two input tensors in turn. */
+typedef void *small_hip_event_t;
+int small_hip_upload_begin(void *dst, const void *src, size_t bytes, small_hip_stream_t after, small_hip_event_t *done);
+int small_hip_upload_wait(small_hip_event_t done, small_hip_stream_t stream);
+int small_hip_upload_finish(small_hip_event_t done);
 /* Library-owned device scratch (no counterpart in the reference, whose layers work in place on the host).  Two kinds
  * of entry point lease a block per (device, stream): small_hip_conv2d_u8 / small_hip_group_conv2d_u8 (the prepared
  * filter: small_hip_conv2d_u8_prepared_filter_bytes, times the group count), and the float32 convolution entry points

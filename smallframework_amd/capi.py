@@ -76,6 +76,9 @@ SIGNATURES = {
     "small_hip_memcpy_d2d": (_i, [_p, _p, _sz, _p]),
     "small_hip_memset": (_i, [_p, _i, _sz, _p]),
     "small_hip_stream_synchronize": (_i, [_p]),
+    "small_hip_upload_begin": (_i, [_p, _p, _sz, _p, C.POINTER(_p)]),
+    "small_hip_upload_wait": (_i, [_p, _p]),
+    "small_hip_upload_finish": (_i, [_p]),
     "small_hip_workspace_reserve": (_i, [_sz, _p]),
     "small_hip_workspace_release": (_i, []),
     "small_hip_workspace_held": (_sz, []),

@@ -236,4 +236,64 @@ int small_hip_stream_synchronize(small_hip_stream_t stream)
     return SMALL_HIP_OK;
 }
 
+// ---- uploads that overlap the compute stream -----------------------------------------------------------------
+namespace
+{
+// one copy stream per device, created on first use (default priority, never destroyed)
+int copy_stream(hipStream_t *out)
+{
+    constexpr int MAX_DEV = 64;
+    static std::mutex mu;
+    static hipStream_t streams[MAX_DEV] = {};
+    int dev = 0;
+    SHP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEV) return einval("small_hip_upload_begin: device index out of range");
+    std::lock_guard<std::mutex> lk(mu);
+    if (!streams[dev]) SHP_HIP(hipStreamCreateWithFlags(&streams[dev], hipStreamNonBlocking));
+    *out = streams[dev];
+    return SMALL_HIP_OK;
+}
+} // namespace
+
+int small_hip_upload_begin(void *dst, const void *src, size_t bytes, small_hip_stream_t after, small_hip_event_t *done)
+{
+    if (!done) return einval("small_hip_upload_begin: null event pointer");
+    *done = nullptr;
+    if (!dst || !src) return einval("small_hip_upload_begin: null pointer");
+    hipStream_t cs = nullptr;
+    if (int rc = copy_stream(&cs)) return rc;
+    hipEvent_t ev = nullptr;
+    SHP_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    // the copy must not overtake work already queued on `after` that still reads dst
+    hipError_t e = hipEventRecord(ev, as_stream(after));
+    if (e == hipSuccess) e = hipStreamWaitEvent(cs, ev, 0);
+    if (e == hipSuccess && bytes) e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, cs);
+    if (e == hipSuccess) e = hipEventRecord(ev, cs);          // re-recorded: now it marks the end of the copy
+    if (e != hipSuccess)
+    {
+        (void)hipEventDestroy(ev);
+        return fail_hip(e, "small_hip_upload_begin");
+    }
+    *done = ev;
+    return SMALL_HIP_OK;
+}
+
+int small_hip_upload_wait(small_hip_event_t done, small_hip_stream_t stream)
+{
+    if (!done) return SMALL_HIP_OK;
+    hipEvent_t ev = static_cast<hipEvent_t>(done);
+    const hipError_t e = hipStreamWaitEvent(as_stream(stream), ev, 0);
+    (void)hipEventDestroy(ev);                                  // released once the queued wait has seen it
+    return e == hipSuccess ? SMALL_HIP_OK : fail_hip(e, "small_hip_upload_wait");
+}
+
+int small_hip_upload_finish(small_hip_event_t done)
+{
+    if (!done) return SMALL_HIP_OK;
+    hipEvent_t ev = static_cast<hipEvent_t>(done);
+    const hipError_t e = hipEventSynchronize(ev);
+    (void)hipEventDestroy(ev);
+    return e == hipSuccess ? SMALL_HIP_OK : fail_hip(e, "small_hip_upload_finish");
+}
+
 } // extern "C"

@@ -317,6 +317,73 @@ int stest_model_time_f32(int which, int variant, int batch, int C, int H, int W,
     });
 }
 
+// A caller that holds HOST buffers: every step a new batch sits in host memory, is uploaded, run, and the logits are read
+// back on the host.  serial: one input tensor, upload -> inference -> read.  overlapped: two input tensors in turn,
+// Tensor::prefetch() of batch i + 1 before inference() of batch i is issued, so the upload rides under the layers.
+// Milliseconds per step of both forms; *mismatches counts overlapped steps whose logits differ from the serial run's
+// logits for the same batch (two distinct batches alternate).
+int stest_model_host_feed_f32(int batch, const size_t *sizes, int nfilters, int steps, int warmup, double *ms_serial,
+                              double *ms_overlapped, int *mismatches)
+{
+    return guarded([&] {
+        const small::shape_type is{(size_t)batch, 3, 224, 224};
+        std::vector<std::unique_ptr<FB>> own;
+        std::vector<FB *> fl;
+        for (int i = 0; i < nfilters; ++i)
+        {
+            own.emplace_back(new FB(sizes[i]));
+            float *p = own.back()->data();
+            for (size_t k = 0; k < sizes[i]; ++k) p[k] = 0.05f * float((int)((k * 2654435761u) >> 24) - 128) / 128.f;
+            fl.push_back(own.back().get());
+        }
+        small::MobileNetTiny<FB> m(is, fl, false, 32, 1000, true);
+        small::Tensor<FB> x[2] = {small::Tensor<FB>(is), small::Tensor<FB>(is)};
+        for (int b = 0; b < 2; ++b)
+        {
+            float *px = x[b].buffer().data();
+            for (size_t k = 0; k < x[b].size(); ++k) px[k] = float((int)(((k + 977u * b) * 40503u) & 255) - 128) / 128.f;
+        }
+        // a new batch "arrives": the host block is written (one element is enough to make the whole tensor stale on the device)
+        auto arrive = [&](int b, int step) { x[b].buffer().data()[0] = float((step & 1) ? 0.25f : -0.25f) + float(b); };
+        std::vector<float> want[2];
+        double total = 0.0;
+        auto read = [&](small::Tensor<FB> const *t, std::vector<float> &dst) {
+            float const *p = t->buffer().data();                // waits for the pass and downloads
+            dst.assign(p, p + t->size());
+        };
+        // serial
+        for (int i = 0; i < warmup + steps; ++i)
+        {
+            if (i == warmup) { small::synchronize(); total = 0.0; }
+            const auto t0 = std::chrono::steady_clock::now();
+            const int b = i & 1;
+            arrive(b, b);
+            auto outs = m.inference(&x[b]);
+            read(outs[0], want[b]);
+            total += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        }
+        *ms_serial = total / steps;
+        // overlapped
+        *mismatches = 0;
+        std::vector<float> got;
+        arrive(0, 0);
+        x[0].prefetch();
+        for (int i = 0; i < warmup + steps; ++i)
+        {
+            if (i == warmup) total = 0.0;
+            const auto t0 = std::chrono::steady_clock::now();
+            const int b = i & 1, nb = b ^ 1;
+            arrive(nb, nb);
+            x[nb].prefetch();                                    // batch i + 1 goes up while batch i runs
+            auto outs = m.inference(&x[b]);
+            read(outs[0], got);
+            total += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            if (got.size() != want[b].size() || std::memcmp(got.data(), want[b].data(), got.size() * sizeof(float)) != 0) ++*mismatches;
+        }
+        *ms_overlapped = total / steps;
+    });
+}
+
 // Resnet8Tiny<QUInt8Buffer>: every tensor of the model shares one set of quantisation fields per role
 // (input, filters, activations), enough to exercise the quantised layer classes end to end.
 int stest_resnet8_u8(int batch, const uint8_t *const *filters, const size_t *sizes, int nfilters, const uint8_t *in,

@@ -124,6 +124,15 @@ class HipLayers(_Shim):
         self._check(rc)
         return ms.value
 
+    def model_host_feed_f32(self, batch, filter_sizes, steps=20, warmup=4):
+        """MobileNetV1 fed from host buffers: -> (ms per step serial, ms per step with Tensor::prefetch, mismatching steps)."""
+        sizes = (C.c_size_t * len(filter_sizes))(*filter_sizes)
+        a, b, bad = C.c_double(), C.c_double(), C.c_int()
+        rc = self.lib.stest_model_host_feed_f32(C.c_int(batch), sizes, C.c_int(len(filter_sizes)), C.c_int(steps), C.c_int(warmup),
+                                                C.byref(a), C.byref(b), C.byref(bad))
+        self._check(rc)
+        return a.value, b.value, bad.value
+
     def fused_two_layers_f32(self, second, variant, ck, cs, cp, k2, s2, p2, Co, Ci, H, W, x, f, bias, dwf, dwbias, n_out,
                              n_inter):
         """The reference-named Conv2D_*_Maxpool2D (second "pool") / Conv2D_*_DepthwiseConv2D_* ("dw") functions of

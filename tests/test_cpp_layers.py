@@ -354,3 +354,16 @@ def test_model_class_throughput(hip):
     print("TinyYoloV2<FloatBuffer> (416x416, LeakyReLU, 125 outputs) batch 16: %.3f ms per inference, %.0f images/s"
           % (ms, 16 / ms * 1e3))
     assert ms < 2.6
+
+
+@pytest.mark.gpu
+def test_host_fed_model_overlaps_upload_and_layers(hip):
+    """A caller that holds host buffers (what the reference's API gives): with two input tensors in turn and
+    Tensor::prefetch(), the upload of batch i + 1 (38.5 MB at batch 64) runs under the layers of batch i.  Same logits as
+    the serial upload -> inference -> read loop, bit for bit, and less time per step."""
+    sizes = [int(np.prod(f.shape)) for f in ol.make_filters(synth, ol.mobilenet_specs(), 1000)]
+    serial, overlapped, bad = hip.model_host_feed_f32(64, sizes)
+    print("MobileNetV1 batch 64 from host buffers: serial %.3f ms/step, overlapped %.3f ms/step (%.0f images/s)"
+          % (serial, overlapped, 64 / overlapped * 1e3))
+    assert bad == 0
+    assert overlapped < 0.9 * serial
