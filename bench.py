@@ -27,11 +27,28 @@ PEAK_HBM = 8.0e12          # B/s, MI355X HBM3E
 PEAK_MFMA_F32 = 157.3e12   # FLOP/s, dense fp32 MFMA
 PEAK_MFMA_I8 = 5.0e15      # OP/s, dense int8 MFMA
 
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (two runs) over this same benchmark and scaled by what the counters read for an
-# in-place ReLU of 822 MB (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00); the summary is
-# profiles/mobilenet_v1_b64_traffic_and_mfma.md.  Keyed by (model, batch, kernel family).
-MEASURED_TRAFFIC_MB_PER_LAUNCH = {("mobilenet_v1", 64, "conv_mfma_f32_*"): 70.0}
+# HBM bytes per launch of the dominant kernel come from the committed counter summary (rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE over this same benchmark, two runs, scaled by what the counters read for an in-place ReLU of 822 MB): the
+# figure is read from that file, together with the number of launches it was measured over, and is reported only while
+# the forward pass still issues that many launches of the kernel family (another kernel mix: null, measure again).
+TRAFFIC_PROFILES = {("mobilenet_v1", 64, "conv_mfma_f32_*"): "profiles/mobilenet_v1_b64_traffic_and_mfma.md"}
+
+
+def measured_traffic_bytes(model_name, batch, family, launches):
+    """-> HBM bytes per launch of `family` from the committed profile, or None (no profile, or measured on another mix)."""
+    rel = TRAFFIC_PROFILES.get((model_name, batch, family))
+    if rel is None:
+        return None
+    try:
+        text = open(os.path.join(ROOT, rel)).read()
+    except OSError:
+        return None
+    import re
+    row = re.search(r"^\| %s \| (\d+) \|" % re.escape(family), text, re.M)
+    per = re.search(r"HBM traffic ([0-9.]+) MB", text)
+    if not row or not per or int(row.group(1)) != launches:
+        return None
+    return round(float(per.group(1)) * 1e6)
 
 
 def log(*a):
@@ -60,7 +77,7 @@ def table_summary(entry, batch):
     fl = [r["frac_of_stream_floor"] for r in entry["layers"] if r.get("frac_of_stream_floor")]
     if len(entry["layers"]) == 1 and fl:
         out["of_bytes_only_kernel"] = fl[0]         # single bandwidth-bound layer: against a kernel that only moves its bytes
-    for k in ("hip_graph_ms_per_step", "one_launch_ms_per_step", "one_launch_images_per_s"):
+    for k in ("hip_graph_ms_per_step", "one_launch_ms_per_step", "one_launch_images_per_s", "roofline"):
         if k in entry:
             out[k] = entry[k]
     return out
@@ -618,9 +635,8 @@ def main():
         ach = d["bytes"] / (d["ms"] * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s",
                 "frac": round(ach / 8000.0, 4), "traffic": None}
-    mt = MEASURED_TRAFFIC_MB_PER_LAUNCH.get((model.name, batch, dom))
-    if mt is not None and not args.unfused:
-        roof["traffic"] = round(mt * 1e6)      # bytes per launch, like algorithmic_per_launch
+    if not args.unfused:
+        roof["traffic"] = measured_traffic_bytes(model.name, batch, dom, d["launches"])   # bytes per launch, or None
     roof.update({"kernel": dom, "launches_per_step": d["launches"],
                  "avg_launch_ms": round(d["ms"] / d["launches"], 5),
                  "algorithmic_per_launch": {"GFLOP": round(d["flops"] / d["launches"] / 1e9, 3),
@@ -677,14 +693,16 @@ def main():
             ex.buf["in"].copy_(hx, non_blocking=True)
             ex.forward()
             hy.copy_(ex.buf[ex.out_name][:n_out], non_blocking=True)
-        for _ in range(args.warmup):
+        # a side measurement whose pipeline needs some steps to fill: at least 100 timed steps after 30
+        h_steps, h_warm = max(args.steps, 100), max(args.warmup, 30)
+        for _ in range(h_warm):
             host_step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(h_steps):
             host_step()
         torch.cuda.synchronize()
-        sh = (time.perf_counter() - t0) / args.steps
+        sh = (time.perf_counter() - t0) / h_steps
         extras["host_buffers_serial_ms_per_step"] = round(sh * 1e3, 4)
         extras["host_buffers_MB_per_step"] = round((hx.numel() * hx.element_size() + hy.numel() * hy.element_size()) / 1e6, 2)
         log("%s: with host buffers, serial (upload + forward + download on one stream) %.3f ms/step" % (model.name, sh * 1e3))
@@ -716,14 +734,14 @@ def main():
             ex.forward()                                   # ... while batch i runs
             hy.copy_(ex.buf[ex.out_name][:n_out], non_blocking=True)
         begin(0)
-        for _ in range(args.warmup):
+        for _ in range(h_warm):
             host_step_overlapped()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(h_steps):
             host_step_overlapped()
         torch.cuda.synchronize()
-        so = (time.perf_counter() - t0) / args.steps
+        so = (time.perf_counter() - t0) / h_steps
         capi.check(lib.small_hip_upload_finish(pending[step_no[0] & 1]))
         same = bool((hy.numpy() == ref_out).all())
         ex.buf["in"] = din[0]
@@ -762,6 +780,17 @@ def main():
                                             "one_launch_images_per_s": round(b / s4, 1),
                                             "one_launch_TOPs": round(b * m2.flops_per_image() / s4 / 1e12, 2),
                                             "one_launch_algorithmic_MB": round(algo / 1e6, 3),
+                                            # the step is one kernel: the model's arithmetic over its launch time, HIP events
+                                            # on the launch stream, against the int8 MFMA peak (neither roofline binds a
+                                            # 25 MOP model of 16..64-channel layers: the figure says how far away they are)
+                                            "roofline": {"bound": "mfma", "kernel": "qmodel_u8_kernel",
+                                                         "achieved": round(b * m2.flops_per_image() / s4 / 1e12, 2),
+                                                         "peak": round(PEAK_MFMA_I8 / 1e12, 1), "unit": "TOP/s",
+                                                         "frac": round(b * m2.flops_per_image() / s4 / PEAK_MFMA_I8, 4),
+                                                         "traffic": None, "launches_per_step": 1,
+                                                         "avg_launch_ms": round(s4 * 1e3, 5),
+                                                         "algorithmic_per_launch": {"GOP": round(b * m2.flops_per_image() / 1e9, 3),
+                                                                                    "MB": round(algo / 1e6, 3)}},
                                             "layers": layer_table(m2, b, ms2)}
             log("%s batch %d: layer by layer %.4f ms/step %.0f images/s | HIP graph %.4f ms/step | ONE LAUNCH %.4f ms/step "
                 "%.0f images/s" % (name, b, s2 * 1e3, b / s2, s3 * 1e3, s4 * 1e3, b / s4))
