@@ -564,6 +564,16 @@ def main():
     x = models.make_input(model, batch)
     ex = models.HipExecutor(model, batch, weights, x, fused=not args.unfused)
 
+    # The machine calibration runs first (float32 MFMA on registers only, a device-to-device copy: about 60 ms of load
+    # whose figures the per-layer tables are read against), so the GPU is in its sustained state when the warm-up
+    # steps start; a fresh process otherwise spends its first tens of milliseconds of load below its sustained clock,
+    # which is what 5 + 20 steps of a 0.9 ms pass would measure.
+    calib = {}
+    if model.dtype == "f32" and not args.no_extras:
+        sustained = mfma_probe_tflops()
+        if sustained is not None:
+            calib["mfma_f32_sustained_TFLOPs"] = round(sustained, 1)
+        calib["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
     sec = time_forward(ex, args.steps, args.warmup)
     one_launch = None
     if model.dtype == "u8" or model.name == "dscnn":
@@ -664,10 +674,7 @@ def main():
                         "`batch` of the 256 compute units busy"}
     if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
-        sustained = mfma_probe_tflops()
-        if sustained is not None:
-            extras["mfma_f32_sustained_TFLOPs"] = round(sustained, 1)
-        extras["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
+        extras.update(calib)
         # the same forward pass replayed from a HIP graph (no host work between the launches)
         ex.capture()
         for _ in range(args.warmup):
@@ -871,7 +878,9 @@ def main():
             model.name, batch, model.in_shape[1], model.in_shape[2], model.in_shape[0],
             "whole model in one launch" if one_launch else
             "Conv2D+bias+activation fused" if not args.unfused else "unfused layer calls"),
-            "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4)},
+            "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4),
+            "before_warmup": ("machine calibration (MFMA probe, device copy: ~60 ms of load), then `warmup` untimed and "
+                              "`steps` timed forward passes") if calib else "nothing"},
         "roofline": roof,
         "cpu_baseline": cpu,
         "layers": table,

@@ -46,7 +46,7 @@ public:
     // launch: small_hip_qmodel_forward for QUInt8Buffer, bit-identical to the layer-by-layer calls and used by default;
     // small_hip_fmodel_forward for FloatBuffer, within the float32 tolerance of them (another summation order) and
     // therefore only on request.  Only the returned tensor is written.
-    // true / false: use / never use that form (environment: SMALL_HIP_ONE_LAUNCH=1 / 0).
+    // true / false: use / never use that form (environment: SMALL_HIP_TUNE=one_launch=1 / 0).
     void set_one_launch(bool on) { m_one_launch = on; }
     // true once inference() has planned (and used) the one-launch form
     bool one_launch_planned() const { return m_qmodel != nullptr || m_fmodel != nullptr; }
