@@ -99,12 +99,20 @@ __device__ __forceinline__ float act_bf(float v, float neg_scale)
     const float n = fmaf(v, neg_scale, 0.f);
     return v > 0.f ? v : n;
 }
+// The same with the kind known at compile time: ReLU is one instruction (a maximum) instead of three, and gives the
+// same bits as act_bf(v, 0) for every input that is a number (negative and -0 -> +0).  A vector instruction costs the
+// matrix pipe of its SIMD about eight cycles whichever wave issues it, so the epilogues' instruction count is launch time.
+template <bool RELU>
+__device__ __forceinline__ float act_k(float v, float neg_scale)
+{
+    return RELU ? fmaxf(v, 0.f) : act_bf(v, neg_scale);
+}
 
 // accumulate / bias / activation in registers, then 16-byte stores: a lane holds channels
 // 8q + 4*half + {0..3} of its pixel in accumulator registers 4q .. 4q+3.  Straight-line code:
 // pixels past the end and channels past Co are computed and not stored, the bias is loaded once
 // per channel quad, PartialConv2D (ACC) is a compile-time variant.
-template <int COT, int PXT, bool ACC>
+template <int COT, int PXT, bool ACC, bool RELU>
 __device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
                                                    int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT],
                                                    const float *lds_bias)
@@ -158,8 +166,8 @@ __device__ __forceinline__ void conv_epilogue_impl(const ConvArgs &a, floatx16 (
                     v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
                 }
                 v.x += bb[c][q].x; v.y += bb[c][q].y; v.z += bb[c][q].z; v.w += bb[c][q].w;
-                v.x = act_bf(v.x, nscale); v.y = act_bf(v.y, nscale);
-                v.z = act_bf(v.z, nscale); v.w = act_bf(v.w, nscale);
+                v.x = act_k<RELU>(v.x, nscale); v.y = act_k<RELU>(v.y, nscale);
+                v.z = act_k<RELU>(v.z, nscale); v.w = act_k<RELU>(v.w, nscale);
                 if (ok) *o = v;
             }
         }
@@ -171,8 +179,11 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
                                               int HoWo, const bool (&pvalid)[PXT], const size_t (&out_pix)[PXT],
                                               const float *lds_bias = nullptr)
 {
-    if (a.accumulate) conv_epilogue_impl<COT, PXT, true>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
-    else conv_epilogue_impl<COT, PXT, false>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
+    // the epilogue runs once per workgroup: a uniform branch picks the straight-line variant (ReLU is one instruction
+    // per value instead of three, and the epilogue's vector instructions are time the matrix pipe stands still)
+    if (a.accumulate) conv_epilogue_impl<COT, PXT, true, false>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
+    else if (a.act == SMALL_HIP_ACT_RELU) conv_epilogue_impl<COT, PXT, false, true>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
+    else conv_epilogue_impl<COT, PXT, false, false>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
 }
 
 // Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 8 pooling windows of
@@ -1167,7 +1178,7 @@ struct StemDwArgs
     const float *dw_bias;   // [Co] or nullptr
 };
 
-template <int CI, int S, int NCOB>
+template <int CI, int S, int NCOB, bool RELU = false>
 __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const ConvArgs a, const StemDwArgs d, int tiles_x, int tiles_y)
 {
     typedef float floatx4v __attribute__((ext_vector_type(4)));
@@ -1288,7 +1299,7 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
         {
             const int row = 4 * wave + t, oh1 = oh0 + row;
             float4 v = make_float4(acc[t][0] + bb.x, acc[t][1] + bb.y, acc[t][2] + bb.z, acc[t][3] + bb.w);
-            v.x = act_bf(v.x, nscale); v.y = act_bf(v.y, nscale); v.z = act_bf(v.z, nscale); v.w = act_bf(v.w, nscale);
+            v.x = act_k<RELU>(v.x, nscale); v.y = act_k<RELU>(v.y, nscale); v.z = act_k<RELU>(v.z, nscale); v.w = act_k<RELU>(v.w, nscale);
             // outside the first layer's output: the depthwise layer's padding
             if (!(col_in && (unsigned)oh1 < (unsigned)a.Ho)) v = make_float4(0.f, 0.f, 0.f, 0.f);
             mid[(row * T + col) * 4 + kq] = v;
@@ -1327,8 +1338,8 @@ __global__ __launch_bounds__(256, 4) void conv_stem3x3_dw3x3_f32_kernel(const Co
                     acc2.x = fmaf(x.x, k.x, acc2.x); acc2.y = fmaf(x.y, k.y, acc2.y);
                     acc2.z = fmaf(x.z, k.z, acc2.z); acc2.w = fmaf(x.w, k.w, acc2.w);
                 }
-            acc2.x = act_bf(acc2.x, nscale); acc2.y = act_bf(acc2.y, nscale);
-            acc2.z = act_bf(acc2.z, nscale); acc2.w = act_bf(acc2.w, nscale);
+            acc2.x = act_k<RELU>(acc2.x, nscale); acc2.y = act_k<RELU>(acc2.y, nscale);
+            acc2.z = act_k<RELU>(acc2.z, nscale); acc2.w = act_k<RELU>(acc2.w, nscale);
             if (ok) dst[(size_t)oh * a.Wo * 4] = acc2;
         }
     }
@@ -1365,7 +1376,7 @@ struct PwDwGeom
     int n_wgs, per_xcd;  // workgroups = tiles x channel groups, and their share per XCD
 };
 
-template <int S, int COT, int CIB>
+template <int S, int COT, int CIB, bool RELU = false>
 __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArgs a, const StemDwArgs d, const PwDwGeom g)
 {
     using TL = PwDwTile<S>;
@@ -1485,20 +1496,34 @@ __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArg
 
     __syncthreads();                                         // every wave has read its last filter operand
     // ---- bias, activation, park in LDS: a lane holds channels c*32 + 8 qq + 4 half + 0..3 of its pixel -------------
+    // pixels outside the pointwise layer's map are the depthwise layer's padding: those lanes store zeros (a branch on
+    // the lane mask: no select per value)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
+    {
+        if (pin[t])
+        {
 #pragma unroll
-        for (int c = 0; c < COT; ++c)
+            for (int c = 0; c < COT; ++c)
 #pragma unroll
-            for (int qq = 0; qq < 4; ++qq)
-            {
-                const int ch = c * 32 + 8 * qq + 4 * half;
-                const float4 bb = *reinterpret_cast<const float4 *>(&s_bias[ch]);
-                float4 v = make_float4(act_bf(acc[c][t][4 * qq + 0] + bb.x, nscale), act_bf(acc[c][t][4 * qq + 1] + bb.y, nscale),
-                                       act_bf(acc[c][t][4 * qq + 2] + bb.z, nscale), act_bf(acc[c][t][4 * qq + 3] + bb.w, nscale));
-                if (!pin[t]) v = make_float4(0.f, 0.f, 0.f, 0.f);      // outside the map: the depthwise layer's padding
-                *reinterpret_cast<float4 *>(&mid[pidx[t] * MIDP + ch]) = v;
-            }
+                for (int qq = 0; qq < 4; ++qq)
+                {
+                    const int ch = c * 32 + 8 * qq + 4 * half;
+                    const float4 bb = *reinterpret_cast<const float4 *>(&s_bias[ch]);
+                    const float4 v = make_float4(act_k<RELU>(acc[c][t][4 * qq + 0] + bb.x, nscale), act_k<RELU>(acc[c][t][4 * qq + 1] + bb.y, nscale),
+                                                 act_k<RELU>(acc[c][t][4 * qq + 2] + bb.z, nscale), act_k<RELU>(acc[c][t][4 * qq + 3] + bb.w, nscale));
+                    *reinterpret_cast<float4 *>(&mid[pidx[t] * MIDP + ch]) = v;
+                }
+        }
+        else
+        {
+#pragma unroll
+            for (int c = 0; c < COT; ++c)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+                    *reinterpret_cast<float4 *>(&mid[pidx[t] * MIDP + c * 32 + 8 * qq + 4 * half]) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     __syncthreads();
 
     // ---- depthwise 3x3 on the parked patch ---------------------------------------------------------------------------
@@ -1548,8 +1573,8 @@ __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArg
                 acc2.x = fmaf(x.x, k.x, acc2.x); acc2.y = fmaf(x.y, k.y, acc2.y);
                 acc2.z = fmaf(x.z, k.z, acc2.z); acc2.w = fmaf(x.w, k.w, acc2.w);
             }
-        acc2.x = act_bf(acc2.x, nscale); acc2.y = act_bf(acc2.y, nscale);
-        acc2.z = act_bf(acc2.z, nscale); acc2.w = act_bf(acc2.w, nscale);
+        acc2.x = act_k<RELU>(acc2.x, nscale); acc2.y = act_k<RELU>(acc2.y, nscale);
+        acc2.z = act_k<RELU>(acc2.z, nscale); acc2.w = act_k<RELU>(acc2.w, nscale);
         if (ok) dst[(size_t)oh * g.Wd * 4] = acc2;
     }
 }
@@ -1933,10 +1958,13 @@ int stem_dw_f32(const char *op, int batch, int kh, int kw, int stride, int pt, i
     const StemDwArgs d{dw_filt, dw_bias};
     const dim3 gs((unsigned)nt, (unsigned)(CoB / ncob));
     void (*ks)(const ConvArgs, const StemDwArgs, int, int) = nullptr;
-#define SHP_SD(CI_, S_) (ncob == 2 ? conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 2> : conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 1>)
+    const bool relu = act == SMALL_HIP_ACT_RELU;           // ReLU has its own instantiation: one instruction per value
+#define SHP_SD_(CI_, S_, R_) (ncob == 2 ? conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 2, R_> : conv_stem3x3_dw3x3_f32_kernel<CI_, S_, 1, R_>)
+#define SHP_SD(CI_, S_) (relu ? SHP_SD_(CI_, S_, true) : SHP_SD_(CI_, S_, false))
     if (stride == 1) ks = Ci == 1 ? SHP_SD(1, 1) : Ci == 2 ? SHP_SD(2, 1) : SHP_SD(3, 1);
     else ks = Ci == 1 ? SHP_SD(1, 2) : Ci == 2 ? SHP_SD(2, 2) : SHP_SD(3, 2);
 #undef SHP_SD
+#undef SHP_SD_
     hipLaunchKernelGGL(ks, gs, dim3(256), 0, as_stream(stream), a, d, tiles_x, tiles_y);
     SHP_LAUNCH_CHECK(op);
     return SMALL_HIP_OK;
@@ -1981,10 +2009,13 @@ int pw_dw_f32(const char *op, int batch, int dw_stride, int dpt, int dpb, int dp
     g.n_wgs = (int)(nt * g.n_cg); g.per_xcd = (g.n_wgs + NUM_XCD - 1) / NUM_XCD;
     const dim3 grid(g.per_xcd * NUM_XCD);
     void (*k)(const ConvArgs, const StemDwArgs, const PwDwGeom) = nullptr;
-#define SHP_PD(S_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 2, 4> : conv_pw_dw3x3_f32_kernel<S_, 2, 8>) \
-                             : (cib == 1 ? conv_pw_dw3x3_f32_kernel<S_, 1, 1> : cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2> : cib == 3 ? conv_pw_dw3x3_f32_kernel<S_, 1, 3> \
-                                : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4> : cib == 6 ? conv_pw_dw3x3_f32_kernel<S_, 1, 6> : conv_pw_dw3x3_f32_kernel<S_, 1, 8>))
+#define SHP_PD_(S_, R_) (cot == 2 ? (cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 2, 2, R_> : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 2, 4, R_> : conv_pw_dw3x3_f32_kernel<S_, 2, 8, R_>) \
+                             : (cib == 1 ? conv_pw_dw3x3_f32_kernel<S_, 1, 1, R_> : cib == 2 ? conv_pw_dw3x3_f32_kernel<S_, 1, 2, R_> : cib == 3 ? conv_pw_dw3x3_f32_kernel<S_, 1, 3, R_> \
+                                : cib == 4 ? conv_pw_dw3x3_f32_kernel<S_, 1, 4, R_> : cib == 6 ? conv_pw_dw3x3_f32_kernel<S_, 1, 6, R_> : conv_pw_dw3x3_f32_kernel<S_, 1, 8, R_>))
+#define SHP_PD(S_) (relu ? SHP_PD_(S_, true) : SHP_PD_(S_, false))
+    const bool relu = act == SMALL_HIP_ACT_RELU;           // ReLU has its own instantiation: one instruction per value
     k = dw_stride == 1 ? SHP_PD(1) : SHP_PD(2);
+#undef SHP_PD_
 #undef SHP_PD
     hipLaunchKernelGGL(k, grid, dim3(256), 0, as_stream(stream), a, d, g);
     SHP_LAUNCH_CHECK(op);
