@@ -111,7 +111,7 @@ def emit(out, tag):
             # bandwidth-bound layers against a kernel that only moves their bytes (same place in the model)
             summary["headline_layers"].update({"bandwidth_layers": len(fl), "of_bytes_only_kernel_min": fl[0],
                                                "of_bytes_only_kernel_median": round(statistics.median(fl), 3)})
-    for k in ("mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "hip_graph_ms_per_step",
+    for k in ("mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "mfma_and_vector_alu_same_simd", "hip_graph_ms_per_step",
               "host_buffers_ms_per_step", "host_buffers_images_per_s", "host_buffers_serial_ms_per_step",
               "host_buffers_result_unchanged"):
         if k in extras:
@@ -357,6 +357,37 @@ def hbm_copy_gbs(nbytes=822083584, steps=10):
     return 2.0 * nbytes * steps / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
+def issue_overlap_us(iters=500):
+    """Calibration: matrix instructions of one wave and vector-ALU instructions of another wave on the same SIMD, timed
+    apart and together (libsmall_hip_probe.so, one workgroup of eight waves per CU; each side is 1024 issue cycles per
+    iteration).  -> {"matrix_us", "vector_us", "both_us"} or None when the probe library is not built.  both = matrix +
+    vector means the two do not overlap: a kernel's vector instructions are time its matrix pipe stands still."""
+    import ctypes as C
+    import torch
+    from smallframework_amd import capi
+    path = os.path.join(os.path.dirname(capi.LIB_PATH), "libsmall_hip_probe.so")
+    if not os.path.exists(path) or not hasattr(C.CDLL(path), "shp_probe_issue_overlap"):
+        return None
+    probe = C.CDLL(path).shp_probe_issue_overlap
+    probe.restype, probe.argtypes = C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    sink = torch.zeros(4, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+    for name, mode in (("matrix_us", 1), ("vector_us", 2), ("both_us", 3)):
+        for timed in (False, True):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                rc = probe(256, mode, iters, C.c_void_p(sink.data_ptr()), st)
+                if rc:
+                    raise RuntimeError("shp_probe_issue_overlap: status %d" % rc)
+            e1.record()
+            torch.cuda.synchronize()
+            if timed:
+                out[name] = round(e0.elapsed_time(e1) / 3 * 1e3, 1)
+    return out
+
+
 def library_gemm_ms(model, batch, steps, warmup):
     """Calibration, not part of the product path: the contraction of every MFMA-sized convolution as a plain
     float32 GEMM [Co x K] . [K x pixels] through torch.mm (the vendor BLAS; no im2col cost counted, TF32 off).
@@ -574,6 +605,9 @@ def main():
         if sustained is not None:
             calib["mfma_f32_sustained_TFLOPs"] = round(sustained, 1)
         calib["hbm_copy_sustained_GBs"] = round(hbm_copy_gbs(), 1)
+        ov = issue_overlap_us()
+        if ov is not None:
+            calib["mfma_and_vector_alu_same_simd"] = ov
     sec = time_forward(ex, args.steps, args.warmup)
     one_launch = None
     if model.dtype == "u8" or model.name == "dscnn":
