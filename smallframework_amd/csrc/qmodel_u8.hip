@@ -55,6 +55,7 @@ constexpr int MAX_TENSORS = 8;
 constexpr int MAX_STEPS = 256;           // K-steps (taps x channel blocks) of one layer
 constexpr int MAX_CO = 128;              // a layer's tables are fetched by one 16-byte load per thread
 constexpr int LDS_LIMIT = 160 * 1024;
+constexpr int FIN_ENTRIES = 514, FIN_BYTES = 528;   // the short epilogue's table (conv_tiles), padded to 16 bytes
 
 enum { K_STEM = 0, K_CONV = 1, K_POOL_AVG = 2, K_POOL_MAX = 3 };
 
@@ -72,11 +73,13 @@ struct QMLayer
     int Ci, Co, H, W, Ho, Wo, kh, kw, stride, pt, pl;
     int S_pad;                           // K-steps padded to a multiple of 4
     int w_off;                           // prepared filter: offset in LDS == offset in the filter image of the blob
-    int tab_off, tab16;                  // the layer's tables in the blob: T[16][Co] int32 | steps[S_pad] int32 | post[512],
-                                         // and their size in 16-byte pieces
+    int tab_off, tab16;                  // the layer's tables in the blob: T[16][Co] int32 | steps[S_pad] int32 | post[512] |
+                                         // fin[528] | postx[512] | pixel table [Ho*Wo][2] uint16, and their size in 16-byte pieces
     int32_t ZF;                          // filter zero point + 128 (convolutions)
     int32_t zI;                          // zero point of the input (pooling)
     int has_post;                        // Accum and / or ReLU follow: the convolution's byte goes through post[]
+    int idx_shift;                       // >= 0: the short epilogue (rshift - 2, see conv_tiles); -1: the general one
+    int geo_off;                         // the pixel table's offset inside the layer's tables (the short epilogue's layers)
     float r_wo, r_cob;                   // 1 / Wo, 1 / (Co / 16)
     int wo_shift;                        // log2(Wo) when Wo is a power of two, else -1
     QOut q;
@@ -217,8 +220,9 @@ __device__ __forceinline__ uint32_t requant_fast(int32_t acc, const FastQ f)
 // NM > 0: the layer has exactly NM MFMA steps (4 K-steps each), the loop is unrolled and the lane's K-step offsets
 // live in registers; NM == 0: any count, offsets read from the table per step.
 // POST: what follows the requantisation, fixed per instantiation so that the epilogue is straight-line code:
-// 0 nothing, 1 the byte goes through post[] (in-place ReLU), 2 Accum (+ ReLU): post[byte + shortcut byte], -1 decided per
-// layer at run time (the general form, also the only one that writes the model's output to global memory).
+// 3 the short epilogue (see there) without Accum, 4 with Accum: postx[byte + shortcut byte]; -1 decided per layer at run
+// time (the general form, also the only one that writes the model's output to global memory); 0 / 1 / 2 are the general
+// form's cases nothing / post[] / Accum as compile-time variants (kept for measurements).
 template <bool STEM, int TP, int NM, bool FAST, int POST = -1>
 __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
                                            int n_waves)
@@ -236,6 +240,8 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
     const int *steps = reinterpret_cast<const int *>(tab + 64 * L.Co);
     const uint8_t *post = tab + 64 * L.Co + 4 * L.S_pad;
     const FastQ fq{L.q.multiplier, L.q.lshift & 31, L.q.rshift, (L.q.rshift - 1) & 31, L.q.rshift > 0 ? 1 : 0};
+    constexpr bool GEO = POST >= 3;                   // the short epilogue's layers carry a pixel table
+    const uint8_t *geo = tab + L.geo_off;
     // the lane's K-steps: offset from the window origin, and the vector the box sum multiplies by (0 past the end:
     // such a step reads valid memory, its filter rows are zero, and it must not count towards the box sum)
     int so[NM > 0 ? NM : 1], ones[NM > 0 ? NM : 1];
@@ -258,6 +264,7 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
         const int cob = work - pg * CoB;
         const uint8_t *wrow = lds + L.w_off + (cob * L.S_pad * 16 + col) * 16 + grp * 256;
         int oh[TP], ow[TP], ih0[TP], iw0[TP];
+        int srcoff[TP], dstoff[TP], casoff[TP];      // GEO: the pixel's three offsets out of the layer's pixel table
         bool pvalid[TP];
 #pragma unroll
         for (int t = 0; t < TP; ++t)
@@ -265,6 +272,16 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
             const int p = (pg * TP + t) * 16 + col;
             pvalid[t] = p < P;
             const int pc = pvalid[t] ? p : P - 1;
+            if (GEO)
+            {
+                const uint16_t *ge = reinterpret_cast<const uint16_t *>(geo + pc * 4);
+                srcoff[t] = ge[0];
+                dstoff[t] = ge[1] & 0xfff0;
+                casoff[t] = ge[1] & 15;
+                oh[t] = ow[t] = ih0[t] = iw0[t] = 0;
+                continue;
+            }
+            srcoff[t] = dstoff[t] = casoff[t] = 0;
             if (wo_shift >= 0) { oh[t] = pc >> wo_shift; ow[t] = pc & (L.Wo - 1); }
             else { oh[t] = (int)(((float)pc + 0.5f) * L.r_wo); ow[t] = pc - oh[t] * L.Wo; }
             ih0[t] = (oh[t] << s_shift) - L.pt;
@@ -286,7 +303,8 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
                 uint32_t b[4] = {0, 0, 0, 0};
                 if (grp < L.kh)
                 {
-                    const uint32_t *row = reinterpret_cast<const uint32_t *>(src + (__mul24(ih0[t] + grp + 1, Wp) + iw0[t] + 1) * 4);
+                    const uint32_t *row = GEO ? reinterpret_cast<const uint32_t *>(src + srcoff[t] + __mul24(grp, Wp) * 4)
+                                              : reinterpret_cast<const uint32_t *>(src + (__mul24(ih0[t] + grp + 1, Wp) + iw0[t] + 1) * 4);
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         if (j < L.kw) b[j] = row[j];
@@ -300,7 +318,7 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
         {
             const uint8_t *pix[TP];
 #pragma unroll
-            for (int t = 0; t < TP; ++t) pix[t] = src + (__mul24(ih0[t] + 1, Wp) + iw0[t] + 1) * 16;
+            for (int t = 0; t < TP; ++t) pix[t] = GEO ? src + srcoff[t] : src + (__mul24(ih0[t] + 1, Wp) + iw0[t] + 1) * 16;
             if (NM > 0)
             {
 #pragma unroll
@@ -341,12 +359,56 @@ __device__ __forceinline__ void conv_tiles(const QMLayer &L, uint8_t *lds, const
             const int sit = si[t][0];
             if (!pvalid[t]) continue;
             // border case of the pixel -> T
-            const int ra = (ih0[t] < 0 ? 2 : 0) + (ih0[t] + L.kh > L.H ? 1 : 0);
-            const int rb = (iw0[t] < 0 ? 2 : 0) + (iw0[t] + L.kw > L.W ? 1 : 0);
-            const uint4 tc = *reinterpret_cast<const uint4 *>(T + __mul24(ra * 4 + rb, L.Co) + cob * CB + 4 * grp);
+            uint4 tc;
+            int opos;
+            if (GEO)
+            {
+                tc = *reinterpret_cast<const uint4 *>(tab + __mul24(casoff[t], L.Co * 4) + (cob * CB + 4 * grp) * 4);
+                opos = dstoff[t] + __mul24(cob * Hop, Wop) * 16 + 4 * grp;
+            }
+            else
+            {
+                const int ra = (ih0[t] < 0 ? 2 : 0) + (ih0[t] + L.kh > L.H ? 1 : 0);
+                const int rb = (iw0[t] < 0 ? 2 : 0) + (iw0[t] + L.kw > L.W ? 1 : 0);
+                tc = *reinterpret_cast<const uint4 *>(T + __mul24(ra * 4 + rb, L.Co) + cob * CB + 4 * grp);
+                opos = (__mul24(cob * Hop + oh[t] + 1, Wop) + ow[t] + 1) * 16 + 4 * grp;
+            }
             const uint32_t tc4[4] = {tc.x, tc.y, tc.z, tc.w};
             const uint32_t base = (uint32_t)L.ZF * (uint32_t)sit;
-            const int opos = (__mul24(cob * Hop + oh[t] + 1, Wop) + ow[t] + 1) * 16 + 4 * grp;
+            if (POST == 3 || POST == 4)
+            {
+                // The short epilogue (positive multiplier, rshift >= 2, result in LDS).  The requantised byte depends on
+                // idx = product >> (30 + rshift) alone, which is the product's high word shifted by rshift - 2: one
+                // shift instead of the 64-bit shift, the rounding bit, the subtraction and the post[] address; the clamp
+                // is the table's domain.  fin[] holds the byte as the tensors store it, so the four bytes go out as four
+                // byte stores with nothing to pack (LDS instructions do not take vector-ALU issue slots; the vector ALU
+                // is what this kernel waits for).
+                const uint8_t *fin = post + 512, *postx = fin + FIN_BYTES;
+                uint8_t *dstp = lds + L.dst_off + opos;
+                uint32_t sc = 0;
+                if (POST == 4) sc = *reinterpret_cast<const uint32_t *>(lds + L.acc_off + opos) ^ 0x80808080u;
+                // all table reads first, then the stores: a store between them would have to be assumed to change the
+                // tables (both are LDS) and each read would wait for its own round trip
+                uint32_t y[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                {
+                    const int32_t v = (int32_t)((uint32_t)acc[t][r] + base + tc4[r]);
+                    const int32_t shifted = (int32_t)((uint32_t)v << fq.ls);
+                    const long long prod = (long long)shifted * (long long)fq.mult + (1ll << 30);
+                    int idx = (int32_t)(prod >> 32) >> L.idx_shift;
+                    idx = idx < 0 ? 0 : (idx > FIN_ENTRIES - 1 ? FIN_ENTRIES - 1 : idx);
+                    y[r] = fin[idx];
+                }
+                if (POST == 4)
+                {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) y[r] = postx[y[r] + ((sc >> (8 * r)) & 0xffu)];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dstp[r] = (uint8_t)y[r];
+                continue;
+            }
             uint32_t packed = 0;
             const bool with_acc = POST >= 0 ? POST == 2 : L.acc_off >= 0;
             const bool with_post = POST >= 0 ? POST != 0 : L.has_post != 0;
@@ -397,10 +459,10 @@ template <bool STEM, int TP>
 __device__ __forceinline__ void conv_tiles_post(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
                                                 int n_waves)
 {
-    if (L.dst_off < 0) conv_tiles<STEM, TP, STEM ? 1 : 0, true, -1>(L, lds, tab, gout, tid, wave, n_waves);   // the model's output
-    else if (L.acc_off >= 0) conv_tiles_nm<STEM, TP, 2>(L, lds, tab, gout, tid, wave, n_waves);
-    else if (L.has_post) conv_tiles_nm<STEM, TP, 1>(L, lds, tab, gout, tid, wave, n_waves);
-    else conv_tiles_nm<STEM, TP, 0>(L, lds, tab, gout, tid, wave, n_waves);
+    // the model's output, and layers the short epilogue does not cover (rshift < 2): the general form
+    if (L.dst_off < 0 || L.idx_shift < 0) conv_tiles<STEM, TP, STEM ? 1 : 0, true, -1>(L, lds, tab, gout, tid, wave, n_waves);
+    else if (L.acc_off >= 0) conv_tiles_nm<STEM, TP, 4>(L, lds, tab, gout, tid, wave, n_waves);
+    else conv_tiles_nm<STEM, TP, 3>(L, lds, tab, gout, tid, wave, n_waves);
 }
 
 // waves [wave0, wave0 + n_waves) of the workgroup compute the layer (all 16 but for the first layer)
@@ -658,7 +720,9 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
             lds_filters += stem ? Co * 64 : (int)prepared_table_offset_u8(kh, kw, Co, Ci);
             if (i == 0) h.first_bytes = lds_filters;
             L.tab_off = tables;                    // relative to the table area, fixed up below
-            const int tb = 64 * Co + 4 * L.S_pad + 512;
+            L.geo_off = 64 * Co + 4 * L.S_pad + 512 + FIN_BYTES + 512;
+            const int tb = L.geo_off + ((Ho * Wo * 4 + 15) & ~15);
+            if ((tb >> 4) > NT) { set_error("%s: layer %d: tables of %d bytes (one 16-byte piece per thread)", op, i, tb); return fail(SMALL_HIP_EUNSUPPORTED); }
             L.tab16 = tb >> 4;
             tables += tb;
             max_t = tb > max_t ? tb : max_t;
@@ -676,6 +740,12 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
                 L.has_post = 1;
             }
         }
+        // the short epilogue: positive multiplier, rshift >= 2, the result stays in LDS (conv_tiles)
+        // (and the pixel table's 16-bit offsets must reach every pixel of the input and output tensors)
+        L.idx_shift = (!pool && L.q.fast && L.q.rshift >= 2 && l.dst != SMALL_HIP_QM_OUTPUT && (H + 2) * (W + 2) * 16 <= 0xffff &&
+                       (L.Ho + 2) * (L.Wo + 2) * 16 <= 0xffff)
+                          ? L.q.rshift - 2
+                          : -1;
         L.r_wo = 1.0f / (float)L.Wo;
         L.r_cob = 1.0f / (float)(L.Co / CB);
         L.wo_shift = -1;
@@ -790,7 +860,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
         // the end; post[t]: what Accum (t = convolution byte + shortcut byte) and / or the in-place ReLU make of a
         // convolution's byte.  Both are plain functions of the layer's constants: computed here, once.
         std::vector<uint8_t> &hb = host_tabs[(size_t)i];
-        hb.assign((size_t)(4 * L.S_pad + 512), 0);
+        hb.assign((size_t)(4 * L.S_pad + 512 + FIN_BYTES + 512 + ((L.Ho * L.Wo * 4 + 15) & ~15)), 0);
         int32_t *st = reinterpret_cast<int32_t *>(hb.data());
         const int CiB = L.kind == K_CONV ? L.Ci / CB : 1, Hp = L.H + 2, Wp = L.W + 2, S = L.kind == K_CONV ? L.kh * L.kw * CiB : 4;
         for (int k = 0; k < L.S_pad; ++k)
@@ -815,6 +885,35 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
                 y = requant_u8(z > 0 ? z : 0, L.q);
             }
             po[t] = (uint8_t)y;
+        }
+        // The short epilogue's tables.  With a positive multiplier and rshift >= 2 the requantised byte is a function of
+        // idx = product >> (30 + rshift) alone: idx = 2 q + b with q = v >> rshift and b = bit rshift - 1 of v, and the
+        // reference's result is clamp(q - b, 0, 255) (its rounding term is -1).  fin[clamp(idx, 0, 513)] is that byte after
+        // post[] and in the tensors' encoding (^ 0x80); in front of an Accum it is the plain byte, and postx[] is post[]
+        // in the tensors' encoding.
+        {
+            uint8_t *fin = po + 512, *postx = fin + FIN_BYTES;
+            for (int idx = 0; idx < FIN_ENTRIES; ++idx)
+            {
+                const int r = (idx >> 1) - (idx & 1);
+                const uint8_t y = (uint8_t)(r < 0 ? 0 : r > 255 ? 255 : r);
+                fin[idx] = pa.has_accum ? y : (uint8_t)((L.has_post ? po[y] : y) ^ 0x80u);
+            }
+            for (int t = 0; t < 512; ++t) postx[t] = (uint8_t)(po[t] ^ 0x80u);
+            // The pixel table: everything the kernel needs to know about output pixel p, as two 16-bit words: the LDS
+            // offset of its window origin in the input tensor's first channel block, and the offset of the pixel in the
+            // output tensor's first channel block (a multiple of 16) with its border case (the row of T) in the low four
+            // bits.  Two LDS reads from one address instead of some thirty vector instructions of index arithmetic per tile.
+            uint16_t *ge = reinterpret_cast<uint16_t *>(postx + 512);
+            const int Wop = L.Wo + 2, esz = L.kind == K_STEM ? 4 : 16;
+            for (int pp = 0; pp < L.Ho * L.Wo; ++pp)
+            {
+                const int oh = pp / L.Wo, ow = pp - oh * L.Wo;
+                const int ih0 = oh * L.stride - L.pt, iw0 = ow * L.stride - L.pl;
+                const int ra = (ih0 < 0 ? 2 : 0) + (ih0 + L.kh > L.H ? 1 : 0), rb = (iw0 < 0 ? 2 : 0) + (iw0 + L.kw > L.W ? 1 : 0);
+                ge[2 * pp + 0] = (uint16_t)(((ih0 + 1) * Wp + iw0 + 1) * esz);
+                ge[2 * pp + 1] = (uint16_t)((((oh + 1) * Wop + ow + 1) * 16) | (ra * 4 + rb));
+            }
         }
         e = hipMemcpyAsync(dblob + L.tab_off + 64 * L.Co, hb.data(), hb.size(), hipMemcpyHostToDevice, s);
         if (e != hipSuccess) return fail_dev(fail_hip(e, "small_hip_qmodel_create: tables"));
