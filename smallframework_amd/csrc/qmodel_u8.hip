@@ -459,7 +459,7 @@ template <bool STEM, int TP>
 __device__ __forceinline__ void conv_tiles_post(const QMLayer &L, uint8_t *lds, const uint8_t *tab, uint8_t *gout, int tid, int wave,
                                                 int n_waves)
 {
-    // the model's output, and layers the short epilogue does not cover (rshift < 2): the general form
+    // the model's output, and layers the short epilogue does not cover (rshift < 2, no room for a pixel table): the general form
     if (L.dst_off < 0 || L.idx_shift < 0) conv_tiles<STEM, TP, STEM ? 1 : 0, true, -1>(L, lds, tab, gout, tid, wave, n_waves);
     else if (L.acc_off >= 0) conv_tiles_nm<STEM, TP, 4>(L, lds, tab, gout, tid, wave, n_waves);
     else conv_tiles_nm<STEM, TP, 3>(L, lds, tab, gout, tid, wave, n_waves);
@@ -719,13 +719,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
             L.w_off = lds_filters;
             lds_filters += stem ? Co * 64 : (int)prepared_table_offset_u8(kh, kw, Co, Ci);
             if (i == 0) h.first_bytes = lds_filters;
-            L.tab_off = tables;                    // relative to the table area, fixed up below
-            L.geo_off = 64 * Co + 4 * L.S_pad + 512 + FIN_BYTES + 512;
-            const int tb = L.geo_off + ((Ho * Wo * 4 + 15) & ~15);
-            if ((tb >> 4) > NT) { set_error("%s: layer %d: tables of %d bytes (one 16-byte piece per thread)", op, i, tb); return fail(SMALL_HIP_EUNSUPPORTED); }
-            L.tab16 = tb >> 4;
-            tables += tb;
-            max_t = tb > max_t ? tb : max_t;
+            L.geo_off = 64 * Co + 4 * L.S_pad + 512 + FIN_BYTES + 512;     // the tables' offsets and sizes: assign_tables below
             const size_t need = stem ? (size_t)Co * (kh + 1) * (kw + 1) * 4 : prepared_bytes_u8(kh, kw, Co, Ci);
             scratch = need > scratch ? need : scratch;
             if (l.accum_src != SMALL_HIP_QM_NONE)
@@ -780,20 +774,42 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
     h.filter_bytes = lds_filters;
     h.later_kib = (lds_filters - h.first_bytes + 1023) >> 10;
     const int filters_end = h.first_bytes + (h.later_kib << 10);
-    int off = align_up(filters_end, 16);
-    h.tab_lds = off; h.tab_bytes = max_t; off += 2 * max_t;
-    int pool_c = 0;
-    for (int i = 0; i < n_layers; ++i)
-        if (h.layer[i].kind == K_POOL_AVG || h.layer[i].kind == K_POOL_MAX) pool_c = h.layer[i].Ci > pool_c ? h.layer[i].Ci : pool_c;
-    h.pool_off = off; off += align_up(pool_c * 4, 16);
     const small_hip_qlayer &l0 = layers[0];
     h.in_C = l0.input_channels; h.in_H = l0.input_height; h.in_W = l0.input_width;
     h.in_elems = h.in_C * h.in_H * h.in_W;
-    h.in_off = off;
-    off += align_up((h.in_C < CB ? 4 : h.in_C) * (h.in_H + 2) * (h.in_W + 2), 16);
     int tensor_off[MAX_TENSORS];
-    for (int t = 0; t < MAX_TENSORS; ++t) { tensor_off[t] = off; off += tensor_bytes[t]; }
-    h.lds_bytes = off;
+    int off = 0;
+    // The pixel tables of the short epilogue are the one part of the plan that is optional: a layer whose table would
+    // not fit the table fetch (one 16-byte piece per thread) goes without, and so do all layers when the model would not
+    // fit LDS with them; those layers take the general epilogue.
+    for (int with_pixels = 1; with_pixels >= 0; --with_pixels)
+    {
+        tables = 0; max_t = 0;
+        for (int i = 0; i < n_layers; ++i)
+        {
+            QMLayer &L = h.layer[i];
+            if (L.kind != K_STEM && L.kind != K_CONV) continue;
+            int tb = L.geo_off;
+            const int with_table = tb + ((L.Ho * L.Wo * 4 + 15) & ~15);
+            if (with_pixels && L.idx_shift >= 0 && (with_table >> 4) <= NT) tb = with_table;
+            else L.idx_shift = -1;
+            L.tab_off = tables;                    // relative to the table area, fixed up below
+            L.tab16 = tb >> 4;
+            tables += tb;
+            max_t = tb > max_t ? tb : max_t;
+        }
+        off = align_up(filters_end, 16);
+        h.tab_lds = off; h.tab_bytes = max_t; off += 2 * max_t;
+        int pool_c = 0;
+        for (int i = 0; i < n_layers; ++i)
+            if (h.layer[i].kind == K_POOL_AVG || h.layer[i].kind == K_POOL_MAX) pool_c = h.layer[i].Ci > pool_c ? h.layer[i].Ci : pool_c;
+        h.pool_off = off; off += align_up(pool_c * 4, 16);
+        h.in_off = off;
+        off += align_up((h.in_C < CB ? 4 : h.in_C) * (h.in_H + 2) * (h.in_W + 2), 16);
+        for (int t = 0; t < MAX_TENSORS; ++t) { tensor_off[t] = off; off += tensor_bytes[t]; }
+        h.lds_bytes = off;
+        if (off <= LDS_LIMIT) break;
+    }
     if (off > LDS_LIMIT)
     {
         set_error("%s: the model needs %d bytes of LDS (filters %d), the limit is %d: run it layer by layer", op, off,
@@ -860,7 +876,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
         // the end; post[t]: what Accum (t = convolution byte + shortcut byte) and / or the in-place ReLU make of a
         // convolution's byte.  Both are plain functions of the layer's constants: computed here, once.
         std::vector<uint8_t> &hb = host_tabs[(size_t)i];
-        hb.assign((size_t)(4 * L.S_pad + 512 + FIN_BYTES + 512 + ((L.Ho * L.Wo * 4 + 15) & ~15)), 0);
+        hb.assign((size_t)(L.tab16 * 16 - 64 * L.Co), 0);
         int32_t *st = reinterpret_cast<int32_t *>(hb.data());
         const int CiB = L.kind == K_CONV ? L.Ci / CB : 1, Hp = L.H + 2, Wp = L.W + 2, S = L.kind == K_CONV ? L.kh * L.kw * CiB : 4;
         for (int k = 0; k < L.S_pad; ++k)
@@ -906,7 +922,7 @@ int small_hip_qmodel_create(int n_layers, const small_hip_qlayer *layers, small_
             // bits.  Two LDS reads from one address instead of some thirty vector instructions of index arithmetic per tile.
             uint16_t *ge = reinterpret_cast<uint16_t *>(postx + 512);
             const int Wop = L.Wo + 2, esz = L.kind == K_STEM ? 4 : 16;
-            for (int pp = 0; pp < L.Ho * L.Wo; ++pp)
+            for (int pp = 0; L.idx_shift >= 0 && pp < L.Ho * L.Wo; ++pp)
             {
                 const int oh = pp / L.Wo, ow = pp - oh * L.Wo;
                 const int ih0 = oh * L.stride - L.pt, iw0 = ow * L.stride - L.pl;

@@ -128,3 +128,85 @@ def test_one_launch_graph_replays_match_eager(name, batch):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "graph replay %d differs from the eager launch" % rep
         assert np.unique(want.view(np.uint8)).size > 1
     ex.close()
+
+
+def _exposed_u8_net(hw, form):
+    """Two or three uint8 convolutions whose bytes stay between 0 and 255 (not saturated), followed by a 1x1 convolution
+    with an identity filter and a unit output scale, so that the model's output IS the last tensor, byte for byte:
+    form "plain": stem -> b0, 3x3 16->16 -> b1;  "relu": stem + in-place ReLU;  "accum": stem -> b0, 3x3 -> b1, 3x3 -> b2 +
+    Accum(b0) + ReLU.
+    -> (model, weights)."""
+    b = models._Builder("u8_exposed_%s_%d" % (form, hw), "u8", (3, hw, hw), "u8")
+    unit = (0, (1 << 31) - 1, 0, 0)
+    half = 1 << 30
+    b.advance(b.conv(16, 3, 1, "same", dst="b0"))
+    q = {"in": (-130, half + 777, 0, 0)}
+    if form == "relu":
+        b.eltwise("relu")
+        q.update(b0=(0, (1 << 31) - 1, 0, 2), b1=unit, b2=unit)
+        out = "b2"
+    elif form == "plain":
+        b.advance(b.conv(16, 3, 1, "same", src="b0", dst="b1"))
+        q.update(b0=(0, half + 12345, 0, 7), b1=(0, half + 54321, 0, 10), b2=unit)
+        out = "b2"
+    else:
+        # the Accum source (b0) may not be the convolution's own input: one more convolution in between
+        b.advance(b.conv(16, 3, 1, "same", src="b0", dst="b1"))
+        b.advance(b.conv(16, 3, 1, "same", src="b1", dst="b2"))
+        b.eltwise("accum", src="b0", dst="b2")
+        b.eltwise("relu")
+        q.update(b0=(0, half + 12345, 0, 7), b1=unit, b2=(0, (1 << 31) - 1, 0, 2))
+        out = "b1"
+    last = b.conv(16, 1, 1, "valid", src=b.cur, dst=out)
+    b.advance(last)
+    m = b.done()
+    m.quant.update(q)
+    for o in m.ops:
+        if o.weight:
+            m.quant[o.weight] = (-129, half, 0, 0)
+    m.quant[last.weight] = (0, half, 0, 0)
+    w = models.make_weights(m)
+    ident = np.zeros(16 * 16, np.uint8)          # packed 1x1 filter [16 ci][16 co]: 1 where ci == co, filter zero point 0
+    ident[np.arange(16) * 16 + np.arange(16)] = 1
+    w[last.weight] = ident
+    return m, w
+
+
+@pytest.mark.parametrize("form,hw", [
+    ("plain", 24), ("relu", 24), ("accum", 24),     # the short epilogue with its pixel tables in every layer but the last
+    ("plain", 60), ("relu", 60),                    # a pixel table of 3600 entries does not fit the table fetch: the general one
+])
+def test_u8_one_launch_epilogue_forms(form, hw, max_lds=163840):
+    """The uint8 one-launch kernel's short epilogue (a table indexed by the product's high word, pixel geometry from a
+    table, with and without ReLU / Accum) and the general one it falls back to, on tensors that are NOT saturated and
+    that the model hands out unchanged: the oracle's bytes."""
+    m, w = _exposed_u8_net(hw, form)
+    batch = 3
+    x = models.make_input(m, batch, seed=5)
+    want = OracleExecutor(m, batch, w, x).forward()
+    assert len(np.unique(want)) > 30, "the exposed tensor should hold many different bytes"
+    ex = models.HipExecutor(m, batch, w, x)
+    ex.build_one_launch()
+    lds = ex.one_launch_lds_bytes()
+    print("u8 net", form, hw, "LDS bytes", lds, "byte values", len(np.unique(want)), flush=True)
+    assert lds <= max_lds
+    ex.forward_one_launch()
+    got = ex.output_one_launch().copy()
+    ex.close()
+    assert_equal_exact(got, want, "u8 one launch, %s, %dx%d" % (form, hw, hw))
+
+
+def test_u8_one_launch_without_room_for_pixel_tables():
+    """A model that fits LDS only without the short epilogue's pixel tables is planned without them (and not refused)."""
+    m, w = _exposed_u8_net(50, "accum")
+    batch = 2
+    x = models.make_input(m, batch, seed=6)
+    ex = models.HipExecutor(m, batch, w, x)
+    ex.build_one_launch()
+    print("u8 net 50 LDS bytes", ex.one_launch_lds_bytes(), flush=True)
+    ex.forward_one_launch()
+    got = ex.output_one_launch().copy()
+    ex.close()
+    want = OracleExecutor(m, batch, w, x).forward()
+    assert_equal_exact(got, want, "u8 one launch without pixel tables")
+    assert len(np.unique(want)) > 30
