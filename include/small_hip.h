@@ -337,9 +337,13 @@ int small_hip_conv2d_u8(int batch, int kernel_height, int kernel_width, int stri
  * small_hip_conv2d_u8; the filter pre-pass writes into a static device array of
  * SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES bytes instead of an allocated block, and the call returns SMALL_HIP_EINVAL
  * when small_hip_conv2d_u8_prepared_filter_bytes(kh, kw, Co, Ci) exceeds that (input_channels of 1..3 need no
- * scratch at all).  It calls no hipMalloc / hipFree.  Every call on one GPU shares that GPU's array: calls that
- * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered by the stream.  Nothing in
- * the array has to start at zero: the pre-pass writes every byte the convolution reads. */
+ * scratch at all).  It calls no hipMalloc / hipFree.  Every call on one GPU shares that GPU's array.  Calls on one
+ * stream are ordered by the stream; calls on different streams or host threads are ordered by the library on the
+ * device (the later call's pre-pass waits for the earlier call's convolution through one event per GPU; no host
+ * wait), so they are safe but do not overlap.  A call recorded into a HIP graph is not ordered that way: a replay
+ * that overlaps another user of the array races, so keep replays and other calls on one stream or order them
+ * yourself; the first call on a GPU (symbol lookup, event creation) must come before any capture.  Nothing in the
+ * array has to start at zero: the pre-pass writes every byte the convolution reads. */
 #define SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES (4u << 20)
 int small_hip_conv2d_u8_noalloc(int batch, int kernel_height, int kernel_width, int stride, int t_pad,
                                 int b_pad, int l_pad, int r_pad, int output_channels, int input_channels,

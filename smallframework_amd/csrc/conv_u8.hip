@@ -541,11 +541,35 @@ int conv_u8_check(const char *op, int batch, int kh, int kw, int stride, int pt,
 constexpr size_t NOALLOC_SCRATCH_BYTES = size_t(SMALL_HIP_NOALLOC_MAX_PREPARED_BYTES);
 static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 
-int static_scratch(const char *op, size_t bytes, void **ptr)
+// Calls on different streams of one GPU share the array: the library orders them on the device (the later call's
+// pre-pass waits for the earlier call's convolution through one event per GPU, created at the first call; no host wait).
+// The lock is held from the wait to the record, so that two host threads cannot interleave their launches.  A call
+// recorded into a HIP graph is not ordered this way (an event of ordinary work must not enter a capture): replays that
+// overlap other users of the array are the caller's to order.
+struct StaticScratchUse
 {
-    constexpr int MAX_DEV = 64;
-    static std::mutex mu;
-    static void *addr[MAX_DEV] = {};
+    std::unique_lock<std::mutex> lock;
+    void *ptr = nullptr;
+    int dev = -1;
+    bool capturing = false;
+};
+struct StaticScratchState
+{
+    static constexpr int MAX_DEV = 64;
+    std::mutex mu;
+    void *addr[MAX_DEV] = {};
+    hipEvent_t done[MAX_DEV] = {};
+    hipStream_t last[MAX_DEV] = {};
+    bool pending[MAX_DEV] = {};
+};
+StaticScratchState &static_state()
+{
+    static StaticScratchState st;
+    return st;
+}
+
+int static_scratch_begin(const char *op, size_t bytes, hipStream_t s, StaticScratchUse *use)
+{
     if (bytes > NOALLOC_SCRATCH_BYTES)
     {
         set_error("%s: the prepared filter needs %zu bytes, the static scratch holds %zu (use "
@@ -555,16 +579,36 @@ int static_scratch(const char *op, size_t bytes, void **ptr)
     }
     int dev = 0;
     SHP_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= MAX_DEV) { set_error("%s: device index out of range", op); return SMALL_HIP_EINVAL; }
-    std::lock_guard<std::mutex> lk(mu);
-    if (!addr[dev])
+    if (dev < 0 || dev >= StaticScratchState::MAX_DEV) { set_error("%s: device index out of range", op); return SMALL_HIP_EINVAL; }
+    StaticScratchState &st = static_state();
+    use->lock = std::unique_lock<std::mutex>(st.mu);
+    use->dev = dev;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    SHP_HIP(hipStreamIsCapturing(s, &cs));
+    use->capturing = cs != hipStreamCaptureStatusNone;
+    if (!st.addr[dev])
     {
+        if (use->capturing)
+        { set_error("%s: the first call on a GPU looks up the static array and cannot be recorded into a graph: call once before the capture", op); return SMALL_HIP_EINVAL; }
         void *p = nullptr;
         SHP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));      // the current device's copy
         if (!p) { set_error("%s: hipGetSymbolAddress returned null", op); return SMALL_HIP_EHIP; }
-        addr[dev] = p;
+        SHP_HIP(hipEventCreateWithFlags(&st.done[dev], hipEventDisableTiming));
+        st.addr[dev] = p;
     }
-    *ptr = addr[dev];
+    if (!use->capturing && st.pending[dev] && st.last[dev] != s) SHP_HIP(hipStreamWaitEvent(s, st.done[dev], 0));
+    use->ptr = st.addr[dev];
+    return SMALL_HIP_OK;
+}
+
+// after the call's last launch has been enqueued on s
+int static_scratch_end(StaticScratchUse *use, hipStream_t s)
+{
+    if (use->capturing || use->dev < 0) return SMALL_HIP_OK;
+    StaticScratchState &st = static_state();
+    SHP_HIP(hipEventRecord(st.done[use->dev], s));
+    st.last[use->dev] = s;
+    st.pending[use->dev] = true;
     return SMALL_HIP_OK;
 }
 
@@ -668,9 +712,11 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
     if (P > 0x7fffffffL / 64) { set_error("%s: batch*Ho*Wo too large for one launch", op); return SMALL_HIP_EINVAL; }
     void *ws = nullptr;
     WorkspaceLease lease;            // held until the launches below are enqueued
+    StaticScratchUse use;            // the same for the static array
     if (static_ws)
     {
-        if (int rc = static_scratch(op, prepared_bytes(kh, kw, Co, Ci), &ws)) return rc;
+        if (int rc = static_scratch_begin(op, prepared_bytes(kh, kw, Co, Ci), s, &use)) return rc;
+        ws = use.ptr;
     }
     else
     {
@@ -678,7 +724,8 @@ int conv_u8(const char *op, int batch, int kh, int kw, int stride, int pt, int p
         ws = lease.ptr;
     }
     if (int rc = prepare_filter(kh, kw, Co, Ci, filt, ws, s)) return rc;
-    return conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s, grp);
+    if (int rc = conv_u8_run(op, batch, kh, kw, stride, pt, pb, pl, pr, Co, Ci, H, W, in, iq, ws, fq, out, oq, fz, s, grp)) return rc;
+    return static_ws ? static_scratch_end(&use, s) : SMALL_HIP_OK;
 }
 
 int fuse_check(const char *op, const uint8_t *accum_input, const small_hip_quant *accum_q, const void *out, Fuse *fz,

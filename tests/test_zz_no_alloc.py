@@ -1,6 +1,8 @@
 """small_hip_conv2d_u8_noalloc: the uint8 convolution for callers that cannot allocate device memory.  Its filter
 pre-pass writes into a static device array instead of an allocated block; results must equal small_hip_conv2d_u8
 bit for bit (and the oracle), on two calls in a row that share the array, the second one smaller."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -115,3 +117,33 @@ def test_noalloc_under_graph_capture(lib, oracle):
         assert rco == 0
         assert_equal_exact(got, want, "graph replay %d vs oracle" % rep)
         assert len(np.unique(want)) > 20
+
+
+def test_noalloc_two_streams_share_the_array(lib, oracle):
+    """Calls issued in turn on two streams (another filter each time, nothing waited for in between) are ordered by the
+    library on the device: every result equals the oracle's."""
+    import torch
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    batch, kh, kw, s, (pt, pb, pl, pr), Co, Ci, H, W = 2, 3, 3, 1, (1, 1, 1, 1), 64, 64, 20, 20
+    args = (batch, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W)
+    iq, fq, oq = hu.q(-120), hu.q(-131), hu.q(5, 1518500250, 0, 9)
+    x = synth.uniform_u8(31, batch * Ci * H * W)
+    dx = hu.dev(x)
+    n = batch * Co * H * W
+    jobs = []
+    torch.cuda.synchronize()
+    for i in range(8):
+        f = synth.uniform_u8(40 + i, Co * Ci * kh * kw)
+        df, dout = hu.dev(f), hu.dev_empty(n, np.uint8)
+        jobs.append((f, df, dout))
+    torch.cuda.synchronize()
+    for i, (f, df, dout) in enumerate(jobs):
+        st = (s1, s2)[i & 1]
+        rc = lib.small_hip_conv2d_u8_noalloc(*args, hu.ptr(dx), hu.qref(iq), hu.ptr(df), hu.qref(fq), hu.ptr(dout), hu.qref(oq),
+                                             C.c_void_p(st.cuda_stream))
+        assert rc == 0, lib.small_hip_last_error()
+    torch.cuda.synchronize()
+    for i, (f, df, dout) in enumerate(jobs):
+        rco, want = oracle.conv2d_u8(batch, CB, kh, kw, s, pt, pb, pl, pr, Co, Ci, H, W, x, _oq(iq), f, _oq(fq), _oq(oq))
+        assert rco == 0
+        assert_equal_exact(hu.host(dout), want, "call %d on stream %d" % (i, i & 1))
