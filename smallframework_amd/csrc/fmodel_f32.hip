@@ -14,7 +14,7 @@
 //   depthwise 3x3 -> 1x1 convolution        one layer: a lane's depthwise results ARE its MFMA operand of the 1x1
 //                                           convolution (the same pixel, the same four channels), so the depthwise
 //                                           tensor is never stored and its arithmetic issues between the MFMAs
-//   whole-image average / max pooling       partial sums per pixel slice, then a fixed-order sum (deterministic)
+//   whole-image average / max pooling       a wave per channel quad: lanes fold pixels, then xor-shuffles (deterministic)
 // A fully connected layer is the 1x1 convolution on the 1x1 image pooling leaves.
 //
 // LDS layout of an activation tensor: [C/16][P][16] floats, the four channel quads of pixel p stored in the order
@@ -512,45 +512,37 @@ __device__ __forceinline__ float4 pool_op(bool is_max, float4 acc, float4 v)
 }
 
 // window == whole image, no padding (AveragePool2D: sum * float(1 / (H * W)), abstract_layer.hpp:514-569).
-// Three stages in a fixed order (deterministic): every thread folds a slice of the pixels, eight threads per channel
-// quad fold the slices, one thread folds those eight.
+// A wave owns a channel quad (wave, wave + 16, ...): its lanes fold the pixels lane, lane + 64, ... in that order, then
+// the wave folds its 64 partial sums with xor-shuffles (32, 16, ... 1): a fixed order (deterministic), no barrier and no
+// LDS staging inside the layer.  (Three stages through LDS with two barriers took 2.4 us of the DS-CNN's 27.)
 __device__ __forceinline__ void pool_layer(const FMLayer &L, float *lds, float *part, float *gout, int tid)
 {
+    (void)part;
     const int C4 = L.Ci / 4, P = L.H * L.W;
-    const int slices = NT / C4;                    // C <= 4096 is checked when the model is created
     const bool is_max = L.kind == K_POOL_MAX;
     const float *src = lds + L.src_off;
-    const int c4 = tid % C4, slice = tid / C4;
-    const int cb = c4 >> 2, q = c4 & 3;
-    if (slice < slices)
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int c4 = wave; c4 < C4; c4 += NW)
     {
+        const int cb = c4 >> 2, q = c4 & 3;
+        // a lane without a pixel holds the operation's neutral element: pixel 0 again for the maximum, zero for the sum
         float4 acc = is_max ? *reinterpret_cast<const float4 *>(src + apos(cb, P, 0, q)) : make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int p = slice; p < P; p += slices)
+        for (int p = lane; p < P; p += WAVE)
             acc = pool_op(is_max, acc, *reinterpret_cast<const float4 *>(src + apos(cb, P, p, q)));
-        *reinterpret_cast<float4 *>(part + (slice * C4 + c4) * 4) = acc;
-    }
-    __syncthreads();
-    // second stage: [8][C4] partials behind the first stage's when there are at least 16 slices (C <= 256); with fewer,
-    // slice 0's thread folds the rest into its own slot
-    const int fold = slices >= 16 ? 8 : 1;
-    float *part2 = fold > 1 ? part + NT * 4 : part;
-    if (slice < fold)
-    {
-        float4 acc = *reinterpret_cast<const float4 *>(part + (slice * C4 + c4) * 4);
-        for (int s = slice + fold; s < slices; s += fold)
-            acc = pool_op(is_max, acc, *reinterpret_cast<const float4 *>(part + (s * C4 + c4) * 4));
-        if (fold > 1) *reinterpret_cast<float4 *>(part2 + (slice * C4 + c4) * 4) = acc;
-        else *reinterpret_cast<float4 *>(part2 + c4 * 4) = acc;
-    }
-    __syncthreads();
-    if (tid < C4)
-    {
-        float4 acc = *reinterpret_cast<const float4 *>(part2 + tid * 4);
-        for (int s = 1; s < fold; ++s)
-            acc = pool_op(is_max, acc, *reinterpret_cast<const float4 *>(part2 + (s * C4 + tid) * 4));
-        if (!is_max) { acc.x *= L.norm; acc.y *= L.norm; acc.z *= L.norm; acc.w *= L.norm; }
-        if (L.dst_off >= 0) *reinterpret_cast<float4 *>(lds + L.dst_off + apos(cb, 1, 0, q)) = acc;
-        else *reinterpret_cast<float4 *>(gout + (size_t)cb * CB + 4 * q) = acc;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1)
+        {
+            const float4 o = make_float4(__shfl_xor(acc.x, d, WAVE), __shfl_xor(acc.y, d, WAVE), __shfl_xor(acc.z, d, WAVE),
+                                         __shfl_xor(acc.w, d, WAVE));
+            acc = pool_op(is_max, acc, o);
+        }
+        if (lane == 0)
+        {
+            if (!is_max) { acc.x *= L.norm; acc.y *= L.norm; acc.z *= L.norm; acc.w *= L.norm; }
+            if (L.dst_off >= 0) *reinterpret_cast<float4 *>(lds + L.dst_off + apos(cb, 1, 0, q)) = acc;
+            else *reinterpret_cast<float4 *>(gout + (size_t)cb * CB + 4 * q) = acc;
+        }
     }
 }
 
