@@ -96,3 +96,22 @@ def test_workspace_queries_without_gpu():
     assert lib.small_hip_conv2d_f32_workspace_bytes(16, 3, 3, 1, 1, 1, 1, 1, 1024, 1024, 13, 13) > 1 << 20
     assert lib.small_hip_conv2d_f32_workspace_bytes(64, 1, 1, 1, 0, 0, 0, 0, 512, 512, 14, 14) == 0
     assert lib.small_hip_conv2d_f32_workspace_bytes(16, 3, 3, 1, 1, 1, 1, 1, 16, 3, 416, 416) == 0
+
+
+def test_every_tune_key_in_the_sources_is_documented():
+    """SMALL_HIP_TUNE keys: every key the kernels' host code or the C++ wrappers read is listed in the comment above
+    tune_int (csrc/common.h), and every key listed there is read somewhere."""
+    import glob
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    used = set()
+    for path in glob.glob(os.path.join(root, "smallframework_amd", "csrc", "*.hip")) + \
+            glob.glob(os.path.join(root, "include", "small", "*.hpp")) + glob.glob(os.path.join(root, "include", "small", "*", "*.hpp")):
+        used.update(re.findall(r'tune_(?:int|pair)\("([a-z_0-9]+)"', open(path).read()))
+    text = open(os.path.join(root, "smallframework_amd", "csrc", "common.h")).read()
+    block = text[text.index("// Measurement switches"):text.index("int tune_int(")]
+    documented = set(re.findall(r"\b([a-z]+(?:_[a-z0-9]+)+)(?==|\b)", block)) & (used | set(re.findall(r"([a-z_0-9]+)=", block)))
+    assert used, "no keys found: the pattern no longer matches the sources"
+    assert used <= documented, "read but not documented: %s" % sorted(used - documented)
+    listed = (set(re.findall(r"([a-z_0-9]+)=", block)) | {"conv_streamk_min", "convq_min_wg", "convq_table_min_wg", "fuse_pool"}) - {"key"}
+    assert listed <= used, "documented but never read: %s" % sorted(listed - used)
