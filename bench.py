@@ -111,7 +111,7 @@ def emit(out, tag):
             # bandwidth-bound layers against a kernel that only moves their bytes (same place in the model)
             summary["headline_layers"].update({"bandwidth_layers": len(fl), "of_bytes_only_kernel_min": fl[0],
                                                "of_bytes_only_kernel_median": round(statistics.median(fl), 3)})
-    for k in ("mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "mfma_and_vector_alu_same_simd", "hip_graph_ms_per_step",
+    for k in ("fresh_process_ms_per_step", "mfma_f32_sustained_TFLOPs", "hbm_copy_sustained_GBs", "mfma_and_vector_alu_same_simd", "hip_graph_ms_per_step",
               "host_buffers_ms_per_step", "host_buffers_images_per_s", "host_buffers_serial_ms_per_step",
               "host_buffers_result_unchanged"):
         if k in extras:
@@ -151,11 +151,11 @@ DEFAULT_COUNTS = {"mobilenet_v1": (200, 100), "tiny_yolo_v2": (200, 100), "layer
 
 
 def counts_for(step_fn, args, at_least=0):
-    """(timed steps, warm-up steps) for a side measurement.  With counts on the command line: those.  Otherwise from
-    the duration of `step_fn` (3 + 10 probe calls), so that the warm-up is about 100 ms of load and the timed region
-    about 200 ms whatever the model's size."""
-    if not args.auto_counts:
-        return max(args.steps, at_least), args.warmup
+    """(timed steps, warm-up steps) for a side measurement, from the duration of `step_fn` (3 + 10 probe calls): the
+    warm-up is about 100 ms of load and the timed region about 200 ms whatever the model's size, and never fewer than
+    the counts on the command line.  (The command line's counts are the headline's; a side configuration is built after
+    host work during which the GPU idles, and 5 + 20 passes of a small model would time the machine's way back from
+    idle, not the kernels.)"""
     import torch
     for _ in range(3):
         step_fn()
@@ -165,7 +165,10 @@ def counts_for(step_fn, args, at_least=0):
         step_fn()
     torch.cuda.synchronize()
     est = max((time.perf_counter() - t0) / 10, 1e-6)
-    return min(8000, max(200, int(0.2 / est) + 1)), min(4000, max(100, int(0.1 / est) + 1))
+    k, w = min(8000, max(200, int(0.2 / est) + 1)), min(4000, max(100, int(0.1 / est) + 1))
+    if not args.auto_counts:
+        k, w = max(k, args.steps), max(w, args.warmup)
+    return max(k, at_least), w
 
 
 def time_forward(ex, steps, warmup):
@@ -555,9 +558,9 @@ def sweep_only(args, torch, models):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults (DEFAULT_COUNTS): the GPU reaches its sustained clock only after some tens of milliseconds of load
-    # (MobileNetV1 batch 64: 1.05 ms/step over steps 4..23 of a fresh process, 1.00 ms/step from step 50 on), so the
-    # default warm-up is about 100 ms of forward passes and the timed region about 200 ms
+    # defaults (DEFAULT_COUNTS): a GPU that has idled needs some tens of milliseconds of convolution load to reach its
+    # sustained state (see the order of the measurements in main), so the default warm-up is about 100 ms of forward
+    # passes and the timed region about 200 ms
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--model", default="mobilenet_v1",
@@ -595,12 +598,20 @@ def main():
     x = models.make_input(model, batch)
     ex = models.HipExecutor(model, batch, weights, x, fused=not args.unfused)
 
-    # The machine calibration runs first (float32 MFMA on registers only, a device-to-device copy: about 60 ms of load
-    # whose figures the per-layer tables are read against), so the GPU is in its sustained state when the warm-up
-    # steps start; a fresh process otherwise spends its first tens of milliseconds of load below its sustained clock,
-    # which is what 5 + 20 steps of a 0.9 ms pass would measure.
+    # Order of the measurements.  A GPU that has been idle runs its first 30-odd forward passes up to 12% slower, whatever
+    # ran before that was not convolution-like: half a second of MFMA instructions on registers or of device copies
+    # leaves the ramp in place, 100 passes of any convolution model (this one on other buffers, another model) remove
+    # it, and the core clock the driver reports stays at 2.36-2.38 GHz throughout.  So the state is the machine's, not
+    # this process's or these buffers', and every figure that is read against a roofline has to be taken in it:
+    #   1. the first `warmup` + `steps` passes of the process, reported beside the headline as the fresh-process figure;
+    #   2. machine calibration (float32 MFMA on registers only, a device-to-device copy, the issue probe);
+    #   3. the per-layer pass (HIP events around every launch, at least 60 passes; medians);
+    #   4. `warmup` untimed and `steps` timed passes: the headline.
     calib = {}
+    fresh = None
     if model.dtype == "f32" and not args.no_extras:
+        fresh = time_forward(ex, args.steps, args.warmup)
+        log("%s: %.3f ms/step over the first %d + %d passes of the process" % (model.name, fresh * 1e3, args.warmup, args.steps))
         sustained = mfma_probe_tflops()
         if sustained is not None:
             calib["mfma_f32_sustained_TFLOPs"] = round(sustained, 1)
@@ -608,6 +619,9 @@ def main():
         ov = issue_overlap_us()
         if ov is not None:
             calib["mfma_and_vector_alu_same_simd"] = ov
+    # per-op device times (HIP events on the launch stream); the headline-only runs the profile commands make keep to
+    # the command line's count
+    ms = time_ops(ex, min(args.steps, 200) if args.no_extras else max(60, min(args.steps, 200)))
     sec = time_forward(ex, args.steps, args.warmup)
     one_launch = None
     if model.dtype == "u8" or model.name == "dscnn":
@@ -621,8 +635,6 @@ def main():
     ips = batch / sec
     log("%s: %.3f ms/step, %.1f images/s" % (model.name, sec * 1e3, ips))
 
-    # per-op device times (HIP events on the launch stream) over the same number of steps
-    ms = time_ops(ex, min(args.steps, 200))
     table = layer_table(model, batch, ms)
     if not args.no_extras:
         # what a kernel that only moves each bandwidth-bound layer's bytes takes in the same place of the model
@@ -709,6 +721,7 @@ def main():
     if model.dtype == "f32" and not args.no_extras:
         # what the float32 matrix pipes sustain on registers alone, beside the published peak used in `roofline`
         extras.update(calib)
+        extras["fresh_process_ms_per_step"] = round(fresh * 1e3, 4)
         # the same forward pass replayed from a HIP graph (no host work between the launches)
         ex.capture()
         for _ in range(args.warmup):
@@ -913,8 +926,10 @@ def main():
             "whole model in one launch" if one_launch else
             "Conv2D+bias+activation fused" if not args.unfused else "unfused layer calls"),
             "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4),
-            "before_warmup": ("machine calibration (MFMA probe, device copy: ~60 ms of load), then `warmup` untimed and "
-                              "`steps` timed forward passes") if calib else "nothing"},
+            "before_warmup": ("the process's first `warmup` + `steps` passes (summary.fresh_process_ms_per_step), machine "
+                              "calibration (MFMA probe, device copy), the per-layer pass (60+ passes with an event "
+                              "after every launch); then `warmup` untimed and `steps` timed forward passes"
+                              if calib else "the per-layer pass (`steps` passes with an event after every launch)")},
         "roofline": roof,
         "cpu_baseline": cpu,
         "layers": table,
