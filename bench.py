@@ -621,7 +621,8 @@ def main():
             calib["mfma_and_vector_alu_same_simd"] = ov
     # per-op device times (HIP events on the launch stream); the headline-only runs the profile commands make keep to
     # the command line's count
-    ms = time_ops(ex, min(args.steps, 200) if args.no_extras else max(60, min(args.steps, 200)))
+    layer_passes = min(args.steps, 200) if args.no_extras else max(60, min(args.steps, 200))
+    ms = time_ops(ex, layer_passes)
     sec = time_forward(ex, args.steps, args.warmup)
     one_launch = None
     if model.dtype == "u8" or model.name == "dscnn":
@@ -926,10 +927,10 @@ def main():
             "whole model in one launch" if one_launch else
             "Conv2D+bias+activation fused" if not args.unfused else "unfused layer calls"),
             "batch": batch, "GFLOP_per_image": round(model.flops_per_image() / 1e9, 4),
-            "before_warmup": ("the process's first `warmup` + `steps` passes (summary.fresh_process_ms_per_step), machine "
-                              "calibration (MFMA probe, device copy), the per-layer pass (60+ passes with an event "
-                              "after every launch); then `warmup` untimed and `steps` timed forward passes"
-                              if calib else "the per-layer pass (`steps` passes with an event after every launch)")},
+            "before_warmup": (("the process's first `warmup` + `steps` passes (summary.fresh_process_ms_per_step), machine "
+                               "calibration (MFMA probe, device copy), " if calib else "") +
+                              "the per-layer pass (%d passes with an event after every launch); then `warmup` untimed and "
+                              "`steps` timed forward passes" % layer_passes)},
         "roofline": roof,
         "cpu_baseline": cpu,
         "layers": table,
