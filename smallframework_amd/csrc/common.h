@@ -24,6 +24,7 @@ void set_error(const char *fmt, ...);
 // Nothing in production needs it; every default is the measured best.  Keys (integers unless noted):
 //   conv_tile=CxP     force the float32 convolution's wave tile (1x1 1x2 2x1 2x2)
 //   conv_tail=0|2     never / always cut left-over tiles into split-K pieces        conv_pw=0   general K loop for 1x1
+//   conv_buf=0        operand streams through flat addresses instead of buffer loads (then conv_pw picks the 1x1 loop)
 //   conv_splitk=0|1   force the split-K kernel off / on                             conv_streamk=0|N  equal-share split off / N per CU
 //   conv_streamk_min  least K-steps for the equal-share split                       stem_lds=0  first layers without the LDS kernel
 //   stem_vec=0|1      16-byte staging of first-layer patches                        smallci_valu=1  vector-ALU first layers

@@ -268,7 +268,17 @@ constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks
 // BLDS: the workgroup runs this body once; its bias values are requested first of all and parked in LDS under the K loop, so
 // the epilogue does not wait for memory once more (a caller that runs several tiles per workgroup would overwrite them
 // while another wave still reads)
-template <int COT, int PXT, bool POOL = false, bool PW = false, bool BLDS = false>
+// BUF: both operand streams come through buffer loads (a resource descriptor per tensor, a 32-bit byte offset per lane, the
+// channel block's offset in a scalar register).  A tap outside the image, a pixel past the end and a step past the last
+// are then an offset the hardware finds out of range and answers with zeros, and a lane's offsets change only when the
+// window position does (once in Ci/16 steps): a K-step issues no vector-ALU instruction for its addresses.  The
+// launcher allows it for tensors of at most 1 GiB (lane offset + scalar offset + 16 stays below 2^31 on either side of
+// the range check, whether or not the hardware adds the scalar offset before it checks).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned BUF_OUT_OF_RANGE = 0x80000000u;
+constexpr long long BUF_MAX_BYTES = 1ll << 30;
+
+template <int COT, int PXT, bool POOL = false, bool PW = false, bool BLDS = false, bool BUF = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
                                               const int cg, const int pxb, const int s_begin = 0, const int s_count = -1,
                                               float *raw = nullptr)
@@ -294,6 +304,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
+    unsigned lane_base[PXT];     // BUF: byte offset of (image, channel half) in the input tensor
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
@@ -319,6 +330,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        lane_base[t] = (unsigned)(((size_t)n * CiB * in_blk + half * 8) * sizeof(float));
         // PW: the pixel's own position (a pixel past the end reads pixel 0 of image 0 and stores nothing)
         if (PW) in_img[t] += (size_t)(oh * a.W + ow) * CB;
     }
@@ -332,6 +344,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // would then have to wait at the top of the loop for loads issued only a step earlier.
     static_assert(A_VECS >= 256 ? A_VECS % 256 == 0 : 256 % A_VECS == 0, "filter vectors vs workgroup size");
     const float *a_src[A_PER_THREAD];
+    unsigned a_voff[A_PER_THREAD];
     int a_dst[A_PER_THREAD];
 #pragma unroll
     for (int j = 0; j < A_PER_THREAD; ++j)
@@ -341,6 +354,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
         int cob = cg * COT * 2 + blk;
         cob = cob < CoB ? cob : CoB - 1;                  // rows past Co: garbage, never stored
         a_src[j] = a.filt + (size_t)cob * CiB * taps * (CB * CB) + within * 4;
+        a_voff[j] = (unsigned)(((size_t)cob * CiB * taps * (CB * CB) + within * 4) * sizeof(float));
         a_dst[j] = blk * A_TILE_FLOATS + within * 4;
     }
     // read position of this lane inside a staged tile pair
@@ -367,7 +381,61 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
     // launcher guarantees fit): a K-step is then one basic block and the compiler can slot this
     // address arithmetic between the MFMAs instead of running it after them.
     const int in_blk32 = a.H * a.W * CB;
+    // BUF: the window position's lane offsets, recomputed only when the position moves
+    unsigned voff[PXT];
+    auto tap_offsets = [&]() {
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = live && pvalid[t] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+            voff[t] = ok ? lane_base[t] + (unsigned)((ih * a.W + iw) * (CB * (int)sizeof(float))) : BUF_OUT_OF_RANGE;
+        }
+    };
+    __amdgpu_buffer_rsrc_t rsrc_in, rsrc_f;
+    if (BUF)
+    {
+        rsrc_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.in), 0,
+                                                    (int)((size_t)a.batch * a.Ci * a.H * a.W * sizeof(float)), 0x00020000);
+        rsrc_f = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.filt), 0,
+                                                   (int)((size_t)CoB * CiB * taps * (CB * CB) * sizeof(float)), 0x00020000);
+        tap_offsets();
+    }
     auto fetch = [&](float4 (&Areg)[A_PER_THREAD], float4 (&B)[PXT][2]) {
+        if (BUF)
+        {
+            const int soff_a = (cib * taps + ta * a.kw + tb) * (CB * CB * (int)sizeof(float));
+#pragma unroll
+            for (int j = 0; j < A_PER_THREAD; ++j)
+                Areg[j] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_f, a_voff[j], soff_a, 0));
+            const int soff_b = cib * (in_blk32 * (int)sizeof(float));
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                B[t][0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_in, voff[t], soff_b, 0));
+                B[t][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_in, voff[t] + 16, soff_b, 0));
+            }
+            // next (tap, channel block); the wave-uniform branch is taken once in Ci/16 steps.  Past the last step the
+            // position stays and the lanes' offsets go out of range (zeros that are staged and never multiplied)
+            if (++cib == CiB)
+            {
+                cib = 0;
+                if (++tb == a.kw)
+                {
+                    tb = 0;
+                    ++ta;
+                }
+                if (ta >= a.kh)
+                {
+                    ta = a.kh - 1;
+                    tb = a.kw - 1;
+                    cib = CiB - 1;
+                    live = false;
+                }
+                tap_offsets();
+            }
+            return;
+        }
         if (PW)
         {
             const int woff = cib * (CB * CB);
@@ -480,7 +548,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
 // The second launch bound (minimum waves per SIMD: 6 / 5 / 2 for one / two / four MFMA tiles per
 // wave) makes the compiler keep the accumulators in the unified register file and pack tighter
 // (2x1: 108 -> 76 registers, 2x2: 184 -> 131, no spills); measured 1-3% faster, tighter bounds spill.
-template <int COT, int PXT, bool POOL = false, bool PW = false>
+template <int COT, int PXT, bool POOL = false, bool PW = false, bool BUF = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_lds_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -488,7 +556,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;            // whole workgroup leaves together: no barrier is skipped
-    conv_lds_tile<COT, PXT, POOL, PW, true>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+    conv_lds_tile<COT, PXT, POOL, PW, true, BUF>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -515,6 +583,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
+    unsigned lane_base[PXT];     // BUF: byte offset of (image, channel half) in the input tensor
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
@@ -540,6 +609,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        lane_base[t] = (unsigned)(((size_t)n * CiB * in_blk + half * 8) * sizeof(float));
     }
     const float *w_row[COT];
 #pragma unroll
@@ -670,7 +740,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
 // single 32x32 tiles, each multiplied by one workgroup whose four waves split the reduction, i.e.
 // 4*COT*PXT times as many workgroups that each last 1/(4*COT*PXT) as long and spread over every CU.
 // The hardware starts workgroups in block-id order, so the tail follows the whole rounds.
-template <int COT, int PXT, bool POOL = false, bool PW = false>
+template <int COT, int PXT, bool POOL = false, bool PW = false, bool BUF = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_hybrid_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -681,7 +751,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     {
         // n_main is a multiple of NUM_XCD: consecutive logical ids share an XCD
         const int lid = (bid % NUM_XCD) * (a.n_main / NUM_XCD) + bid / NUM_XCD;
-        conv_lds_tile<COT, PXT, POOL, PW, true>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
+        conv_lds_tile<COT, PXT, POOL, PW, true, BUF>(a, lds_a, lid % a.n_co_groups, lid / a.n_co_groups);
         return;
     }
     constexpr int SUB = 4 * COT * PXT;            // 32x32 tiles per whole workgroup tile
@@ -708,7 +778,7 @@ constexpr int SK_CHUNKS = 2 * NUM_CU;
 template <int COT, int PXT>
 constexpr int sk_part_floats() { return 4 * COT * PXT * 16 * WAVE; }
 
-template <int COT, int PXT>
+template <int COT, int PXT, bool BUF = false>
 __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2)) void conv_mfma_f32_streamk_kernel(const ConvArgs a)
 {
     __shared__ float lds_a[2][COT * 2 * A_TILE_FLOATS];
@@ -730,7 +800,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
             const int first = (int)(((long)tile * nsteps) / a.sk_chunk);          // the run that starts the tile
             raw = a.sk_scratch + ((size_t)tile * a.sk_parts + (lid - first)) * sk_part_floats<COT, PXT>();
         }
-        conv_lds_tile<COT, PXT>(a, lds_a, tile % a.n_co_groups, tile / a.n_co_groups, sb, cnt, raw);
+        conv_lds_tile<COT, PXT, false, false, false, BUF>(a, lds_a, tile % a.n_co_groups, tile / a.n_co_groups, sb, cnt, raw);
         k0 += cnt;
         __syncthreads();                                              // the next tile stages into the same LDS buffers
     }
@@ -1606,6 +1676,16 @@ bool tail_pays(int n_main, int rest, int nsteps)
     return knob == 2 || rest <= NUM_CU / 2;
 }
 
+// Operand streams through buffer loads (conv_lds_tile's BUF form)?  An ordinary convolution (no slabs) whose input and
+// filter are at most BUF_MAX_BYTES each; SMALL_HIP_TUNE key conv_buf=0 keeps the flat-address form.
+bool buffer_form(const ConvArgs &a)
+{
+    static const bool off = tune_int("conv_buf", 1) == 0;
+    const long long in_bytes = (long long)a.batch * a.Ci * a.H * a.W * (long long)sizeof(float);
+    const long long f_bytes = (long long)((a.Co + CB - 1) / CB * CB) * a.Ci * a.kh * a.kw * (long long)sizeof(float);
+    return !off && a.slabs == 0 && in_bytes <= BUF_MAX_BYTES && f_bytes <= BUF_MAX_BYTES;
+}
+
 template <int COT, int PXT>
 void launch_mfma(ConvArgs &a, hipStream_t s)
 {
@@ -1616,7 +1696,10 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
     // pointwise form of the main loop (SMALL_HIP_TUNE key conv_pw=0 switches it off)
     static const bool pw_off = tune_int("conv_pw", 1) == 0;
-    const bool pw = !pw_off && a.kh == 1 && a.kw == 1 && a.stride == 1 && a.stride_h == 1 && a.pt == 0 && a.pl == 0 &&
+    // (only where the buffer-load form is not allowed: that one needs no special case for 1x1 windows and is faster,
+    // MobileNetV1 batch 64: 512 -> 512 @14x14 55.8 -> 52.5 us, 1024 -> 1024 @7x7 64.4 -> 54.9 us)
+    const bool buf = buffer_form(a);
+    const bool pw = !buf && !pw_off && a.kh == 1 && a.kw == 1 && a.stride == 1 && a.stride_h == 1 && a.pt == 0 && a.pl == 0 &&
                     a.Ho == a.H && a.Wo == a.W;
     const unsigned slabs_y = a.slabs > 0 ? a.slabs : 1;
     if (tail_pays<COT, PXT>(n_main, rest, a.kh * a.kw * (a.Ci / CB)))
@@ -1624,12 +1707,14 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
         a.n_main = n_main;
         const dim3 grid(n_main + rest * 4 * COT * PXT, slabs_y);
         if (pw) hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, false, true>), grid, dim3(256), 0, s, a);
+        else if (buf) hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, false, false, true>), grid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT>), grid, dim3(256), 0, s, a);
     }
     else
     {
         const dim3 grid(a.per_xcd * NUM_XCD, slabs_y);
         if (pw) hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, false, true>), grid, dim3(256), 0, s, a);
+        else if (buf) hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, false, false, true>), grid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT>), grid, dim3(256), 0, s, a);
     }
 }
@@ -1678,7 +1763,8 @@ int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
     WorkspaceLease lease;            // held until both launches are enqueued
     if (int rc = lease_workspace(bytes, s, &lease)) return rc;
     a.sk_scratch = static_cast<float *>(lease.ptr);
-    hipLaunchKernelGGL((conv_mfma_f32_streamk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    if (buffer_form(a)) hipLaunchKernelGGL((conv_mfma_f32_streamk_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_mfma_f32_streamk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
     SHP_LAUNCH_CHECK(op);
     hipLaunchKernelGGL((conv_streamk_fixup_kernel<COT, PXT>), dim3(a.n_blocks), dim3(256), 0, s, a);
     SHP_LAUNCH_CHECK(op);
@@ -1839,10 +1925,11 @@ void launch_mfma_pool(ConvArgs &a, hipStream_t s)
     if (tail_pays<COT, PXT>(n_main, rest, a.kh * a.kw * (a.Ci / CB)))
     {
         a.n_main = n_main;
-        hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, true>), dim3(n_main + rest * 4 * COT * PXT), dim3(256), 0, s, a);
+        if (buffer_form(a)) hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, true, false, true>), dim3(n_main + rest * 4 * COT * PXT), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((conv_mfma_f32_hybrid_kernel<COT, PXT, true>), dim3(n_main + rest * 4 * COT * PXT), dim3(256), 0, s, a);
     }
-    else
-        hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    else if (buffer_form(a)) hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true, false, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_mfma_f32_lds_kernel<COT, PXT, true>), dim3(a.per_xcd * NUM_XCD), dim3(256), 0, s, a);
 }
 
 // Conv2D + bias + activation + MaxPool2D 2x2 stride 2 (no pool padding) in one launch
