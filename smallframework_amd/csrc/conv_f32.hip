@@ -61,7 +61,17 @@ struct ConvArgs
     // ([tile][part < sk_parts][SK_PART_FLOATS]) for conv_streamk_fixup_kernel to add up in run order
     int sk_chunk, sk_chunks, sk_parts;
     float *sk_scratch;
+    // pixel index -> (image, row, column) without run-time divisions (conv_lds_tile, conv_splitk_tile): by Ho*Wo and Wo, in
+    // the pooling form by (Ho/2)*(Wo/2) and Wo/2
+    FastDiv fd_plane, fd_row;
 };
+
+void set_pixel_divisors(ConvArgs &a, bool pool)
+{
+    const int Wr = pool ? a.Wo >> 1 : a.Wo, Hr = pool ? a.Ho >> 1 : a.Ho;
+    a.fd_plane = make_fast_div((unsigned)(Hr * Wr > 0 ? Hr * Wr : 1));
+    a.fd_row = make_fast_div((unsigned)(Wr > 0 ? Wr : 1));
+}
 
 // the arguments of this workgroup's slab (uniform per workgroup: three scalar pointer additions)
 __device__ __forceinline__ ConvArgs slab_args(ConvArgs a)
@@ -107,6 +117,12 @@ __device__ __forceinline__ float act_k(float v, float neg_scale)
 {
     return RELU ? fmaxf(v, 0.f) : act_bf(v, neg_scale);
 }
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned BUF_OUT_OF_RANGE = 0x80000000u;
+constexpr long long BUF_MAX_BYTES = 1ll << 30;
+constexpr int BUF_RSRC_FLAGS = 0x00020000;            // raw buffer of 32-bit elements
+constexpr unsigned BUF_SCALAR_OUT_OF_RANGE = 1u << 30; // a scalar offset that puts every lane out of range (>= BUF_MAX_BYTES)
 
 // accumulate / bias / activation in registers, then 16-byte stores: a lane holds channels
 // 8q + 4*half + {0..3} of its pixel in accumulator registers 4q .. 4q+3.  Straight-line code:
@@ -186,17 +202,72 @@ __device__ __forceinline__ void conv_epilogue(const ConvArgs &a, floatx16 (&acc)
     else conv_epilogue_impl<COT, PXT, false, false>(a, acc, cg, half, HoWo, pvalid, out_pix, lds_bias);
 }
 
+// The same through buffer stores (conv_lds_tile's BUF form).  ovoff: the lane's byte offset of (pixel, channel 4 * half of
+// channel block 0) in the output tensor, or BUF_OUT_OF_RANGE for a lane that stores nothing; the channel quad's offset
+// is wave-uniform, channels past Co get one that is out of range for every lane.  One vector addition per store and no
+// predicate: nine vector instructions (offset, bias, activation) per 16-byte store.
+// The uniform offset is added to the lane offset and NOT passed as the store's scalar offset: a 16-byte buffer store must
+// be followed by a wait state before a vector instruction overwrites its data registers, the compiler inserts that wait
+// state only for stores without a scalar-offset register, and this hardware needs it with one as well (seen here: the
+// second data register of the one store whose next instruction rewrote it reached memory with the new value in four
+// lanes of every sixteen, in some waves).
+template <int COT, int PXT, bool ACC, bool RELU>
+__device__ __forceinline__ void conv_epilogue_buf_impl(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
+                                                       int HoWo, const unsigned (&ovoff)[PXT], const float *lds_bias)
+{
+    const float nscale = act_scale(a.act, a.slope);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        a.out, 0, (int)((size_t)a.batch * a.Co * HoWo * sizeof(float)), BUF_RSRC_FLAGS);
+#pragma unroll
+    for (int c = 0; c < COT; ++c)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int co8 = (cg * COT + c) * 32 + 8 * q;                        // wave-uniform; Co is a multiple of 16
+            const unsigned soff = co8 < a.Co ? (unsigned)(((co8 / CB) * HoWo * CB + (co8 % CB)) * (int)sizeof(float))
+                                             : BUF_SCALAR_OUT_OF_RANGE;
+            const float4 bb = *reinterpret_cast<const float4 *>(lds_bias + c * 32 + 8 * q + 4 * half);
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                float4 v = make_float4(acc[c][t][4 * q + 0], acc[c][t][4 * q + 1], acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
+                if (ACC)
+                {
+                    const float4 old = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, ovoff[t], soff, 0));
+                    v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+                }
+                v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+                v.x = act_k<RELU>(v.x, nscale); v.y = act_k<RELU>(v.y, nscale);
+                v.z = act_k<RELU>(v.z, nscale); v.w = act_k<RELU>(v.w, nscale);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, ovoff[t] + soff, 0, 0);
+            }
+        }
+}
+
+template <int COT, int PXT>
+__device__ __forceinline__ void conv_epilogue_buf(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half, int HoWo,
+                                                  const unsigned (&ovoff)[PXT], const float *lds_bias)
+{
+    if (a.accumulate) conv_epilogue_buf_impl<COT, PXT, true, false>(a, acc, cg, half, HoWo, ovoff, lds_bias);
+    else if (a.act == SMALL_HIP_ACT_RELU) conv_epilogue_buf_impl<COT, PXT, false, true>(a, acc, cg, half, HoWo, ovoff, lds_bias);
+    else conv_epilogue_buf_impl<COT, PXT, false, false>(a, acc, cg, half, HoWo, ovoff, lds_bias);
+}
+
 // Epilogue with MaxPool2D 2x2 stride 2 (no padding) fused: the wave's 32-pixel tiles are 8 pooling windows of
 // four pixels (pool_tile_pixel), so a window is this lane, lane ^ 1 (next column) and lanes ^ 2 (next row): bias
 // and activation, two shuffles and maxima per value, and the first lane of each window stores the pooled pixel
 // into [N][Co/16][Ho/2][Wo/2][16].
-template <int COT, int PXT>
+// BUFS: the store goes through a buffer resource (pvoff: the lane's byte offset of (pooled pixel, channel 4 * half of
+// channel block 0), or BUF_OUT_OF_RANGE for the three lanes of a window that store nothing), as in conv_epilogue_buf_impl.
+template <int COT, int PXT, bool BUFS = false>
 __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (&acc)[COT][PXT], int cg, int half,
                                                    const bool (&pool_ok)[PXT], const size_t (&pool_pix)[PXT],
-                                                   const float *lds_bias = nullptr)
+                                                   const float *lds_bias = nullptr, const unsigned *pvoff = nullptr)
 {
     const float nscale = act_scale(a.act, a.slope);
     const int HpWp = (a.Ho >> 1) * (a.Wo >> 1);
+    __amdgpu_buffer_rsrc_t rsrc;
+    if (BUFS) rsrc = __builtin_amdgcn_make_buffer_rsrc(a.out, 0, (int)((size_t)a.batch * a.Co * HpWp * sizeof(float)), BUF_RSRC_FLAGS);
 #pragma unroll
     for (int c = 0; c < COT; ++c)
 #pragma unroll
@@ -220,7 +291,16 @@ __device__ __forceinline__ void conv_epilogue_pool(const ConvArgs &a, floatx16 (
                     const float w = __shfl_xor(v, 2, WAVE);
                     m[e] = v > w ? v : w;
                 }
-                if (pool_ok[t] && co4 < a.Co)
+                if (BUFS)
+                {
+                    const int co8 = co4 - 4 * half;                              // wave-uniform
+                    const unsigned soff = co8 < a.Co ? (unsigned)(((co8 / CB) * HpWp * CB + (co8 % CB)) * (int)sizeof(float))
+                                                     : BUF_SCALAR_OUT_OF_RANGE;
+                    // (lane offset + uniform offset as the vector offset: see conv_epilogue_buf_impl)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, make_float4(m[0], m[1], m[2], m[3])), rsrc,
+                                                           pvoff[t] + soff, 0, 0);
+                }
+                else if (pool_ok[t] && co4 < a.Co)
                     *reinterpret_cast<float4 *>(a.out + pool_pix[t] + (size_t)(co4 / CB) * HpWp * CB + (co4 % CB)) =
                         make_float4(m[0], m[1], m[2], m[3]);
             }
@@ -240,9 +320,9 @@ __device__ __forceinline__ void pool_tile_pixel(const ConvArgs &a, const int til
     const int p = tile * 32 + col;
     pvalid = p < a.P;
     const int w = pvalid ? p >> 2 : 0;
-    n = w / HpWp;
+    n = fast_div(w, a.fd_plane);
     const int r = w - n * HpWp;
-    const int ph = r / Wp, pw = r - ph * Wp;
+    const int ph = fast_div(r, a.fd_row), pw = r - ph * Wp;
     oh = 2 * ph + ((col >> 1) & 1);
     ow = 2 * pw + (col & 1);
     pool_ok = pvalid && (col & 3) == 0;
@@ -274,9 +354,6 @@ constexpr int A_TILE_FLOATS = 272;   // 256 + 16 pad: consecutive channel blocks
 // window position does (once in Ci/16 steps): a K-step issues no vector-ALU instruction for its addresses.  The
 // launcher allows it for tensors of at most 1 GiB (lane offset + scalar offset + 16 stays below 2^31 on either side of
 // the range check, whether or not the hardware adds the scalar offset before it checks).
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-constexpr unsigned BUF_OUT_OF_RANGE = 0x80000000u;
-constexpr long long BUF_MAX_BYTES = 1ll << 30;
 
 template <int COT, int PXT, bool POOL = false, bool PW = false, bool BLDS = false, bool BUF = false>
 __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[2][COT * 2 * A_TILE_FLOATS],
@@ -305,6 +382,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
 
     const float *in_img[PXT];
     unsigned lane_base[PXT];     // BUF: byte offset of (image, channel half) in the input tensor
+    unsigned ovoff[PXT];         // BUF: byte offset of (output pixel, channel 4 * half) in the output tensor, or out of range
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
@@ -320,9 +398,9 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
             const int p = ((pxb * 4 + wave) * PXT + t) * 32 + col;
             pvalid[t] = p < a.P;
             const int pc = pvalid[t] ? p : 0;
-            n = pc / HoWo;
+            n = fast_div(pc, a.fd_plane);
             rem = pc - n * HoWo;
-            oh = rem / a.Wo;
+            oh = fast_div(rem, a.fd_row);
             ow = rem - oh * a.Wo;
             pool_ok[t] = false;
             out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
@@ -331,6 +409,7 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
         lane_base[t] = (unsigned)(((size_t)n * CiB * in_blk + half * 8) * sizeof(float));
+        ovoff[t] = (POOL ? pool_ok[t] : pvalid[t]) ? (unsigned)((out_pix[t] + 4 * half) * sizeof(float)) : BUF_OUT_OF_RANGE;
         // PW: the pixel's own position (a pixel past the end reads pixel 0 of image 0 and stores nothing)
         if (PW) in_img[t] += (size_t)(oh * a.W + ow) * CB;
     }
@@ -541,6 +620,12 @@ __device__ __forceinline__ void conv_lds_tile(const ConvArgs &a, float (&lds_a)[
                     r4[((c * PXT + t) * 4 + q) * WAVE] = make_float4(acc[c][t][4 * q], acc[c][t][4 * q + 1], acc[c][t][4 * q + 2], acc[c][t][4 * q + 3]);
         return;
     }
+    if (BUF && BLDS)
+    {
+        if (POOL) conv_epilogue_pool<COT, PXT, true>(a, acc, cg, half, pool_ok, out_pix, s_bias, ovoff);
+        else conv_epilogue_buf<COT, PXT>(a, acc, cg, half, HoWo, ovoff, s_bias);
+        return;
+    }
     if (POOL) conv_epilogue_pool<COT, PXT>(a, acc, cg, half, pool_ok, out_pix, BLDS ? s_bias : nullptr);
     else conv_epilogue<COT, PXT>(a, acc, cg, half, HoWo, pvalid, out_pix, BLDS ? s_bias : nullptr);
 }
@@ -583,7 +668,6 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
-    unsigned lane_base[PXT];     // BUF: byte offset of (image, channel half) in the input tensor
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
@@ -599,9 +683,9 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
             const int p = (pxb * PXT + t) * 32 + col;
             pvalid[t] = p < a.P;
             const int pc = pvalid[t] ? p : 0;
-            n = pc / HoWo;
+            n = fast_div(pc, a.fd_plane);
             rem = pc - n * HoWo;
-            oh = rem / a.Wo;
+            oh = fast_div(rem, a.fd_row);
             ow = rem - oh * a.Wo;
             pool_ok[t] = false;
             out_pix[t] = ((size_t)n * CoB * HoWo + rem) * CB;
@@ -609,7 +693,6 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
-        lane_base[t] = (unsigned)(((size_t)n * CiB * in_blk + half * 8) * sizeof(float));
     }
     const float *w_row[COT];
 #pragma unroll
@@ -1652,6 +1735,7 @@ __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArg
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
+    set_pixel_divisors(a, false);
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
     a.n_px_blocks = (a.P + 32 * PXT - 1) / (32 * PXT);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
@@ -1683,12 +1767,14 @@ bool buffer_form(const ConvArgs &a)
     static const bool off = tune_int("conv_buf", 1) == 0;
     const long long in_bytes = (long long)a.batch * a.Ci * a.H * a.W * (long long)sizeof(float);
     const long long f_bytes = (long long)((a.Co + CB - 1) / CB * CB) * a.Ci * a.kh * a.kw * (long long)sizeof(float);
-    return !off && a.slabs == 0 && in_bytes <= BUF_MAX_BYTES && f_bytes <= BUF_MAX_BYTES;
+    const long long out_bytes = (long long)a.batch * a.Co * a.Ho * a.Wo * (long long)sizeof(float);   // the pooled tensor is smaller
+    return !off && a.slabs == 0 && in_bytes <= BUF_MAX_BYTES && f_bytes <= BUF_MAX_BYTES && out_bytes <= BUF_MAX_BYTES;
 }
 
 template <int COT, int PXT>
 void launch_mfma(ConvArgs &a, hipStream_t s)
 {
+    set_pixel_divisors(a, false);
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
@@ -1758,6 +1844,7 @@ template <int COT, int PXT>
 int launch_streamk(const char *op, ConvArgs &a, hipStream_t s, bool *done)
 {
     *done = false;
+    set_pixel_divisors(a, false);
     const size_t bytes = streamk_plan<COT, PXT>(a);
     if (bytes == 0) return SMALL_HIP_OK;
     WorkspaceLease lease;            // held until both launches are enqueued
@@ -1917,6 +2004,7 @@ int conv_f32(const char *op, int batch, int kh, int kw, int stride, int pt, int 
 template <int COT, int PXT>
 void launch_mfma_pool(ConvArgs &a, hipStream_t s)
 {
+    set_pixel_divisors(a, true);
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
