@@ -651,12 +651,14 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
 // the fixed order 0+1+2+3 (deterministic) and runs the epilogue.  Operands go straight from global
 // memory to the MFMA registers (nothing is shared between the waves until the reduction).
 // POOL: the 32-pixel tiles are the pooling form's groups of 8 windows and the epilogue pools (pool_tile_pixel)
-template <int COT, int PXT, bool POOL = false>
+// BUF: operands through buffer loads, as in conv_lds_tile (each wave has its own K range, so its window position and
+// scalar offsets are the wave's)
+template <int COT, int PXT, bool POOL = false, bool BUF = false>
 __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)[3][COT * PXT][16][64],
                                                  const int cg, const int pxb)
 {
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 31;
     const int half = lane >> 5;
 
@@ -668,6 +670,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     const float *zero_half = g_zero_block + half * 8;
 
     const float *in_img[PXT];
+    unsigned lane_base[PXT];     // BUF: byte offset of (image, channel half) in the input tensor
     int ih0[PXT], iw0[PXT];
     bool pvalid[PXT];
     size_t out_pix[PXT];
@@ -693,14 +696,17 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
         ih0[t] = oh * a.stride_h - a.pt;
         iw0[t] = ow * a.stride - a.pl;
         in_img[t] = a.in + (size_t)n * CiB * in_blk + half * 8;
+        lane_base[t] = (unsigned)(((size_t)n * CiB * in_blk + half * 8) * sizeof(float));
     }
     const float *w_row[COT];
+    unsigned w_voff[COT];        // BUF: byte offset of this lane's filter row in the filter tensor
 #pragma unroll
     for (int c = 0; c < COT; ++c)
     {
         const int co = (cg * COT + c) * 32 + col;
         const int cc = co < a.Co ? co : a.Co - 1;
         w_row[c] = a.filt + (size_t)(cc / CB) * CiB * taps * (CB * CB) + (cc % CB) + half * 8 * CB;
+        w_voff[c] = (unsigned)(((size_t)(cc / CB) * CiB * taps * (CB * CB) + (cc % CB) + half * 8 * CB) * sizeof(float));
     }
 
     floatx16 acc[COT][PXT];
@@ -722,7 +728,55 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     int ta = tap0 / a.kw, tb = tap0 - (tap0 / a.kw) * a.kw;
     int left = mine;                 // steps still to be loaded
 
+    // BUF: the window position's lane offsets (out of range for a masked tap, and for every lane once the wave's steps
+    // have all been requested)
+    const int in_blk32 = a.H * a.W * CB;
+    unsigned voff[PXT];
+    auto tap_offsets = [&]() {
+#pragma unroll
+        for (int t = 0; t < PXT; ++t)
+        {
+            const int ih = ih0[t] + ta, iw = iw0[t] + tb;
+            const bool ok = left > 0 && pvalid[t] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+            voff[t] = ok ? lane_base[t] + (unsigned)((ih * a.W + iw) * (CB * (int)sizeof(float))) : BUF_OUT_OF_RANGE;
+        }
+    };
+    __amdgpu_buffer_rsrc_t rsrc_in, rsrc_f;
+    if (BUF)
+    {
+        rsrc_in = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.in), 0,
+                                                    (int)((size_t)a.batch * a.Ci * a.H * a.W * sizeof(float)), BUF_RSRC_FLAGS);
+        rsrc_f = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.filt), 0,
+                                                   (int)((size_t)CoB * CiB * taps * (CB * CB) * sizeof(float)), BUF_RSRC_FLAGS);
+        tap_offsets();
+    }
     auto load_step = [&](float (&A)[COT][8], float4 (&B)[PXT][2]) {
+        if (BUF)
+        {
+            const int soff_b = cib * (in_blk32 * (int)sizeof(float));
+#pragma unroll
+            for (int t = 0; t < PXT; ++t)
+            {
+                B[t][0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_in, voff[t], soff_b, 0));
+                B[t][1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_in, voff[t] + 16, soff_b, 0));
+            }
+            const int soff_a = (cib * taps + ta * a.kw + tb) * (CB * CB * (int)sizeof(float));
+#pragma unroll
+            for (int c = 0; c < COT; ++c)
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk)
+                    A[c][kk] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                             rsrc_f, w_voff[c] + kk * (CB * (int)sizeof(float)), soff_a, 0));
+            --left;
+            if (left <= 0) tap_offsets();          // nothing more to request: every lane out of range
+            else if (++cib == CiB)                 // the next window position (wave-uniform, once in Ci/16 steps)
+            {
+                cib = 0;
+                if (++tb == a.kw) { tb = 0; ++ta; }
+                tap_offsets();
+            }
+            return;
+        }
         const bool live = left > 0;
         const int tap = ta * a.kw + tb;
 #pragma unroll
@@ -804,7 +858,7 @@ __device__ __forceinline__ void conv_splitk_tile(const ConvArgs &a, float (&red)
     }
 }
 
-template <int COT, int PXT>
+template <int COT, int PXT, bool BUF = false>
 __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArgs a0)
 {
     const ConvArgs a = slab_args(a0);
@@ -812,7 +866,7 @@ __global__ __launch_bounds__(256) void conv_mfma_f32_splitk_kernel(const ConvArg
     const int bid = blockIdx.x;
     const int lid = (bid % NUM_XCD) * a.per_xcd + bid / NUM_XCD;
     if (lid >= a.n_blocks) return;
-    conv_splitk_tile<COT, PXT>(a, red, lid % a.n_co_groups, lid / a.n_co_groups);
+    conv_splitk_tile<COT, PXT, false, BUF>(a, red, lid % a.n_co_groups, lid / a.n_co_groups);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -845,7 +899,7 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
     const int co32 = (lid % a.n_co_groups) * COT + sub % COT;
     const int px32 = (lid / a.n_co_groups) * (4 * PXT) + sub / COT;
     if (co32 * 32 >= a.Co || px32 * 32 >= a.P) return;     // uniform over the workgroup
-    conv_splitk_tile<1, 1, POOL>(a, red, co32, px32);
+    conv_splitk_tile<1, 1, POOL, BUF>(a, red, co32, px32);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1732,6 +1786,17 @@ __global__ __launch_bounds__(256, 2) void conv_pw_dw3x3_f32_kernel(const ConvArg
     }
 }
 
+// Operand streams through buffer loads (conv_lds_tile's BUF form)?  An ordinary convolution (no slabs) whose input and
+// filter are at most BUF_MAX_BYTES each; SMALL_HIP_TUNE key conv_buf=0 keeps the flat-address form.
+bool buffer_form(const ConvArgs &a)
+{
+    static const bool off = tune_int("conv_buf", 1) == 0;
+    const long long in_bytes = (long long)a.batch * a.Ci * a.H * a.W * (long long)sizeof(float);
+    const long long f_bytes = (long long)((a.Co + CB - 1) / CB * CB) * a.Ci * a.kh * a.kw * (long long)sizeof(float);
+    const long long out_bytes = (long long)a.batch * a.Co * a.Ho * a.Wo * (long long)sizeof(float);   // the pooled tensor is smaller
+    return !off && a.slabs == 0 && in_bytes <= BUF_MAX_BYTES && f_bytes <= BUF_MAX_BYTES && out_bytes <= BUF_MAX_BYTES;
+}
+
 template <int COT, int PXT>
 void launch_splitk(ConvArgs &a, hipStream_t s)
 {
@@ -1740,7 +1805,9 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
     a.n_px_blocks = (a.P + 32 * PXT - 1) / (32 * PXT);
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
-    hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), dim3(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1), dim3(256), 0, s, a);
+    const dim3 grid(a.per_xcd * NUM_XCD, a.slabs > 0 ? a.slabs : 1);
+    if (buffer_form(a)) hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_mfma_f32_splitk_kernel<COT, PXT>), grid, dim3(256), 0, s, a);
 }
 
 // Whole rounds + cut tail (conv_mfma_f32_hybrid_kernel) or whole tiles only?  A split-K piece multiplies about half as
@@ -1758,17 +1825,6 @@ bool tail_pays(int n_main, int rest, int nsteps)
     (void)n_main;
     if (knob == 0 || rest == 0 || nsteps < 8) return false;
     return knob == 2 || rest <= NUM_CU / 2;
-}
-
-// Operand streams through buffer loads (conv_lds_tile's BUF form)?  An ordinary convolution (no slabs) whose input and
-// filter are at most BUF_MAX_BYTES each; SMALL_HIP_TUNE key conv_buf=0 keeps the flat-address form.
-bool buffer_form(const ConvArgs &a)
-{
-    static const bool off = tune_int("conv_buf", 1) == 0;
-    const long long in_bytes = (long long)a.batch * a.Ci * a.H * a.W * (long long)sizeof(float);
-    const long long f_bytes = (long long)((a.Co + CB - 1) / CB * CB) * a.Ci * a.kh * a.kw * (long long)sizeof(float);
-    const long long out_bytes = (long long)a.batch * a.Co * a.Ho * a.Wo * (long long)sizeof(float);   // the pooled tensor is smaller
-    return !off && a.slabs == 0 && in_bytes <= BUF_MAX_BYTES && f_bytes <= BUF_MAX_BYTES && out_bytes <= BUF_MAX_BYTES;
 }
 
 template <int COT, int PXT>
