@@ -906,12 +906,11 @@ __global__ __launch_bounds__(256, (COT * PXT == 2 ? 5 : COT * PXT == 1 ? 6 : 2))
 // Equal shares of the reduction for launches with few tiles and a long reduction (3x3 convolutions with 512 / 1024
 // channels on a 13x13 map: 352 workgroup tiles for 256 compute units, 288 or 576 K-steps each).  Whole tiles leave a
 // second round in which a third of the machine works; cutting only the left-over tiles four ways (the hybrid kernel) leaves
-// the first round with one wave per SIMD.  Here all K-steps of the launch, tile after tile, are cut into 2 x 256 equal runs;
-// a workgroup multiplies its run (the end of one tile and the start of the next, as a rule) with the LDS-staged body, two
+// the first round with one wave per SIMD.  Here all K-steps of the launch, tile after tile, are cut into 3 x 256 equal runs;
+// a workgroup multiplies its run (the end of one tile and the start of the next, as a rule) with the LDS-staged body, three
 // workgroups per compute unit, all finishing together.  A run that is not a whole tile leaves its raw accumulators in a
-// scratch block; conv_streamk_fixup_kernel adds the two or three runs of a tile in run order (deterministic) and applies
+// scratch block; conv_streamk_fixup_kernel adds the runs of a tile in run order (deterministic) and applies
 // accumulate / bias / activation.
-constexpr int SK_CHUNKS = 2 * NUM_CU;
 template <int COT, int PXT>
 constexpr int sk_part_floats() { return 4 * COT * PXT * 16 * WAVE; }
 
@@ -1812,7 +1811,7 @@ void launch_splitk(ConvArgs &a, hipStream_t s)
 
 // Whole rounds + cut tail (conv_mfma_f32_hybrid_kernel) or whole tiles only?  A split-K piece multiplies about half as
 // fast as a whole tile (operands straight from global memory, one MFMA chain per wave), so the cut tail wins while the
-// left-over tiles fill at most half a round and loses beyond, whatever the wave tile and the number of whole rounds.
+// left-over tiles fill at most two thirds of a round and loses beyond, whatever the wave tile and the number of whole rounds.
 // Batch sweeps, left-over tiles of 256 -> gain (+) or loss (-) in us: 1x1 256->256 @28x28 (16 K-steps) 32: +3, 128: +1,
 // 224: -3; 512->512 @14x14 (32) 80: +2..6, 176: -2, 224: -6; 3x3 64->128 @52x52 (36) 84: +1, 168: -3, 252: -7;
 // 3x3 128->256 @26x26 (72) 20: +25, 84: +10, 128: +4, 168: -3, 216: -10; 3x3 256->512 @13x13 (144) 40: +42, 128: +13,
@@ -1824,7 +1823,9 @@ bool tail_pays(int n_main, int rest, int nsteps)
     static const int knob = tune_int("conv_tail", 1);
     (void)n_main;
     if (knob == 0 || rest == 0 || nsteps < 8) return false;
-    return knob == 2 || rest <= NUM_CU / 2;
+    // with the split-K pieces on buffer loads the break-even moved up: left-over tiles 160..168 now gain 3..8 us (3x3
+    // 128->256 @26x26, 64->128 @52x52 with pooling), 212..252 still lose 1..4 us
+    return knob == 2 || rest <= 11 * NUM_CU / 16;
 }
 
 template <int COT, int PXT>
@@ -1873,12 +1874,12 @@ struct GroupSlabs
 // the shape does not qualify.  Few tiles that do not fill whole rounds and a long reduction (measured, batch 16 on 13x13
 // maps: 512 -> 1024 3x3 287 -> 264 us, 1024 -> 1024 519 -> 467 us, 256 -> 512 (144 steps) 81 -> 69 us; with 72 steps or
 // fewer the fix-up pass costs more than the balance gains).  SMALL_HIP_TUNE keys conv_streamk=<workgroups per compute
-// unit> (default 2, 0 = never), conv_streamk_min=<steps> (default 128)
+// unit> (default 3: 512 -> 1024 @13x13 b16 200.8 -> 198.2 us, 1024 -> 1024 420 -> 416 against 2; 0 = never), conv_streamk_min=<steps> (default 128)
 template <int COT, int PXT>
 size_t streamk_plan(ConvArgs &a)
 {
     static const int min_steps = tune_int("conv_streamk_min", 128);
-    static const int per_cu = tune_int("conv_streamk", 2);
+    static const int per_cu = tune_int("conv_streamk", 3);
     if (per_cu <= 0 || a.slabs != 0 || a.Co % (32 * COT) != 0) return 0;
     a.n_co_groups = (a.Co + 32 * COT - 1) / (32 * COT);
     a.n_px_blocks = (a.P + 32 * PXT * 4 - 1) / (32 * PXT * 4);
