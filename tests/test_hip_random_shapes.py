@@ -149,3 +149,20 @@ def test_depthwise_and_pools_f32_random(lib, oracle, case):
     assert lib.small_hip_avgpool2d_f32(*args, hu.ptr(dx), hu.ptr(da), hu.stream()) == 0
     _, wa = oracle.avgpool2d_f32(batch, CB, kh, kw, s, pt, pb, pl, pr, Cn, H, W, x)
     assert_close_f32(hu.host(da), wa, what="avgpool %s" % (case,))
+
+
+def test_conv2d_f32_flat_address_form():
+    """The float32 convolution's flat-address form (what tensors beyond the buffer-load form's size limit get, and what
+    SMALL_HIP_TUNE=conv_buf=0 selects) on the same seeded shapes.  The switch is read once per process, so the cases run
+    in a child process of their own."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, SMALL_HIP_TUNE="conv_buf=0")
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.join(root, "tests", "test_hip_random_shapes.py"), "-q", "-x",
+                        "-m", "gpu", "-k", "test_conv2d_f32_random", "-p", "no:cacheprovider"],
+                       cwd=root, env=env, capture_output=True, text=True, timeout=600)
+    tail = "\n".join(r.stdout.splitlines()[-15:])
+    assert r.returncode == 0, tail
+    assert " passed" in tail and "failed" not in tail, tail
