@@ -14,6 +14,9 @@
 //     through LDS once per workgroup (conv_lds_tile) or read directly (conv_splitk_tile).
 //   - D: a lane holds 4 consecutive output channels of one pixel per register quad, i.e. 16-byte
 //     stores into the packed [px][16] output, after accumulate / bias / activation in registers.
+// Addresses: tensors of at most 1 GiB (every case that occurs in practice) are read and written through buffer
+// resources, so that a K-step and a store need no address arithmetic on the vector ALU, whose instructions cost
+// the SIMD's matrix pipe their issue time (BUF template parameter); larger tensors take the flat-address forms.
 // A wave owns COT x PXT tiles of 32 x 32; the four waves of a workgroup share the output channel
 // group and take consecutive pixel tiles.  Workgroup ids are re-mapped so that all channel groups
 // of a pixel range run on one XCD and share its L2.  Kernels:
@@ -1837,7 +1840,7 @@ void launch_mfma(ConvArgs &a, hipStream_t s)
     a.n_blocks = a.n_co_groups * a.n_px_blocks;
     a.per_xcd = (a.n_blocks + NUM_XCD - 1) / NUM_XCD;
     const int n_main = a.n_blocks / NUM_CU * NUM_CU, rest = a.n_blocks - n_main;
-    // pointwise form of the main loop (SMALL_HIP_TUNE key conv_pw=0 switches it off)
+    // flat addresses: pointwise form of the main loop for 1x1 windows (SMALL_HIP_TUNE key conv_pw=0 switches it off)
     static const bool pw_off = tune_int("conv_pw", 1) == 0;
     // (only where the buffer-load form is not allowed: that one needs no special case for 1x1 windows and is faster,
     // MobileNetV1 batch 64: 512 -> 512 @14x14 55.8 -> 52.5 us, 1024 -> 1024 @7x7 64.4 -> 54.9 us)
